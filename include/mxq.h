@@ -1,0 +1,148 @@
+/*
+ * mxq.h — C ABI of the MI355X (gfx950) quantized-weight matmul path.
+ *
+ * Drop-in replacement boundary for the `src/ops` quantized matmul family of the
+ * Mach X inference engine.  Every entry point mirrors one reference free
+ * function `sycl::event ie::f(sycl::queue&, <device pointers>, <dims>, deps)`
+ * (include/ie/ops.hpp:3-7) with these mechanical changes:
+ *   - `sycl::queue&`  -> `mx_stream_t` (a hipStream_t passed as void*; NULL = the
+ *                        default stream); ordering is stream order, so there is
+ *                        no `deps` argument and no returned event;
+ *   - `sycl::half*`   -> `uint16_t*` (IEEE binary16 bit patterns);
+ *   - the return value is an `int` status (MX_OK = 0).  Where the reference
+ *     silently returns an empty event on an unsupported shape
+ *     (src/ops/gemm_q4k_xmx.cpp:120-121) this ABI returns MX_ERR_SHAPE and
+ *     launches nothing.  Argument checks run before any HIP call.
+ * All pointers are caller-owned device memory unless a comment says "host".
+ * Weight layouts are the unchanged GGUF block layouts
+ * (include/ie/quant_blocks.hpp) in "W[K,N] column-packed" order: output row n
+ * owns K/blk consecutive blocks (src/ops/gemv_q4k.cpp:3-11).
+ * Argument order is (K, N) for GEMV and (M, K, N) for GEMM, as in the reference.
+ */
+#ifndef MXQ_H
+#define MXQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mx_stream_t;
+
+enum {
+    MX_OK = 0,
+    MX_ERR_NULL = 1,        /* a required pointer is NULL */
+    MX_ERR_SHAPE = 2,       /* a dimension violates the documented precondition */
+    MX_ERR_ALIGN = 3,       /* a pointer violates the documented alignment */
+    MX_ERR_LAUNCH = 4,      /* the HIP runtime reported an error (see mx_last_hip_error) */
+    MX_ERR_UNSUPPORTED = 5  /* valid arguments, combination not built */
+};
+
+const char* mx_status_string(int status);
+int mx_last_hip_error(void);  /* hipError_t of the last MX_ERR_LAUNCH on this thread */
+int mx_version(void);
+
+/* ---------------------------------------------------------------- activation quantizers
+ * quantize_q8_1   include/ie/ops.hpp:301-304, src/ops/gemv_q8dot.cpp:94-124
+ * quantize_q8_1s  include/ie/ops.hpp:307-310, src/ops/gemv_q8dot.cpp:57-91
+ * x: n elements (n % 32 == 0; several rows are simply contiguous) -> n/32
+ * block_q8_1x (40 B) / block_q8_1s (48 B).  d = amax/127, q = round-half-away,
+ * s = d * sum(q).  `_f32` variants take fp32 activations (same math).  */
+int mx_quantize_q8_1(mx_stream_t s, const uint16_t* x_f16, void* out_q8, uint64_t n);
+int mx_quantize_q8_1_f32(mx_stream_t s, const float* x, void* out_q8, uint64_t n);
+int mx_quantize_q8_1s(mx_stream_t s, const uint16_t* x_f16, void* out_q8s, uint64_t n);
+int mx_quantize_q8_1s_f32(mx_stream_t s, const float* x, void* out_q8s, uint64_t n);
+
+/* ---------------------------------------------------------------- block dequant
+ * dequant_q8_0/q4_K/q6_K  include/ie/dequant.hpp, src/ops/dequant_kernels.cpp:55-269
+ * dequant_mxfp4           src/ops/dequant_kernels.cpp:325-359
+ * Bit-exact with ie::ref::dequant_* (include/ie/dequant_ref.hpp:32-96); fp16
+ * output is the single RNE rounding of that fp32 value.  n_elements must be a
+ * whole number of blocks.  `_f32` variants write the unrounded fp32 value.  */
+int mx_dequant_q8_0(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
+int mx_dequant_q4_K(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
+int mx_dequant_q6_K(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
+int mx_dequant_mxfp4(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
+int mx_dequant_q8_0_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
+int mx_dequant_q4_K_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
+int mx_dequant_q6_K_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
+int mx_dequant_mxfp4_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
+/* dequant_*_to_Bt  src/ops/dequant_kernels.cpp:282-320,392-431,611-632,364-390:
+ * whole matrix -> fp16 Bt[k*N + n].  */
+int mx_dequant_q8_0_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q4_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q6_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_mxfp4_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+
+/* ---------------------------------------------------------------- decode GEMV, int-dot on q8 activations
+ * y[n] = sum_k deq(W)[n,k] * (d8 * q8)[k], fp32 accumulate, fp16 out.
+ * x_q8: block_q8_1x stream from mx_quantize_q8_1 (8-byte aligned).
+ * K % 256 == 0 for K-quants, K % 32 == 0 for Q8_0 / MXFP4.  W 16-byte aligned
+ * (Q4_K, SoA planes) or 2-byte aligned (Q6_K, AoS Q8_0).
+ *
+ * gemv_q4_K_q8          include/ie/ops.hpp:312-316, src/ops/gemv_q8dot.cpp:261-357
+ * gemv_q6_K_q8(_ktiled) include/ie/ops.hpp:375-391, src/ops/gemv_q6k.cpp:335-589
+ * gemv_q8_0_soa_q8(_g)  include/ie/ops.hpp:351-364, src/ops/gemv_q8dot.cpp:609-707
+ * gemv_mxfp4_soa_q8     include/ie/ops.hpp:498-502, src/ops/gemv_mxfp4.cpp:80-154
+ * mx_gemv_q8_0_q8 takes the AoS GGUF block_q8_0 array (no reference counterpart:
+ * the reference only has the SoA kernel).  */
+int mx_gemv_q4_K_q8(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_K_q8(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q8_0_q8(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q8_0_soa_q8(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y,
+                        uint32_t K, uint32_t N);
+int mx_gemv_mxfp4_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* qs_plane, const uint8_t* e_plane,
+                         uint16_t* y, uint32_t K, uint32_t N);
+/* gemv_mxfp4_soa_q8_x2  include/ie/ops.hpp:507-513, src/ops/gemv_mxfp4.cpp:165-250:
+ * gate and up share x; per-row fp32 bias (may be NULL) added after the reduce.  */
+int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x_q8, const uint8_t* gate_qs, const uint8_t* gate_e,
+                            const uint8_t* up_qs, const uint8_t* up_e, const float* gate_bias,
+                            const float* up_bias, uint16_t* gate_y, uint16_t* up_y, uint32_t K, uint32_t N);
+
+/* Batched-T variants: weights read once, dotted against T activation rows.
+ * x_q8 = T contiguous block_q8_1x rows (row t at block t*(K/32)); y[t*N + n].
+ * 1 <= T <= 16 (T > 8 runs as two passes).
+ * gemv_q4_K_q8_batched   include/ie/ops.hpp:332-336, src/ops/gemv_q8dot.cpp:375-470
+ * gemv_q6_soa_q8_batched include/ie/ops.hpp:420-426 (the reference batches Q6_K only
+ *                        in its SoA form; here the GGUF AoS blocks are batched directly)
+ * Q8_0 / MXFP4 batched have no reference counterpart (T >= 2 falls to dequant +
+ * GEMM there, src/model/qwen35_dense.cpp:811-831).  */
+int mx_gemv_q4_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W,
+                                uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_mxfp4_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* qs_plane, const uint8_t* e_plane,
+                                 uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* fp32-output twins of the T = 1 int-dot kernels (no reference counterpart; for
+ * callers that keep fp32 activations end to end).  */
+int mx_gemv_q4_K_q8_f32(mx_stream_t s, const void* x_q8, const void* W, float* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_K_q8_f32(mx_stream_t s, const void* x_q8, const void* W, float* y, uint32_t K, uint32_t N);
+int mx_gemv_q8_0_q8_f32(mx_stream_t s, const void* x_q8, const void* W, float* y, uint32_t K, uint32_t N);
+
+/* ---------------------------------------------------------------- decode GEMV, float activations
+ * gemv_q4_K           include/ie/ops.hpp:468-472, src/ops/gemv_q4k.cpp:55-149
+ * gemv_q6_K           include/ie/ops.hpp (gemv_q6_K), src/ops/gemv_q6k.cpp:591-633
+ * gemv_mxfp4_soa_f16  include/ie/ops.hpp:493-497, src/ops/gemv_mxfp4.cpp:257-305
+ * A fp16 [K], y fp16 [N]; `_f32`: fp32 A, fp32 y (the shape of BASELINE config 1).  */
+int mx_gemv_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_mxfp4_soa_f16(mx_stream_t s, const uint16_t* A, const uint8_t* qs_plane, const uint8_t* e_plane,
+                          uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q4_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
+int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
+
+/* ---------------------------------------------------------------- host repackers (host pointers)
+ * MXFP4 AoS -> SoA planes  src/model/gptoss.cpp:180-208
+ * Q8_0  AoS -> SoA planes  src/model/qwen35moe_split.cpp:134-144  */
+int mx_repack_mxfp4_to_soa(const void* blocks, uint64_t n_blocks, uint8_t* qs_plane, uint8_t* e_plane);
+int mx_repack_q8_0_to_soa(const void* blocks, uint64_t n_blocks, int8_t* qs_plane, uint16_t* d_plane);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXQ_H */

@@ -1,0 +1,12 @@
+"""MI355X-native quantized-weight matmul path (GGUF Q4_K / Q6_K / Q8_0 / MXFP4).
+
+`ops` mirrors the reference's `src/ops` free functions on torch device tensors;
+every call goes through the C ABI of libmxq.so (include/mxq.h).  PyTorch is
+used only for device memory and the current HIP stream.
+"""
+from . import _lib
+
+lib = _lib.load()
+
+from . import ops  # noqa: E402
+from .ops import MxError  # noqa: E402,F401

@@ -1,0 +1,63 @@
+"""Build recipe for libmxq.so (hipcc, gfx950 only).
+
+    python -m machx_inference_engine_amd.build [--force]
+
+Each translation unit under csrc/ is compiled to an object in csrc/build/ and the
+objects are linked into machx_inference_engine_amd/libmxq.so.  The library is
+built in-tree so that it travels with the source tree.
+"""
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
+LIB = os.path.join(_HERE, "libmxq.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+         # no compiler-generated packed fp32 ops (v_pk_{add,mul,fma}_f32)
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _sources():
+    return sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".cpp")))
+
+
+def _headers_mtime():
+    hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    hs.append(os.path.join(_HERE, "..", "include", "mxq.h"))
+    return max(os.path.getmtime(h) for h in hs)
+
+
+def _compile(src, force):
+    obj = os.path.join(OBJ, src.rsplit(".", 1)[0] + ".o")
+    path = os.path.join(CSRC, src)
+    if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(path), _headers_mtime()):
+        return obj, None
+    cmd = [HIPCC] + FLAGS + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", path, "-o", obj]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, p.stderr[-6000:]))
+    return obj, p.stderr
+
+
+def build(force=False, jobs=8, verbose=False):
+    os.makedirs(OBJ, exist_ok=True)
+    with cf.ThreadPoolExecutor(jobs) as ex:
+        res = list(ex.map(lambda s: _compile(s, force), _sources()))
+    objs = [o for o, _ in res]
+    if verbose:
+        for _, err in res:
+            if err:
+                sys.stderr.write(err)
+    if force or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs):
+        p = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, capture_output=True, text=True)
+        if p.returncode != 0:
+            raise RuntimeError("link failed:\n" + p.stderr[-4000:])
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv, verbose=True))

@@ -1,0 +1,382 @@
+// gemv.hip — dense decode GEMV entry points (T = 1 and batched T <= 16) for
+// Q4_K / Q6_K / Q8_0 / MXFP4 weights: int-dot on q8 activations and the
+// float-activation variants.  Kernel structure: mxq_gemv_core.h.
+#include "mxq_gemv_core.h"
+#include "mxq_host.h"
+
+namespace mxq {
+
+// One launch can carry two independent (weights, output, bias) segments that
+// share the activation (the fused gate/up form); blockIdx.y picks the segment.
+template <class F, class OutT>
+struct GemvSeg {
+    typename F::W w;
+    OutT* y;
+    const float* bias;
+};
+
+template <class F, int T, int R, int G, class OutT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> seg0, GemvSeg<F, OutT> seg1, const uint8_t* xq8,
+                                                                uint32_t K, uint32_t N, uint32_t KT, uint32_t T_real) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
+    const GemvSeg<F, OutT>& seg = blockIdx.y ? seg1 : seg0;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    const size_t q8_row_bytes = (size_t)(K / 32) * kQ81xBytes;
+    auto xrow = [&](uint32_t t) { return xq8 + (size_t)(t < T_real ? t : T_real - 1) * q8_row_bytes; };
+    const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    const uint32_t n_tiles = (K + KT - 1) / KT;
+    ActTile<F::HAS_MIN> act;
+    bool staged = false;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
+        const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
+        uint32_t rows[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) rows[r] = (row0 + r < N) ? row0 + r : N - 1;
+        float acc[R][T];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < T; ++t) acc[r][t] = 0.f;
+        for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+            const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
+            if (n_tiles > 1 || !staged) {
+                __syncthreads();
+                act = stage_act<F::HAS_MIN, T>(lds, xrow, k0, kt, KT);
+                __syncthreads();
+                staged = true;
+            }
+            gemv_tile<F, T, R, G>(seg.w, rows, k0 / 32, kt / 32, gl, act, acc);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                float v = group_sum<G>(acc[r][t]);
+                if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N && (uint32_t)t < T_real) {
+                    if (seg.bias) v += seg.bias[row0 + r];
+                    store_out(seg.y + (size_t)t * N + row0 + r, v);
+                }
+            }
+    }
+}
+
+// ---------------------------------------------------------------- float activations (T = 1)
+// Same unit walk; activations staged as fp32 plus per-16 sums; the fold is the
+// reference's acc += (d*sc) * sum(a*q) - (dmin*m) * sum(a)  (src/ops/gemv_q4k.cpp:119-146).
+template <bool UNSIGNED>
+__device__ __forceinline__ float code_to_f(uint32_t w, int j) {
+    if (UNSIGNED) return (float)((w >> (8 * j)) & 0xFFu);
+    return (float)(int)(int8_t)(w >> (8 * j));
+}
+
+template <class F, bool UNSIGNED, int R, int G, class ActT, class OutT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w, const ActT* A, OutT* y, uint32_t K, uint32_t N, uint32_t KT) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    float* xa = reinterpret_cast<float*>(lds);          // [KT]
+    float* s16 = xa + KT;                                // [KT/16]
+    constexpr int GROUPS = 64 / G;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    const uint32_t n_tiles = (K + KT - 1) / KT;
+    bool staged = false;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
+        const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
+        uint32_t rows[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) rows[r] = (row0 + r < N) ? row0 + r : N - 1;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = 0.f;
+        for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+            const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
+            if (n_tiles > 1 || !staged) {
+                __syncthreads();
+                for (uint32_t i = threadIdx.x; i < kt / 16; i += blockDim.x) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const float v = load_act(A + k0 + i * 16 + j);
+                        xa[i * 16 + j] = v;
+                        s += v;
+                    }
+                    s16[i] = s;
+                }
+                __syncthreads();
+                staged = true;
+            }
+            const uint32_t u0 = k0 / 32, n_units = kt / 32;
+            for (uint32_t ul = gl; ul < n_units; ul += G) {
+                typename F::Raw raw[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) raw[r] = F::load(w, rows[r], u0 + ul);
+                const uint32_t ea = F::elem_off(ul), eb = ea + F::EB_OFF;
+                float fa[16], fb[16];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 va = *reinterpret_cast<const float4*>(xa + ea + 4 * i);
+                    const float4 vb = *reinterpret_cast<const float4*>(xa + eb + 4 * i);
+                    fa[4 * i] = va.x; fa[4 * i + 1] = va.y; fa[4 * i + 2] = va.z; fa[4 * i + 3] = va.w;
+                    fb[4 * i] = vb.x; fb[4 * i + 1] = vb.y; fb[4 * i + 2] = vb.z; fb[4 * i + 3] = vb.w;
+                }
+                const float sa = s16[ea >> 4], sb = s16[eb >> 4];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    Unit un;
+                    F::decode(raw[r], u0 + ul, un);
+                    float da = 0.f, db = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            da += fa[4 * i + j] * code_to_f<UNSIGNED>(un.a[i], j);
+                            db += fb[4 * i + j] * code_to_f<UNSIGNED>(un.b[i], j);
+                        }
+                    float v = un.ca * da + un.cb * db;
+                    if (F::HAS_MIN) v -= un.ma * sa + un.mb * sb;
+                    acc[r] += v;
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float v = group_sum<G>(acc[r]);
+            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N) store_out(y + row0 + r, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- host dispatch
+static int cu_count() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    }
+    return n;
+}
+
+constexpr uint32_t kLdsBudget = 48 * 1024;
+constexpr int kRows = 2;
+
+static uint32_t pick_group(uint32_t units) {
+    const uint32_t w64 = (units + 63) / 64 * 64, w32 = (units + 31) / 32 * 32;
+    return w32 < w64 ? 32 : 64;
+}
+
+template <class F, int T, int G, class OutT>
+static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8,
+                        uint32_t K, uint32_t N, uint32_t T_real) {
+    constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
+    const uint32_t per_elem_x8 = F::HAS_MIN ? 11 : 9;  // bytes per activation element * 8
+    uint32_t KT = (kLdsBudget * 8 / (per_elem_x8 * T)) / 256 * 256;
+    if (KT > K) KT = (K + 255) / 256 * 256;
+    if (KT == 0) return MX_ERR_SHAPE;
+    const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
+    const uint32_t cap = (uint32_t)cu_count() * 8;
+    dim3 grid(n_rg < cap ? n_rg : cap, nseg);
+    const uint32_t lds = act_tile_bytes(T, KT, F::HAS_MIN);
+    hipLaunchKernelGGL((gemv_q8_kernel<F, T, kRows, G, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real);
+    return launch_status();
+}
+
+template <class F, int G, class OutT>
+static int launch_q8_g(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8, uint32_t K,
+                       uint32_t N, uint32_t T) {
+    switch (T) {
+        case 1: return launch_q8_tg<F, 1, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 2: return launch_q8_tg<F, 2, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 3: return launch_q8_tg<F, 3, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 4: return launch_q8_tg<F, 4, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 5:
+        case 6: return launch_q8_tg<F, 6, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 7:
+        case 8: return launch_q8_tg<F, 8, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+    }
+    return MX_ERR_SHAPE;
+}
+
+// T up to 16: passes of at most 8 tokens.
+template <class F, class OutT>
+static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, int nseg, const void* xq8, uint32_t K, uint32_t N, uint32_t T) {
+    const uint8_t* x = static_cast<const uint8_t*>(xq8);
+    const uint32_t G = pick_group(K / 32);
+    for (uint32_t t0 = 0; t0 < T; t0 += 8) {
+        const uint32_t tn = (T - t0 < 8) ? T - t0 : 8;
+        GemvSeg<F, OutT> a = s0, b = s1;
+        a.y = s0.y + (size_t)t0 * N;
+        if (nseg > 1) b.y = s1.y + (size_t)t0 * N;
+        const uint8_t* xt = x + (size_t)t0 * (K / 32) * kQ81xBytes;
+        const int rc = (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn)
+                                 : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn);
+        if (rc != MX_OK) return rc;
+    }
+    return MX_OK;
+}
+
+static int check_common(const void* x, const void* y, uint32_t K, uint32_t N, uint32_t T, uint32_t k_align) {
+    MX_REQUIRE_PTR(x);
+    MX_REQUIRE_PTR(y);
+    MX_REQUIRE_SHAPE(K > 0 && N > 0 && K % k_align == 0);
+    MX_REQUIRE_SHAPE(T >= 1 && T <= 16);
+    return MX_OK;
+}
+
+template <class OutT>
+static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, OutT* y, uint32_t K, uint32_t N, uint32_t T) {
+    const uint32_t k_align = fmt == 0 ? 32 : 256;
+    if (int rc = check_common(xq8, y, K, N, T, k_align)) return rc;
+    MX_REQUIRE_PTR(W);
+    MX_REQUIRE_ALIGN(xq8, 8);
+    MX_REQUIRE_ALIGN(W, fmt == 1 ? 16 : 2);
+    const uint8_t* base = static_cast<const uint8_t*>(W);
+    if (fmt == 1) {
+        GemvSeg<FmtQ4K, OutT> g{{base, K / 256 * (uint32_t)kQ4KBytes}, y, nullptr};
+        return launch_q8<FmtQ4K, OutT>(s, g, g, 1, xq8, K, N, T);
+    }
+    if (fmt == 2) {
+        GemvSeg<FmtQ6K, OutT> g{{base, K / 256 * (uint32_t)kQ6KBytes}, y, nullptr};
+        return launch_q8<FmtQ6K, OutT>(s, g, g, 1, xq8, K, N, T);
+    }
+    GemvSeg<FmtQ8Aos, OutT> g{{base, K / 32 * (uint32_t)kQ8_0Bytes}, y, nullptr};
+    return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T);
+}
+
+template <class F, bool UNSIGNED, class ActT, class OutT>
+static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, OutT* y, uint32_t K, uint32_t N) {
+    uint32_t KT = 8192;
+    if (KT > K) KT = (K + 255) / 256 * 256;
+    const uint32_t lds = KT * 4 + KT / 16 * 4;
+    const uint32_t G = pick_group(K / 32);
+    const uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
+    const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
+    const uint32_t cap = (uint32_t)cu_count() * 8;
+    dim3 grid(n_rg < cap ? n_rg : cap);
+    if (G == 32)
+        hipLaunchKernelGGL((gemv_fact_kernel<F, UNSIGNED, kRows, 32, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+    else
+        hipLaunchKernelGGL((gemv_fact_kernel<F, UNSIGNED, kRows, 64, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+    return launch_status();
+}
+
+template <class ActT, class OutT>
+static int gemv_aos_fact(int fmt, mx_stream_t s, const ActT* A, const void* W, OutT* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y, K, N, 1, fmt == 0 ? 32 : 256)) return rc;
+    MX_REQUIRE_PTR(W);
+    MX_REQUIRE_ALIGN(W, fmt == 1 ? 16 : 2);
+    const uint8_t* base = static_cast<const uint8_t*>(W);
+    if (fmt == 1) return launch_fact<FmtQ4K, true>(s, FmtQ4K::W{base, K / 256 * (uint32_t)kQ4KBytes}, A, y, K, N);
+    if (fmt == 2) return launch_fact<FmtQ6K, true>(s, FmtQ6K::W{base, K / 256 * (uint32_t)kQ6KBytes}, A, y, K, N);
+    return launch_fact<FmtQ8Aos, false>(s, FmtQ8Aos::W{base, K / 32 * (uint32_t)kQ8_0Bytes}, A, y, K, N);
+}
+
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+int mx_gemv_q4_K_q8(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return gemv_aos_q8<half_t>(1, s, x, W, reinterpret_cast<half_t*>(y), K, N, 1);
+}
+int mx_gemv_q6_K_q8(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return gemv_aos_q8<half_t>(2, s, x, W, reinterpret_cast<half_t*>(y), K, N, 1);
+}
+int mx_gemv_q8_0_q8(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return gemv_aos_q8<half_t>(0, s, x, W, reinterpret_cast<half_t*>(y), K, N, 1);
+}
+int mx_gemv_q4_K_q8_batched(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    return gemv_aos_q8<half_t>(1, s, x, W, reinterpret_cast<half_t*>(y), K, N, T);
+}
+int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    return gemv_aos_q8<half_t>(2, s, x, W, reinterpret_cast<half_t*>(y), K, N, T);
+}
+int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    return gemv_aos_q8<half_t>(0, s, x, W, reinterpret_cast<half_t*>(y), K, N, T);
+}
+int mx_gemv_q4_K_q8_f32(mx_stream_t s, const void* x, const void* W, float* y, uint32_t K, uint32_t N) {
+    return gemv_aos_q8<float>(1, s, x, W, y, K, N, 1);
+}
+int mx_gemv_q6_K_q8_f32(mx_stream_t s, const void* x, const void* W, float* y, uint32_t K, uint32_t N) {
+    return gemv_aos_q8<float>(2, s, x, W, y, K, N, 1);
+}
+int mx_gemv_q8_0_q8_f32(mx_stream_t s, const void* x, const void* W, float* y, uint32_t K, uint32_t N) {
+    return gemv_aos_q8<float>(0, s, x, W, y, K, N, 1);
+}
+
+int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K,
+                                uint32_t N, uint32_t T) {
+    if (int rc = check_common(x, y, K, N, T, 32)) return rc;
+    MX_REQUIRE_PTR(qs_W);
+    MX_REQUIRE_PTR(d_W);
+    MX_REQUIRE_ALIGN(x, 8);
+    MX_REQUIRE_ALIGN(qs_W, 16);
+    MX_REQUIRE_ALIGN(d_W, 2);
+    GemvSeg<FmtQ8Soa, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtQ8Soa, half_t>(s, g, g, 1, x, K, N, T);
+}
+int mx_gemv_q8_0_soa_q8(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K, uint32_t N) {
+    return mx_gemv_q8_0_soa_q8_batched(s, x, qs_W, d_W, y, K, N, 1);
+}
+
+int mx_gemv_mxfp4_soa_q8_batched(mx_stream_t s, const void* x, const uint8_t* qs, const uint8_t* e, uint16_t* y, uint32_t K, uint32_t N,
+                                 uint32_t T) {
+    if (int rc = check_common(x, y, K, N, T, 32)) return rc;
+    MX_REQUIRE_PTR(qs);
+    MX_REQUIRE_PTR(e);
+    MX_REQUIRE_ALIGN(x, 8);
+    MX_REQUIRE_ALIGN(qs, 16);
+    GemvSeg<FmtMxfp4Soa, half_t> g{{qs, e, K}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtMxfp4Soa, half_t>(s, g, g, 1, x, K, N, T);
+}
+int mx_gemv_mxfp4_soa_q8(mx_stream_t s, const void* x, const uint8_t* qs, const uint8_t* e, uint16_t* y, uint32_t K, uint32_t N) {
+    return mx_gemv_mxfp4_soa_q8_batched(s, x, qs, e, y, K, N, 1);
+}
+int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x, const uint8_t* gate_qs, const uint8_t* gate_e, const uint8_t* up_qs,
+                            const uint8_t* up_e, const float* gate_bias, const float* up_bias, uint16_t* gate_y, uint16_t* up_y,
+                            uint32_t K, uint32_t N) {
+    if (int rc = check_common(x, gate_y, K, N, 1, 32)) return rc;
+    MX_REQUIRE_PTR(up_y);
+    MX_REQUIRE_PTR(gate_qs);
+    MX_REQUIRE_PTR(gate_e);
+    MX_REQUIRE_PTR(up_qs);
+    MX_REQUIRE_PTR(up_e);
+    MX_REQUIRE_ALIGN(x, 8);
+    MX_REQUIRE_ALIGN(gate_qs, 16);
+    MX_REQUIRE_ALIGN(up_qs, 16);
+    GemvSeg<FmtMxfp4Soa, half_t> g{{gate_qs, gate_e, K}, reinterpret_cast<half_t*>(gate_y), gate_bias};
+    GemvSeg<FmtMxfp4Soa, half_t> u{{up_qs, up_e, K}, reinterpret_cast<half_t*>(up_y), up_bias};
+    return launch_q8<FmtMxfp4Soa, half_t>(s, g, u, 2, x, K, N, 1);
+}
+
+int mx_gemv_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return gemv_aos_fact(1, s, reinterpret_cast<const half_t*>(A), W, reinterpret_cast<half_t*>(y), K, N);
+}
+int mx_gemv_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return gemv_aos_fact(2, s, reinterpret_cast<const half_t*>(A), W, reinterpret_cast<half_t*>(y), K, N);
+}
+int mx_gemv_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return gemv_aos_fact(0, s, reinterpret_cast<const half_t*>(A), W, reinterpret_cast<half_t*>(y), K, N);
+}
+int mx_gemv_q4_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N) {
+    return gemv_aos_fact(1, s, A, W, y, K, N);
+}
+int mx_gemv_q6_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N) {
+    return gemv_aos_fact(2, s, A, W, y, K, N);
+}
+int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N) {
+    return gemv_aos_fact(0, s, A, W, y, K, N);
+}
+int mx_gemv_mxfp4_soa_f16(mx_stream_t s, const uint16_t* A, const uint8_t* qs, const uint8_t* e, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y, K, N, 1, 32)) return rc;
+    MX_REQUIRE_PTR(qs);
+    MX_REQUIRE_PTR(e);
+    MX_REQUIRE_ALIGN(qs, 16);
+    return launch_fact<FmtMxfp4Soa, false>(s, FmtMxfp4Soa::W{qs, e, K}, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y), K, N);
+}
+
+}  // extern "C"

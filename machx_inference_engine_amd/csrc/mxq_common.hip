@@ -1,0 +1,26 @@
+// mxq_common.hip — status strings, version, last-error slot.
+#include "mxq_host.h"
+
+namespace mxq {
+thread_local int g_last_hip_error = 0;
+}
+
+extern "C" {
+
+const char* mx_status_string(int status) {
+    switch (status) {
+        case MX_OK: return "ok";
+        case MX_ERR_NULL: return "required pointer is NULL";
+        case MX_ERR_SHAPE: return "dimension violates a precondition";
+        case MX_ERR_ALIGN: return "pointer violates the required alignment";
+        case MX_ERR_LAUNCH: return "HIP runtime error";
+        case MX_ERR_UNSUPPORTED: return "combination not built";
+    }
+    return "unknown status";
+}
+
+int mx_last_hip_error(void) { return mxq::g_last_hip_error; }
+
+int mx_version(void) { return 100; }
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+"""The C-ABI library: loads without a GPU, exports every symbol include/mxq.h
+declares, and rejects bad arguments before any HIP call."""
+import ctypes as C
+import os
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from machx_inference_engine_amd import _lib
+    return _lib.load(), _lib.parse_header()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    l, protos = lib
+    assert len(protos) >= 40
+    raw = C.CDLL(os.path.join(ROOT, "machx_inference_engine_amd", "libmxq.so"))
+    for name in protos:
+        assert hasattr(raw, name), name
+
+
+def test_status_strings_and_version(lib):
+    l, _ = lib
+    assert l.mx_version() >= 100
+    assert l.mx_status_string(0) == b"ok"
+    assert len({l.mx_status_string(i) for i in range(6)}) == 6
+
+
+def test_argument_validation_without_gpu(lib):
+    l, protos = lib
+    OK, NULL, SHAPE, ALIGN = 0, 1, 2, 3
+    p16, p8, p2 = 0x1000, 0x1008, 0x1002
+    # NULL pointers
+    assert l.mx_gemv_q4_K_q8(None, None, p16, p16, 4096, 4096) == NULL
+    assert l.mx_gemv_q4_K_q8(None, p16, None, p16, 4096, 4096) == NULL
+    assert l.mx_quantize_q8_1(None, None, p16, 64) == NULL
+    assert l.mx_dequant_q6_K(None, p16, None, 256) == NULL
+    # shape preconditions: K % 256 for K-quants, K % 32 for Q8_0 / MXFP4, T in 1..16, n % 32
+    assert l.mx_gemv_q4_K_q8(None, p16, p16, p16, 4096 + 32, 16) == SHAPE
+    assert l.mx_gemv_q6_K_q8(None, p16, p16, p16, 100, 16) == SHAPE
+    assert l.mx_gemv_q8_0_q8(None, p16, p16, p16, 48, 16) == SHAPE
+    assert l.mx_gemv_mxfp4_soa_q8(None, p16, p16, p16, p16, 2880 + 16, 16) == SHAPE
+    assert l.mx_gemv_q4_K_q8(None, p16, p16, p16, 4096, 0) == SHAPE
+    assert l.mx_gemv_q4_K_q8_batched(None, p16, p16, p16, 4096, 16, 0) == SHAPE
+    assert l.mx_gemv_q4_K_q8_batched(None, p16, p16, p16, 4096, 16, 17) == SHAPE
+    assert l.mx_quantize_q8_1(None, p16, p16, 33) == SHAPE
+    assert l.mx_dequant_q4_K(None, p16, p16, 255) == SHAPE
+    assert l.mx_dequant_q8_0_to_Bt(None, p16, p16, 48, 4) == SHAPE
+    # alignment: Q4_K weights 16 B, q8 stream 8 B, SoA quant plane 16 B
+    assert l.mx_gemv_q4_K_q8(None, p16, p8, p16, 4096, 16) == ALIGN
+    assert l.mx_gemv_q4_K_q8(None, 0x1004, p16, p16, 4096, 16) == ALIGN
+    assert l.mx_gemv_q8_0_soa_q8(None, p16, p8, p16, p16, 4096, 16) == ALIGN
+    assert l.mx_gemv_q6_K_q8(None, p16, 0x1001, p16, 4096, 16) == ALIGN
+    # host repackers work without a GPU
+    import numpy as np
+    blk = np.arange(17 * 3, dtype=np.uint8)
+    qs, e = np.zeros(48, np.uint8), np.zeros(3, np.uint8)
+    assert l.mx_repack_mxfp4_to_soa(blk.ctypes.data, 3, qs.ctypes.data, e.ctypes.data) == OK
+    assert e.tolist() == [0, 17, 34] and qs[:16].tolist() == list(range(1, 17))
+    assert l.mx_repack_mxfp4_to_soa(None, 3, qs.ctypes.data, e.ctypes.data) == NULL

@@ -1,0 +1,170 @@
+"""GPU parity: decode GEMV (T = 1 and batched) for Q4_K / Q6_K / Q8_0 / MXFP4,
+int-dot kernels against the q8-chain oracle, float-activation kernels against
+the float-chain oracle.  Gate: max_rel <= 1e-3 and cosine >= 0.99999."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import check, dev, host, weights
+
+pytestmark = pytest.mark.gpu
+
+
+def acts(seed, T, K):
+    """fp32 N(0,1) activations rounded to fp16 (what the fp16 entry points see)."""
+    return O.round_fp16(O.normal(seed, (T, K), 0.0, 1.0))
+
+
+def run_q8(mx, fmt, W, xq, K, N, T):
+    name = O.FMT_NAMES[fmt]
+    Wd, xd = dev(W), dev(xq)
+    if fmt == O.MXFP4:
+        qs, e = O.repack_mxfp4_to_soa(W)
+        f = mx.ops.gemv_mxfp4_soa_q8 if T == 1 else mx.ops.gemv_mxfp4_soa_q8_batched
+        args = (xd, dev(qs), dev(e), K, N) + ((T,) if T > 1 else ())
+        return host(f(*args)).astype(np.float32)
+    f = getattr(mx.ops, "gemv_%s_q8%s" % (name, "" if T == 1 else "_batched"))
+    args = (xd, Wd, K, N) + ((T,) if T > 1 else ())
+    return host(f(*args)).astype(np.float32)
+
+
+SHAPES = [(256, 8), (512, 70), (2048, 512), (4096, 300), (2816, 33)]
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0, O.MXFP4))
+@pytest.mark.parametrize("K,N", SHAPES)
+def test_gemv_q8_small_shapes(mx, fmt, K, N):
+    if fmt in (O.Q8_0, O.MXFP4) and K == 2816:
+        K = 2880  # K % 32 == 0 but not % 256 (gpt-oss hidden)
+    W = weights(fmt, 100 + fmt, N, K)
+    x = acts(200 + K, 1, K)
+    xq = host(mx.ops.quantize_q8_1(dev(x).half()))
+    assert np.array_equal(xq, O.quantize_q8_1(x))
+    ref = O.gemv_q8chain(fmt, W, xq, K, N)
+    got = run_q8(mx, fmt, W, xq, K, N, 1)
+    check(got, ref[0], "gemv_%s_q8 K=%d N=%d" % (O.FMT_NAMES[fmt], K, N))
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0, O.MXFP4))
+@pytest.mark.parametrize("T", (2, 3, 4, 5, 7, 8, 11, 16))
+def test_gemv_q8_batched(mx, fmt, T):
+    K, N = (2880, 130) if fmt == O.MXFP4 else (2048, 130)
+    W = weights(fmt, 300 + fmt, N, K)
+    x = acts(400 + T, T, K)
+    xq = O.quantize_q8_1(x)
+    ref = O.gemv_q8chain(fmt, W, xq, K, N)
+    got = run_q8(mx, fmt, W, xq, K, N, T)
+    assert got.shape == (T, N)
+    check(got, ref, "gemv_%s_q8_batched T=%d" % (O.FMT_NAMES[fmt], T))
+    # per-row numerics identical to the T=1 kernel's gate (row t alone)
+    one = run_q8(mx, fmt, W, xq[: K // 32 * 40], K, N, 1)
+    check(one, ref[0], "row 0 alone")
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+def test_gemv_q8_multi_tile_K(mx, fmt):
+    """K large enough that the activation is staged in several LDS tiles (T=8, K=14336)."""
+    K, N, T = 14336, 64, 8
+    W = weights(fmt, 500 + fmt, N, K)
+    xq = O.quantize_q8_1(acts(501, T, K))
+    check(run_q8(mx, fmt, W, xq, K, N, T), O.gemv_q8chain(fmt, W, xq, K, N), "multi-tile %s" % O.FMT_NAMES[fmt])
+
+
+def test_gemv_q8_0_soa_matches_aos(mx):
+    K, N = 4096, 96
+    W = weights(O.Q8_0, 600, N, K)
+    xq = O.quantize_q8_1(acts(601, 4, K))
+    qs, d = O.repack_q8_0_to_soa(W)
+    ref = O.gemv_q8chain(O.Q8_0, W, xq, K, N)
+    soa1 = host(mx.ops.gemv_q8_0_soa_q8(dev(xq[: K // 32 * 40]), dev(qs), dev(d), K, N)).astype(np.float32)
+    check(soa1, ref[0], "gemv_q8_0_soa_q8")
+    soa4 = host(mx.ops.gemv_q8_0_soa_q8_batched(dev(xq), dev(qs), dev(d), K, N, 4)).astype(np.float32)
+    check(soa4, ref, "gemv_q8_0_soa_q8_batched")
+    aos4 = run_q8(mx, O.Q8_0, W, xq, K, N, 4)
+    assert np.array_equal(aos4, soa4)   # same arithmetic, only the addresses differ
+
+
+def test_gemv_mxfp4_x2_bias(mx):
+    K, N = 2880, 200
+    Wg, Wu = weights(O.MXFP4, 700, N, K), weights(O.MXFP4, 701, N, K)
+    xq = O.quantize_q8_1(acts(702, 1, K))
+    bg, bu = O.normal(703, N), O.normal(704, N)
+    gq, ge = O.repack_mxfp4_to_soa(Wg)
+    uq, ue = O.repack_mxfp4_to_soa(Wu)
+    gy, uy = mx.ops.gemv_mxfp4_soa_q8_x2(dev(xq), dev(gq), dev(ge), dev(uq), dev(ue), dev(bg), dev(bu), K, N)
+    check(host(gy).astype(np.float32), O.gemv_q8chain(O.MXFP4, Wg, xq, K, N)[0] + bg, "x2 gate")
+    check(host(uy).astype(np.float32), O.gemv_q8chain(O.MXFP4, Wu, xq, K, N)[0] + bu, "x2 up")
+    gy2, uy2 = mx.ops.gemv_mxfp4_soa_q8_x2(dev(xq), dev(gq), dev(ge), dev(uq), dev(ue), None, None, K, N)
+    assert np.array_equal(host(gy2), host(mx.ops.gemv_mxfp4_soa_q8(dev(xq), dev(gq), dev(ge), K, N)))
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+@pytest.mark.parametrize("K,N", [(256, 8), (2048, 300), (4096, 512)])
+def test_gemv_float_activation(mx, fmt, K, N):
+    """W4A16-style kernels vs the reference's CPU path (fp32 dequant + fp32 dot) and its fp64 twin."""
+    name = O.FMT_NAMES[fmt]
+    W = weights(fmt, 800 + fmt, N, K)
+    x16 = acts(801, 1, K)
+    ref64 = O.gemv_f64(fmt, W, x16, K, N)[0]
+    got16 = host(getattr(mx.ops, "gemv_" + name)(dev(x16[0]).half(), dev(W), K, N)).astype(np.float32)
+    check(got16, ref64, "gemv_%s fp16" % name)
+    x32 = O.normal(802, (1, K), 0.0, 1.0)
+    got32 = host(getattr(mx.ops, "gemv_" + name)(dev(x32[0]), dev(W), K, N))
+    check(got32, O.gemv_f64(fmt, W, x32, K, N)[0], "gemv_%s fp32" % name, max_rel=1e-4)
+    # the reference's own sequential-fp32 CPU result sits within fp32 accumulation noise of ours
+    check(got32, O.gemv_f32chain(fmt, W, x32, K, N)[0], "vs fp32 chain", max_rel=2e-4)
+
+
+def test_gemv_mxfp4_f16(mx):
+    K, N = 2880, 256
+    W = weights(O.MXFP4, 900, N, K)
+    x = acts(901, 1, K)
+    qs, e = O.repack_mxfp4_to_soa(W)
+    got = host(mx.ops.gemv_mxfp4_soa_f16(dev(x[0]).half(), dev(qs), dev(e), K, N)).astype(np.float32)
+    check(got, O.gemv_f64(O.MXFP4, W, x, K, N)[0], "gemv_mxfp4_soa_f16")
+
+
+def test_gemv_q8_fp32_out_tight(mx):
+    """fp32-output twins: the fp32 fold must sit within 2e-5 of the fp64 q8-chain."""
+    K, N = 4096, 256
+    for fmt in (O.Q4_K, O.Q6_K, O.Q8_0):
+        W = weights(fmt, 1000 + fmt, N, K)
+        xq = O.quantize_q8_1(acts(1001, 1, K))
+        got = host(mx.ops.gemv_q8_f32(O.FMT_NAMES[fmt], dev(xq), dev(W), K, N))
+        check(got, O.gemv_q8chain(fmt, W, xq, K, N)[0], "gemv_%s_q8_f32" % O.FMT_NAMES[fmt], max_rel=1e-4)
+
+
+def test_gemv_integer_part_exact(mx):
+    """Weights with unit scales make the fold exact, so the kernel's integer dot
+    must equal the brute-force int64 dot bit for bit (Q8_0: d = 1)."""
+    K, N = 1024, 40
+    qs = (O.rand_bytes(1100, N * K).view(np.int8)).reshape(N, K)
+    blk = np.zeros((N, K // 32, 34), np.uint8)
+    blk[:, :, 0:2] = np.array([0x3C00], np.uint16).view(np.uint8)
+    blk[:, :, 2:] = qs.reshape(N, K // 32, 32).view(np.uint8)
+    xq = np.zeros((K // 32, 40), np.uint8)
+    q8 = O.rand_bytes(1101, K).view(np.int8).reshape(K // 32, 32)
+    xq[:, 0:4] = np.array([1.0], np.float32).view(np.uint8)
+    xq[:, 8:] = q8.view(np.uint8)
+    got = host(mx.ops.gemv_q8_f32("q8_0", dev(xq.ravel()), dev(blk.reshape(N, -1)), K, N))
+    exact = qs.astype(np.int64) @ q8.reshape(K).astype(np.int64)
+    assert np.array_equal(got.astype(np.int64), exact)   # |sum| < 2^24, so fp32 holds it exactly
+
+
+def test_full_size_properties_config1(mx):
+    """BASELINE config 1 at full size (Q4_K 4096x4096): linearity in the
+    activation scale and agreement between the int-dot and float chains at the
+    activation-quantisation noise level (max_err/rms < 3e-2, tests/unit/q8dot_test.cpp:120-135)."""
+    K = N = 4096
+    W = weights(O.Q4_K, 1200, N, K)
+    x = acts(1201, 1, K)
+    Wd = dev(W)
+    yq = host(mx.ops.gemv_q4_K_q8(mx.ops.quantize_q8_1(dev(x).half()), Wd, K, N)).astype(np.float64)
+    yf = host(mx.ops.gemv_q4_K(dev(x[0]), Wd, K, N)).astype(np.float64)
+    rms = np.sqrt(np.mean(yf ** 2))
+    assert np.abs(yq - yf).max() / rms < 3e-2
+    y2 = host(mx.ops.gemv_q4_K(dev(2 * x[0]), Wd, K, N)).astype(np.float64)
+    assert np.allclose(y2, 2 * yf, rtol=1e-6, atol=1e-6 * rms)
+    check(yf, O.gemv_f64(O.Q4_K, W, x, K, N)[0], "config1 float chain", max_rel=1e-4)
+    check(yq, O.gemv_q8chain(O.Q4_K, W, O.quantize_q8_1(x), K, N)[0], "config1 q8 chain")
