@@ -15,7 +15,10 @@ struct GemvSeg {
     const float* bias;
 };
 
-template <class F, int T, int R, int G, class OutT>
+// Persistent workgroups: each stages the activation tile(s) and then streams
+// its share of row groups.  With a single K-tile (every decode shape at T <= 2)
+// the activation is staged once per workgroup.
+template <class F, int T, int R, int G, int U, class OutT>
 __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> seg0, GemvSeg<F, OutT> seg1, const uint8_t* xq8,
                                                                 uint32_t K, uint32_t N, uint32_t KT, uint32_t T_real) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -28,13 +31,10 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
     auto xrow = [&](uint32_t t) { return xq8 + (size_t)(t < T_real ? t : T_real - 1) * q8_row_bytes; };
     const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
     const uint32_t n_tiles = (K + KT - 1) / KT;
-    ActTile<F::HAS_MIN> act;
+    ActTile act;
     bool staged = false;
     for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
         const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
-        uint32_t rows[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) rows[r] = (row0 + r < N) ? row0 + r : N - 1;
         float acc[R][T];
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -42,13 +42,18 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
             for (int t = 0; t < T; ++t) acc[r][t] = 0.f;
         for (uint32_t tile = 0; tile < n_tiles; ++tile) {
             const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
+            typename F::Cursor cu[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) cu[r] = F::cursor(seg.w, (row0 + r < N) ? row0 + r : N - 1, k0 / 64 + gl);
+            const uint32_t n_units = (kt + 63) / 64;
+            const bool half_tail = (kt & 63u) != 0;
             if (n_tiles > 1 || !staged) {
                 __syncthreads();
-                act = stage_act<F::HAS_MIN, T>(lds, xrow, k0, kt, KT);
+                act = stage_act<F::SUM_GRAN, T>(lds, xrow, k0, kt, KT);
                 __syncthreads();
                 staged = true;
             }
-            gemv_tile<F, T, R, G>(seg.w, rows, k0 / 32, kt / 32, gl, act, acc);
+            gemv_rows<F, T, R, G, U>(cu, n_units, half_tail, gl, act, acc);
         }
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -72,7 +77,7 @@ __device__ __forceinline__ float code_to_f(uint32_t w, int j) {
     return (float)(int)(int8_t)(w >> (8 * j));
 }
 
-template <class F, bool UNSIGNED, int R, int G, class ActT, class OutT>
+template <class F, int R, int G, class ActT, class OutT>
 __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w, const ActT* A, OutT* y, uint32_t K, uint32_t N, uint32_t KT) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* xa = reinterpret_cast<float*>(lds);          // [KT]
@@ -86,9 +91,6 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
     bool staged = false;
     for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
         const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
-        uint32_t rows[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) rows[r] = (row0 + r < N) ? row0 + r : N - 1;
         float acc[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -96,11 +98,11 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
             const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
             if (n_tiles > 1 || !staged) {
                 __syncthreads();
-                for (uint32_t i = threadIdx.x; i < kt / 16; i += blockDim.x) {
+                for (uint32_t i = threadIdx.x; i < (kt + 63) / 64 * 4; i += blockDim.x) {
                     float s = 0.f;
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
-                        const float v = load_act(A + k0 + i * 16 + j);
+                        const float v = (i * 16 < kt) ? load_act(A + k0 + i * 16 + j) : 0.f;
                         xa[i * 16 + j] = v;
                         s += v;
                     }
@@ -109,35 +111,34 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
                 __syncthreads();
                 staged = true;
             }
-            const uint32_t u0 = k0 / 32, n_units = kt / 32;
-            for (uint32_t ul = gl; ul < n_units; ul += G) {
+            const uint32_t n_units = (kt + 63) / 64;
+            const bool half_tail = (kt & 63u) != 0;
+            typename F::Cursor cu[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) cu[r] = F::cursor(w, (row0 + r < N) ? row0 + r : N - 1, k0 / 64 + gl);
+            for (uint32_t it = 0; it * G + gl < n_units; ++it) {
+                const uint32_t ul = it * G + gl, e0 = F::elem_off(ul);
                 typename F::Raw raw[R];
 #pragma unroll
-                for (int r = 0; r < R; ++r) raw[r] = F::load(w, rows[r], u0 + ul);
-                const uint32_t ea = F::elem_off(ul), eb = ea + F::EB_OFF;
-                float fa[16], fb[16];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float4 va = *reinterpret_cast<const float4*>(xa + ea + 4 * i);
-                    const float4 vb = *reinterpret_cast<const float4*>(xa + eb + 4 * i);
-                    fa[4 * i] = va.x; fa[4 * i + 1] = va.y; fa[4 * i + 2] = va.z; fa[4 * i + 3] = va.w;
-                    fb[4 * i] = vb.x; fb[4 * i + 1] = vb.y; fb[4 * i + 2] = vb.z; fb[4 * i + 3] = vb.w;
-                }
-                const float sa = s16[ea >> 4], sb = s16[eb >> 4];
+                for (int r = 0; r < R; ++r) raw[r] = load_unit<F, G>(cu[r], it, half_tail && ul == n_units - 1);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     Unit un;
-                    F::decode(raw[r], u0 + ul, un);
-                    float da = 0.f, db = 0.f;
+                    F::decode(raw[r], cu[r], un);
+                    float v = 0.f;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t eg = e0 + g * F::GROUP_OFF;
+                        float dq = 0.f;
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            da += fa[4 * i + j] * code_to_f<UNSIGNED>(un.a[i], j);
-                            db += fb[4 * i + j] * code_to_f<UNSIGNED>(un.b[i], j);
+                        for (int i = 0; i < 4; ++i) {
+                            const float4 x = *reinterpret_cast<const float4*>(xa + eg + 4 * i);
+                            dq += x.x * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 0) + x.y * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 1) +
+                                  x.z * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 2) + x.w * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 3);
                         }
-                    float v = un.ca * da + un.cb * db;
-                    if (F::HAS_MIN) v -= un.ma * sa + un.mb * sb;
+                        v += un.c[g] * dq;
+                        if (F::SUM_GRAN != 0) v -= un.m[g] * s16[eg >> 4];
+                    }
                     acc[r] += v;
                 }
             }
@@ -161,26 +162,38 @@ static int cu_count() {
 }
 
 constexpr uint32_t kLdsBudget = 48 * 1024;
-constexpr int kRows = 2;
+constexpr int kRows = 2;             // rows per lane group, float-activation kernels
+constexpr uint32_t kWgsPerCu = 4;    // persistent grid: workgroups per CU
+// rows per lane group / unroll of the unit walk: one row and two units in flight
+// for a single token, two rows sharing each activation read when batched
+template <int T> struct GemvShape { static constexpr int R = (T == 1) ? 1 : 2, U = (T == 1) ? 2 : 1; };
 
+// lanes per row: the G in {16, 32, 64} that wastes the fewest lane slots, larger on ties
 static uint32_t pick_group(uint32_t units) {
-    const uint32_t w64 = (units + 63) / 64 * 64, w32 = (units + 31) / 32 * 32;
-    return w32 < w64 ? 32 : 64;
+    uint32_t best = 64, waste = (units + 63) / 64 * 64 - units;
+    for (uint32_t g : {32u, 16u}) {
+        const uint32_t w = (units + g - 1) / g * g - units;
+        if (w < waste) { best = g; waste = w; }
+    }
+    return best;
 }
 
 template <class F, int T, int G, class OutT>
 static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8,
                         uint32_t K, uint32_t N, uint32_t T_real) {
-    constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
-    const uint32_t per_elem_x8 = F::HAS_MIN ? 11 : 9;  // bytes per activation element * 8
-    uint32_t KT = (kLdsBudget * 8 / (per_elem_x8 * T)) / 256 * 256;
-    if (KT > K) KT = (K + 255) / 256 * 256;
-    if (KT == 0) return MX_ERR_SHAPE;
+    constexpr int R = GemvShape<T>::R, U = GemvShape<T>::U;
+    constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
+    const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);   // LDS bytes per 32 activation elements
+    const uint32_t KT_max = (kLdsBudget / (per_elem_x32 * T)) * 32 / 256 * 256;
+    if (KT_max == 0) return MX_ERR_SHAPE;
+    const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
+    const uint32_t KT = (K256 + n_tiles - 1) / n_tiles * 256;   // balanced tiles
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
-    const uint32_t cap = (uint32_t)cu_count() * 8;
-    dim3 grid(n_rg < cap ? n_rg : cap, nseg);
-    const uint32_t lds = act_tile_bytes(T, KT, F::HAS_MIN);
-    hipLaunchKernelGGL((gemv_q8_kernel<F, T, kRows, G, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real);
+    const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu / nseg;
+    const uint32_t per = (n_rg + cap - 1) / cap;                // row groups per workgroup
+    dim3 grid((n_rg + per - 1) / per, nseg);
+    const uint32_t lds = act_tile_bytes(T, KT, F::SUM_GRAN);
+    hipLaunchKernelGGL((gemv_q8_kernel<F, T, R, G, U, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real);
     return launch_status();
 }
 
@@ -204,15 +217,16 @@ static int launch_q8_g(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg
 template <class F, class OutT>
 static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, int nseg, const void* xq8, uint32_t K, uint32_t N, uint32_t T) {
     const uint8_t* x = static_cast<const uint8_t*>(xq8);
-    const uint32_t G = pick_group(K / 32);
+    const uint32_t G = pick_group((K + 63) / 64);
     for (uint32_t t0 = 0; t0 < T; t0 += 8) {
         const uint32_t tn = (T - t0 < 8) ? T - t0 : 8;
         GemvSeg<F, OutT> a = s0, b = s1;
         a.y = s0.y + (size_t)t0 * N;
         if (nseg > 1) b.y = s1.y + (size_t)t0 * N;
         const uint8_t* xt = x + (size_t)t0 * (K / 32) * kQ81xBytes;
-        const int rc = (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn)
-                                 : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn);
+        const int rc = (G == 16)   ? launch_q8_g<F, 16, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn)
+                       : (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn)
+                                   : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn);
         if (rc != MX_OK) return rc;
     }
     return MX_OK;
@@ -246,20 +260,22 @@ static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, O
     return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T);
 }
 
-template <class F, bool UNSIGNED, class ActT, class OutT>
+template <class F, class ActT, class OutT>
 static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, OutT* y, uint32_t K, uint32_t N) {
     uint32_t KT = 8192;
     if (KT > K) KT = (K + 255) / 256 * 256;
     const uint32_t lds = KT * 4 + KT / 16 * 4;
-    const uint32_t G = pick_group(K / 32);
+    const uint32_t G = pick_group((K + 63) / 64);
     const uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
     const uint32_t cap = (uint32_t)cu_count() * 8;
     dim3 grid(n_rg < cap ? n_rg : cap);
-    if (G == 32)
-        hipLaunchKernelGGL((gemv_fact_kernel<F, UNSIGNED, kRows, 32, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+    if (G == 16)
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+    else if (G == 32)
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 32, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
     else
-        hipLaunchKernelGGL((gemv_fact_kernel<F, UNSIGNED, kRows, 64, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 64, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
     return launch_status();
 }
 
@@ -269,9 +285,9 @@ static int gemv_aos_fact(int fmt, mx_stream_t s, const ActT* A, const void* W, O
     MX_REQUIRE_PTR(W);
     MX_REQUIRE_ALIGN(W, fmt == 1 ? 16 : 2);
     const uint8_t* base = static_cast<const uint8_t*>(W);
-    if (fmt == 1) return launch_fact<FmtQ4K, true>(s, FmtQ4K::W{base, K / 256 * (uint32_t)kQ4KBytes}, A, y, K, N);
-    if (fmt == 2) return launch_fact<FmtQ6K, true>(s, FmtQ6K::W{base, K / 256 * (uint32_t)kQ6KBytes}, A, y, K, N);
-    return launch_fact<FmtQ8Aos, false>(s, FmtQ8Aos::W{base, K / 32 * (uint32_t)kQ8_0Bytes}, A, y, K, N);
+    if (fmt == 1) return launch_fact<FmtQ4K>(s, FmtQ4K::W{base, K / 256 * (uint32_t)kQ4KBytes}, A, y, K, N);
+    if (fmt == 2) return launch_fact<FmtQ6K>(s, FmtQ6K::W{base, K / 256 * (uint32_t)kQ6KBytes}, A, y, K, N);
+    return launch_fact<FmtQ8Aos>(s, FmtQ8Aos::W{base, K / 32 * (uint32_t)kQ8_0Bytes}, A, y, K, N);
 }
 
 }  // namespace mxq
@@ -376,7 +392,7 @@ int mx_gemv_mxfp4_soa_f16(mx_stream_t s, const uint16_t* A, const uint8_t* qs, c
     MX_REQUIRE_PTR(qs);
     MX_REQUIRE_PTR(e);
     MX_REQUIRE_ALIGN(qs, 16);
-    return launch_fact<FmtMxfp4Soa, false>(s, FmtMxfp4Soa::W{qs, e, K}, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y), K, N);
+    return launch_fact<FmtMxfp4Soa>(s, FmtMxfp4Soa::W{qs, e, K}, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y), K, N);
 }
 
 }  // extern "C"

@@ -1,16 +1,26 @@
 // mxq_formats.h — per-format "weight unit" decoders used by the GEMV kernels.
 //
-// A unit is the slice of one weight row that one lane handles per step: 32
-// weights, delivered as two groups (A, B) of 16 int8 codes (4 dwords each) plus
-// the fp32 coefficients of the fold
-//     acc += ca * (d8[A] * idotA) - ma * s16[A] + cb * (d8[B] * idotB) - mb * s16[B]
-// where idot = sum(code * q8), d8 = activation block scale, s16 = d8 * sum(q8)
-// over the 16 activations of the group.  Consecutive units of a row are
-// consecutive 16- or 32-byte chunks of the weight stream, so a wave's loads
-// are fully coalesced 128-bit loads.
+// A unit is the slice of one weight row that one lane handles per step: 64
+// weights, delivered as four groups of 16 int8 codes (4 dwords each) plus the
+// fp32 coefficients of the fold
+//     acc += sum_g  c[g] * (d8[g] * idot[g]) - m[g] * s[g]
+// where idot[g] = sum(code * q8) over the group, d8 = scale of the activation
+// block the group lies in and s = d8 * sum(q8) over the group (the min / offset
+// term of the K-quants).  Group g covers row elements
+// [elem_off(u) + GROUP_OFF * g, +16).  Consecutive units of a row are
+// consecutive chunks of the weight stream, so a wave's loads are coalesced
+// 128-bit loads of whole super-blocks, and a block header is unpacked by four
+// lanes only.
 //
-// Group A covers row elements [ea, ea+16), group B [ea + EB_OFF, +16) with
-// ea = F::elem_off(u).
+// PAIRED formats: groups (0,1) lie in one 32-element activation block and share
+// one weight scale, likewise (2,3); their integer dots are accumulated in one
+// chain and folded once.
+//
+// Addressing: a lane that walks units u, u+G, u+2G ... of a row keeps a Cursor
+// (the address of its first unit); step i of the walk loads at
+// cursor + i * G * bytes-per-unit, a compile-time offset in unrolled code.  The
+// position of a unit inside its 256-element super-block (u % 4) is the same for
+// every step of a lane because G is a multiple of 4.
 #pragma once
 
 #include "mxq_device.h"
@@ -18,204 +28,311 @@
 namespace mxq {
 
 struct Unit {
-    uint32_t a[4], b[4];
-    float ca, ma, cb, mb;
+    uint32_t q[4][4];
+    float c[4], m[4];
 };
 
-// 128-bit load from a 2-byte aligned address (Q6_K and AoS Q8_0 blocks are only
-// 2-byte aligned).  Global memory accepts unaligned vector loads on gfx950.
+// Loads from 2-byte aligned addresses (Q6_K and AoS Q8_0 blocks are only 2-byte
+// aligned).  Global memory accepts unaligned vector loads on gfx950.
 __device__ __forceinline__ uint4 load_u4_a2(const uint8_t* p) {
     struct __attribute__((packed, aligned(2))) U4 { uint32_t x, y, z, w; };
     const U4 v = *reinterpret_cast<const U4*>(p);
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+__device__ __forceinline__ uint2 load_u2_a2(const uint8_t* p) {
+    struct __attribute__((packed, aligned(2))) U2 { uint32_t x, y; };
+    const U2 v = *reinterpret_cast<const U2*>(p);
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t load_u1_a2(const uint8_t* p) {
+    struct __attribute__((packed, aligned(2))) U1 { uint32_t x; };
+    return reinterpret_cast<const U1*>(p)->x;
+}
 
 // ---------------------------------------------------------------- Q4_K (AoS GGUF blocks)
-// Unit u = (block u/8, qs chunk c = u%8).  Chunk c holds qs[16c, 16c+16): low
-// nibbles are elements 64g + 16h + [0,16) of sub-block 2g, high nibbles the same
-// positions of sub-block 2g+1, g = c/2, h = c%2 (include/ie/dequant_ref.hpp:38-53).
+// Unit u = (block u/4, 64-element group g = u%4): the 32 bytes qs[32g, 32g+32),
+// whose low nibbles are sub-block 2g and high nibbles sub-block 2g+1
+// (include/ie/dequant_ref.hpp:38-53).  Groups: 0,1 = sub-block 2g (elements
+// 0..15, 16..31), 2,3 = sub-block 2g+1.
 struct FmtQ4K {
     struct W {
         const uint8_t* base;
         uint32_t row_bytes;
     };
-    struct Raw {
-        uint4 qs, hdr;
+    struct Cursor {
+        const uint8_t* blk;   // block of the lane's first unit
+        uint32_t g;
     };
-    static constexpr bool HAS_MIN = true;
-    static constexpr uint32_t EB_OFF = 32;
+    struct Raw {
+        uint4 hdr, q0, q1;
+    };
+    static constexpr int SUM_GRAN = 32;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
     static constexpr uint32_t K_ALIGN = 256;
-    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) {
-        const uint32_t c = u & 7u;
-        return (u >> 3) * 256u + (c >> 1) * 64u + (c & 1u) * 16u;
+    static constexpr bool CODES_UNSIGNED = true;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {w.base + (size_t)n * w.row_bytes + (size_t)(u >> 2) * kQ4KBytes, u & 3u};
     }
-    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t u) {
-        const uint8_t* blk = w.base + (size_t)n * w.row_bytes + (size_t)(u >> 3) * kQ4KBytes;
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const uint8_t* blk = cu.blk + (size_t)i * (G / 4 * kQ4KBytes);
+        const uint4* q = reinterpret_cast<const uint4*>(blk + 16 + cu.g * 32u);
         Raw r;
         r.hdr = *reinterpret_cast<const uint4*>(blk);
-        r.qs = *reinterpret_cast<const uint4*>(blk + 16 + (u & 7u) * 16u);
+        r.q0 = q[0];
+        r.q1 = q[1];
         return r;
     }
-    __device__ static __forceinline__ void decode(const Raw& r, uint32_t u, Unit& o) {
-        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) {
+        const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w}, q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            o.a[i] = q[i] & 0x0F0F0F0Fu;
-            o.b[i] = (q[i] >> 4) & 0x0F0F0F0Fu;
+            o.q[0][i] = q0[i] & 0x0F0F0F0Fu;
+            o.q[1][i] = q1[i] & 0x0F0F0F0Fu;
+            o.q[2][i] = (q0[i] >> 4) & 0x0F0F0F0Fu;
+            o.q[3][i] = (q1[i] >> 4) & 0x0F0F0F0Fu;
         }
         uint32_t sc, mn;
-        q4k_scale_pair(r.hdr.y, r.hdr.z, r.hdr.w, (int)((u & 7u) >> 1), sc, mn);
+        q4k_scale_pair(r.hdr.y, r.hdr.z, r.hdr.w, (int)cu.g, sc, mn);
         const float d = h2f(r.hdr.x & 0xFFFFu), dmin = h2f(r.hdr.x >> 16);
-        o.ca = d * (float)(sc & 0xFFu);
-        o.cb = d * (float)(sc >> 8);
-        o.ma = dmin * (float)(mn & 0xFFu);
-        o.mb = dmin * (float)(mn >> 8);
+        o.c[0] = o.c[1] = d * (float)(sc & 0xFFu);
+        o.c[2] = o.c[3] = d * (float)(sc >> 8);
+        o.m[0] = o.m[1] = dmin * (float)(mn & 0xFFu);
+        o.m[2] = o.m[3] = dmin * (float)(mn >> 8);
     }
 };
 
 // ---------------------------------------------------------------- Q6_K (AoS GGUF blocks)
-// Unit u = (block u/8, ql chunk c = u%8), h = c/4, r = c%4.  Chunk c holds
-// ql[16c, 16c+16) whose low nibbles are elements 128h + 32(r/2) + 16(r%2) + [0,16)
-// and whose high nibbles are the elements 64 further on; the matching 2-bit
-// planes sit in qh[32h + 16(r%2) + [0,16)] at bit 2(r/2) and 2(r/2)+4
-// (include/ie/dequant_ref.hpp:78-96).  Codes are kept unsigned (0..63); the -32
-// offset goes into the min term: ma = 32 * ca.
+// Unit u = (block u/4, half h = (u/2)%2, j = u%2): ql[64h + 16j + [0,16)] (subs 0
+// and 2 in its low / high nibbles), ql[64h + 32 + 16j + [0,16)] (subs 1 and 3) and
+// qh[32h + 16j + [0,16)] whose four 2-bit fields are the high bits of subs 0..3
+// (include/ie/dequant_ref.hpp:78-96).  Group s = sub s: elements
+// 128h + 32s + 16j + [0,16), per-16 scale scales[8h + 2s + j].  Codes stay
+// unsigned (0..63); the -32 offset goes into the min term: m = 32 * c.
 struct FmtQ6K {
     struct W {
         const uint8_t* base;
         uint32_t row_bytes;
     };
+    struct Cursor {
+        const uint8_t* blk;
+        uint32_t hj;          // 2h + j
+    };
     struct Raw {
-        uint4 ql, qh;
-        int sca, scb;
+        uint4 qla, qlb, qh;
+        uint2 sc;             // scales[8h .. 8h+8)
         uint32_t d;
     };
-    static constexpr bool HAS_MIN = true;
-    static constexpr uint32_t EB_OFF = 64;
+    static constexpr int SUM_GRAN = 16;
+    static constexpr bool PAIRED = false;
+    static constexpr uint32_t GROUP_OFF = 32;
     static constexpr uint32_t K_ALIGN = 256;
+    static constexpr bool CODES_UNSIGNED = true;
     __device__ static __forceinline__ uint32_t elem_off(uint32_t u) {
-        const uint32_t c = u & 7u;
-        return (u >> 3) * 256u + (c >> 2) * 128u + ((c >> 1) & 1u) * 32u + (c & 1u) * 16u;
+        return (u >> 2) * 256u + ((u >> 1) & 1u) * 128u + (u & 1u) * 16u;
     }
-    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t u) {
-        const uint8_t* blk = w.base + (size_t)n * w.row_bytes + (size_t)(u >> 3) * kQ6KBytes;
-        const uint32_t c = u & 7u, h = c >> 2, r = c & 3u;
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {w.base + (size_t)n * w.row_bytes + (size_t)(u >> 2) * kQ6KBytes, u & 3u};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const uint8_t* blk = cu.blk + (size_t)i * (G / 4 * kQ6KBytes);
+        const uint32_t h = cu.hj >> 1, j = cu.hj & 1u;
         Raw o;
-        o.ql = load_u4_a2(blk + c * 16u);
-        o.qh = load_u4_a2(blk + 128 + (h * 2u + (r & 1u)) * 16u);
-        const int8_t* sc = reinterpret_cast<const int8_t*>(blk + 192 + h * 8u + (r >> 1) * 2u + (r & 1u));
-        o.sca = sc[0];
-        o.scb = sc[4];
+        o.qla = load_u4_a2(blk + 64u * h + 16u * j);
+        o.qlb = load_u4_a2(blk + 64u * h + 32u + 16u * j);
+        o.qh = load_u4_a2(blk + 128 + 32u * h + 16u * j);
+        o.sc = load_u2_a2(blk + 192 + 8u * h);
         o.d = *reinterpret_cast<const uint16_t*>(blk + 208);
         return o;
     }
-    __device__ static __forceinline__ void decode(const Raw& r, uint32_t u, Unit& o) {
-        const uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
-        const uint32_t sh = ((u >> 1) & 1u) * 2u;
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) {
+        const uint32_t la[4] = {r.qla.x, r.qla.y, r.qla.z, r.qla.w}, lb[4] = {r.qlb.x, r.qlb.y, r.qlb.z, r.qlb.w};
+        const uint32_t qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t hsh = qh[i] >> sh;
-            o.a[i] = (ql[i] & 0x0F0F0F0Fu) | ((hsh & 0x03030303u) << 4);
-            o.b[i] = ((ql[i] >> 4) & 0x0F0F0F0Fu) | (hsh & 0x30303030u);
+            o.q[0][i] = (la[i] & 0x0F0F0F0Fu) | ((qh[i] << 4) & 0x30303030u);
+            o.q[1][i] = (lb[i] & 0x0F0F0F0Fu) | ((qh[i] << 2) & 0x30303030u);
+            o.q[2][i] = ((la[i] >> 4) & 0x0F0F0F0Fu) | (qh[i] & 0x30303030u);
+            o.q[3][i] = ((lb[i] >> 4) & 0x0F0F0F0Fu) | ((qh[i] >> 2) & 0x30303030u);
         }
         const float d = h2f(r.d);
-        o.ca = d * (float)r.sca;
-        o.cb = d * (float)r.scb;
-        o.ma = 32.f * o.ca;
-        o.mb = 32.f * o.cb;
+        const uint32_t j8 = (cu.hj & 1u) * 8u;   // scale of sub s = byte 2s + j of sc
+        o.c[0] = d * (float)(int)(int8_t)(r.sc.x >> j8);
+        o.c[1] = d * (float)(int)(int8_t)(r.sc.x >> (16u + j8));
+        o.c[2] = d * (float)(int)(int8_t)(r.sc.y >> j8);
+        o.c[3] = d * (float)(int)(int8_t)(r.sc.y >> (16u + j8));
+#pragma unroll
+        for (int g = 0; g < 4; ++g) o.m[g] = 32.f * o.c[g];
     }
 };
 
 // ---------------------------------------------------------------- Q8_0, SoA planes
 // qs[n*K + k] int8, d[n*(K/32) + b] fp16 bits (src/ops/gemv_q8dot.cpp:601-607).
-// Unit u = block u: 32 bytes of qs, one scale.
+// Unit u = blocks 2u, 2u+1: 64 bytes of qs, two scales.
 struct FmtQ8Soa {
     struct W {
         const int8_t* qs;
         const uint16_t* d;
         uint32_t K;
     };
-    struct Raw {
-        uint4 lo, hi;
-        uint32_t d;
+    struct Cursor {
+        const uint4* qs;
+        const uint8_t* d;
     };
-    static constexpr bool HAS_MIN = false;
-    static constexpr uint32_t EB_OFF = 16;
+    struct Raw {
+        uint4 q[4];
+        uint32_t d2;   // d of block 2u | d of block 2u+1 << 16
+    };
+    static constexpr int SUM_GRAN = 0;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
     static constexpr uint32_t K_ALIGN = 32;
-    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 32u; }
-    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t u) {
-        const uint4* p = reinterpret_cast<const uint4*>(w.qs + (size_t)n * w.K + (size_t)u * 32u);
+    static constexpr bool CODES_UNSIGNED = false;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {reinterpret_cast<const uint4*>(w.qs + (size_t)n * w.K + (size_t)u * 64u),
+                reinterpret_cast<const uint8_t*>(w.d + (size_t)n * (w.K >> 5) + 2u * u)};
+    }
+    // `half_only`: the row ends after the unit's first block (K % 64 == 32)
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool half_only = false) {
+        const uint4* p = cu.qs + (size_t)i * (G * 4);
         Raw r;
-        r.lo = p[0];
-        r.hi = p[1];
-        r.d = w.d[(size_t)n * (w.K >> 5) + u];
+        r.q[0] = p[0];
+        r.q[1] = p[1];
+        if (half_only) {
+            r.q[2] = r.q[3] = make_uint4(0, 0, 0, 0);
+            r.d2 = *reinterpret_cast<const uint16_t*>(cu.d + (size_t)i * (G * 4));
+        } else {
+            r.q[2] = p[2];
+            r.q[3] = p[3];
+            r.d2 = load_u1_a2(cu.d + (size_t)i * (G * 4));
+        }
         return r;
     }
-    __device__ static __forceinline__ void decode(const Raw& r, uint32_t, Unit& o) {
-        o.a[0] = r.lo.x; o.a[1] = r.lo.y; o.a[2] = r.lo.z; o.a[3] = r.lo.w;
-        o.b[0] = r.hi.x; o.b[1] = r.hi.y; o.b[2] = r.hi.z; o.b[3] = r.hi.w;
-        o.ca = o.cb = h2f(r.d);
-        o.ma = o.mb = 0.f;
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            o.q[g][0] = r.q[g].x; o.q[g][1] = r.q[g].y; o.q[g][2] = r.q[g].z; o.q[g][3] = r.q[g].w;
+            o.m[g] = 0.f;
+        }
+        o.c[0] = o.c[1] = h2f(r.d2 & 0xFFFFu);
+        o.c[2] = o.c[3] = h2f(r.d2 >> 16);
     }
 };
 
 // ---------------------------------------------------------------- Q8_0, AoS GGUF blocks
-// 34-byte blocks {fp16 d; int8 qs[32]}: one lane per block, quants read as two
-// 128-bit loads at 2-byte alignment.
+// 34-byte blocks {fp16 d; int8 qs[32]}: one lane per block pair (68 bytes),
+// quants read as four 128-bit loads at 2-byte alignment.
 struct FmtQ8Aos {
     struct W {
         const uint8_t* base;
         uint32_t row_bytes;
     };
+    struct Cursor {
+        const uint8_t* blk;
+    };
     typedef FmtQ8Soa::Raw Raw;
-    static constexpr bool HAS_MIN = false;
-    static constexpr uint32_t EB_OFF = 16;
+    static constexpr int SUM_GRAN = 0;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
     static constexpr uint32_t K_ALIGN = 32;
-    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 32u; }
-    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t u) {
-        const uint8_t* blk = w.base + (size_t)n * w.row_bytes + (size_t)u * kQ8_0Bytes;
+    static constexpr bool CODES_UNSIGNED = false;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {w.base + (size_t)n * w.row_bytes + (size_t)u * (2 * kQ8_0Bytes)};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool half_only = false) {
+        const uint8_t* blk = cu.blk + (size_t)i * (G * 2 * kQ8_0Bytes);
         Raw r;
-        r.d = *reinterpret_cast<const uint16_t*>(blk);
-        r.lo = load_u4_a2(blk + 2);
-        r.hi = load_u4_a2(blk + 18);
+        r.d2 = *reinterpret_cast<const uint16_t*>(blk);
+        r.q[0] = load_u4_a2(blk + 2);
+        r.q[1] = load_u4_a2(blk + 18);
+        if (half_only) {
+            r.q[2] = r.q[3] = make_uint4(0, 0, 0, 0);
+        } else {
+            r.d2 |= (uint32_t)*reinterpret_cast<const uint16_t*>(blk + 34) << 16;
+            r.q[2] = load_u4_a2(blk + 36);
+            r.q[3] = load_u4_a2(blk + 52);
+        }
         return r;
     }
-    __device__ static __forceinline__ void decode(const Raw& r, uint32_t u, Unit& o) { FmtQ8Soa::decode(r, u, o); }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
+        FmtQ8Soa::decode(r, FmtQ8Soa::Cursor{}, o);
+    }
 };
 
 // ---------------------------------------------------------------- MXFP4, SoA planes
 // qs_plane[n*(K/2) + 16b + j], e_plane[n*(K/32) + b] (src/ops/gemv_mxfp4.cpp:13-16).
-// Unit u = block u: 16 bytes of codes (low nibbles = elements 0..15, high =
-// 16..31), one E8M0 exponent.  Codes become doubled E2M1 values as int8; the
-// block scale is 2^(e-128).
+// Unit u = blocks 2u, 2u+1: 32 bytes of codes (per block: low nibbles = elements
+// 0..15, high = 16..31), two E8M0 exponents.  Codes become doubled E2M1 values as
+// int8; the block scale is 2^(e-128).
 struct FmtMxfp4Soa {
     struct W {
         const uint8_t* qs;
         const uint8_t* e;
         uint32_t K;
     };
-    struct Raw {
-        uint4 qs;
-        uint32_t e;
+    struct Cursor {
+        const uint4* qs;
+        const uint8_t* e;
     };
-    static constexpr bool HAS_MIN = false;
-    static constexpr uint32_t EB_OFF = 16;
+    struct Raw {
+        uint4 qa, qb;
+        uint32_t e2;
+    };
+    static constexpr int SUM_GRAN = 0;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
     static constexpr uint32_t K_ALIGN = 32;
-    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 32u; }
-    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t u) {
+    static constexpr bool CODES_UNSIGNED = false;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {reinterpret_cast<const uint4*>(w.qs + (size_t)n * (w.K >> 1) + (size_t)u * 32u), w.e + (size_t)n * (w.K >> 5) + 2u * u};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool half_only = false) {
+        const uint4* p = cu.qs + (size_t)i * (G * 2);
+        const uint8_t* e = cu.e + (size_t)i * (G * 2);
         Raw r;
-        r.qs = *reinterpret_cast<const uint4*>(w.qs + (size_t)n * (w.K >> 1) + (size_t)u * 16u);
-        r.e = w.e[(size_t)n * (w.K >> 5) + u];
+        r.qa = p[0];
+        if (half_only) {
+            r.qb = make_uint4(0, 0, 0, 0);
+            r.e2 = e[0];
+        } else {
+            r.qb = p[1];
+            r.e2 = (uint32_t)e[0] | ((uint32_t)e[1] << 8);
+        }
         return r;
     }
-    __device__ static __forceinline__ void decode(const Raw& r, uint32_t, Unit& o) {
-        mxfp4_decode_word(r.qs.x, o.a[0], o.b[0]);
-        mxfp4_decode_word(r.qs.y, o.a[1], o.b[1]);
-        mxfp4_decode_word(r.qs.z, o.a[2], o.b[2]);
-        mxfp4_decode_word(r.qs.w, o.a[3], o.b[3]);
-        o.ca = o.cb = e8m0_half(r.e);
-        o.ma = o.mb = 0.f;
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
+        mxfp4_decode_word(r.qa.x, o.q[0][0], o.q[1][0]);
+        mxfp4_decode_word(r.qa.y, o.q[0][1], o.q[1][1]);
+        mxfp4_decode_word(r.qa.z, o.q[0][2], o.q[1][2]);
+        mxfp4_decode_word(r.qa.w, o.q[0][3], o.q[1][3]);
+        mxfp4_decode_word(r.qb.x, o.q[2][0], o.q[3][0]);
+        mxfp4_decode_word(r.qb.y, o.q[2][1], o.q[3][1]);
+        mxfp4_decode_word(r.qb.z, o.q[2][2], o.q[3][2]);
+        mxfp4_decode_word(r.qb.w, o.q[2][3], o.q[3][3]);
+        o.c[0] = o.c[1] = e8m0_half(r.e2 & 0xFFu);
+        o.c[2] = o.c[3] = e8m0_half(r.e2 >> 8);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) o.m[g] = 0.f;
     }
 };
+
+// K-quant loads never run past a row (K % 256 == 0), so they ignore half_only.
+template <class F, int G>
+__device__ __forceinline__ typename F::Raw load_unit(const typename F::Cursor& cu, uint32_t i, bool half_only) {
+    if constexpr (F::K_ALIGN == 256) {
+        return F::template load<G>(cu, i);
+    } else {
+        return F::template load<G>(cu, i, half_only);
+    }
+}
 
 }  // namespace mxq

@@ -2,13 +2,14 @@
 // fused gate/up and expert-indexed entry points.
 //
 // Work decomposition (wave64):
-//   * a group of G lanes (G = 32 or 64) owns R consecutive weight rows; lane l of
-//     the group walks units l, l+G, l+2G ... of each row, so one wave-wide load
-//     instruction fetches 64 consecutive 16-byte chunks of a row (coalesced
-//     128-bit loads of whole super-blocks);
+//   * a group of G lanes (G = 16, 32 or 64) owns R consecutive weight rows; lane l
+//     of the group walks 64-weight units l, l+G, l+2G ... of each row, so one
+//     wave-wide load instruction fetches consecutive 16-byte chunks of a row
+//     (coalesced 128-bit loads of whole super-blocks);
 //   * the T activation rows (block_q8_1x streams) are staged once per K-tile in
-//     LDS as three planes — int8 quants, fp32 block scales, fp32 per-16 sums —
-//     and every lane reads the 2 x 16 quants that face its unit with two
+//     LDS as two planes — the int8 quants and a header plane holding the block
+//     scale d8 (plus, for the K-quants, d8 * sum(q8) per 32 or per 16 elements) —
+//     and every lane reads the 64 quants that face its unit with four
 //     ds_read_b128;
 //   * scale/min unpacking, the int8 dot (v_dot4_i32_i8) and the fp32 fold run in
 //     registers; the per-row result is reduced across the group with DPP.
@@ -22,90 +23,141 @@ namespace mxq {
 constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / 64;
 
-// LDS footprint of one activation tile.
-__host__ __device__ constexpr uint32_t act_tile_bytes(uint32_t T, uint32_t KT, bool has_min) {
-    return T * (KT + KT / 8 + (has_min ? KT / 4 : 0));
+// Header plane entry size per 32 activation elements:
+//   SUM_GRAN 0  : float  d8                       (4 B / 32)
+//   SUM_GRAN 32 : float2 {d8, d8*sum32}           (8 B / 32)
+//   SUM_GRAN 16 : float2 {d8, d8*sum16} per 16    (16 B / 32)
+__host__ __device__ constexpr uint32_t hdr_bytes_per32(int sum_gran) { return sum_gran == 0 ? 4 : (sum_gran == 32 ? 8 : 16); }
+__host__ __device__ constexpr uint32_t act_tile_bytes(uint32_t T, uint32_t KT, int sum_gran) {
+    return T * (KT + KT / 32 * hdr_bytes_per32(sum_gran));
 }
 
-template <bool HAS_MIN>
 struct ActTile {
-    const uint4* qs;    // [T][KT/16] 16-quant chunks
-    const float* d8;    // [T][KT/32]
-    const float* s16;   // [T][KT/16]   (HAS_MIN only)
+    const uint4* qs;      // [T][KT/16] 16-quant chunks
+    const uint8_t* hdr;   // [T][KT/32] entries, see hdr_bytes_per32
     uint32_t KT;
 };
 
 // Stage T q8_1x rows, elements [k0, k0+kt), into LDS.  `xrow(t)` -> pointer to
 // the first block of activation row t.  All threads of the block call this.
-template <bool HAS_MIN, int T, class RowFn>
-__device__ __forceinline__ ActTile<HAS_MIN> stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc) {
+template <int SUM_GRAN, int T, class RowFn>
+__device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc) {
     uint4* qs = reinterpret_cast<uint4*>(lds);
-    float* d8 = reinterpret_cast<float*>(lds + (size_t)T * KT_alloc);
-    float* s16 = d8 + (size_t)T * (KT_alloc / 32);
-    const uint32_t halves = kt / 16;
+    uint8_t* hdr = lds + (size_t)T * KT_alloc;
+    const uint32_t halves = (kt + 63) / 64 * 4;   // padded to whole 64-element units with zeros
     for (uint32_t i = threadIdx.x; i < (uint32_t)T * halves; i += blockDim.x) {
         const uint32_t t = i / halves, hb = i - t * halves;
-        const uint8_t* blk = xrow(t) + (size_t)(k0 / 32 + (hb >> 1)) * kQ81xBytes;
-        const uint2* q = reinterpret_cast<const uint2*>(blk + 8 + (hb & 1u) * 16u);
-        const uint2 q0 = q[0], q1 = q[1];
-        const float d = *reinterpret_cast<const float*>(blk);
+        uint2 q0 = make_uint2(0, 0), q1 = q0;
+        float2 ds = make_float2(0.f, 0.f);                          // {d, s = d * sum32}
+        if (hb * 16 < kt) {
+            const uint8_t* blk = xrow(t) + (size_t)(k0 / 32 + (hb >> 1)) * kQ81xBytes;
+            const uint2* q = reinterpret_cast<const uint2*>(blk + 8 + (hb & 1u) * 16u);
+            q0 = q[0];
+            q1 = q[1];
+            ds = *reinterpret_cast<const float2*>(blk);
+        }
         qs[(size_t)t * (KT_alloc / 16) + hb] = make_uint4(q0.x, q0.y, q1.x, q1.y);
-        if ((hb & 1u) == 0) d8[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = d;
-        if (HAS_MIN) {
+        if (SUM_GRAN == 16) {
             int s = dot4(0x01010101u, q0.x, 0);
             s = dot4(0x01010101u, q0.y, s);
             s = dot4(0x01010101u, q1.x, s);
             s = dot4(0x01010101u, q1.y, s);
-            s16[(size_t)t * (KT_alloc / 16) + hb] = d * (float)s;
+            reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 16) + hb] = make_float2(ds.x, ds.x * (float)s);
+        } else if ((hb & 1u) == 0) {
+            if (SUM_GRAN == 32)
+                reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = ds;
+            else
+                reinterpret_cast<float*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = ds.x;
         }
     }
-    ActTile<HAS_MIN> a;
-    a.qs = qs;
-    a.d8 = d8;
-    a.s16 = s16;
-    a.KT = KT_alloc;
-    return a;
+    return ActTile{qs, hdr, KT_alloc};
 }
 
-// Accumulate one K-tile: units [u0, u0 + n_units) of rows `rows[r]` against the
-// staged activations.  `gl` = lane index inside its G-lane group.
-template <class F, int T, int R, int G>
-__device__ __forceinline__ void gemv_tile(const typename F::W& w, const uint32_t (&rows)[R], uint32_t u0, uint32_t n_units,
-                                          uint32_t gl, const ActTile<F::HAS_MIN>& act, float (&acc)[R][T]) {
-    for (uint32_t ul = gl; ul < n_units; ul += G) {
-        typename F::Raw raw[R];
+__device__ __forceinline__ int dot16(const uint32_t (&w)[4], const uint4& x, int c) {
+    c = dot4(w[0], x.x, c);
+    c = dot4(w[1], x.y, c);
+    c = dot4(w[2], x.z, c);
+    return dot4(w[3], x.w, c);
+}
+
+// One step of the unit walk: R decoded units (one per row, same tile-local unit
+// `ul`) against the T staged activation rows.
+template <class F, int T, int R>
+__device__ __forceinline__ void gemv_step(const typename F::Raw (&raw)[R], const typename F::Cursor (&cu)[R], uint32_t ul,
+                                          const ActTile& act, float (&acc)[R][T]) {
+    Unit un[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) raw[r] = F::load(w, rows[r], u0 + ul);
-        Unit un[R];
+    for (int r = 0; r < R; ++r) F::decode(raw[r], cu[r], un[r]);
+    const uint32_t e0 = F::elem_off(ul);
 #pragma unroll
-        for (int r = 0; r < R; ++r) F::decode(raw[r], u0 + ul, un[r]);
-        const uint32_t ea = F::elem_off(ul), eb = ea + F::EB_OFF;
+    for (int t = 0; t < T; ++t) {
+        uint4 x[4];
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const uint4 xa = act.qs[(size_t)t * (act.KT / 16) + (ea >> 4)];
-            const uint4 xb = act.qs[(size_t)t * (act.KT / 16) + (eb >> 4)];
-            const float da = act.d8[(size_t)t * (act.KT / 32) + (ea >> 5)];
-            const float db = act.d8[(size_t)t * (act.KT / 32) + (eb >> 5)];
-            float sa = 0.f, sb = 0.f;
-            if (F::HAS_MIN) {
-                sa = act.s16[(size_t)t * (act.KT / 16) + (ea >> 4)];
-                sb = act.s16[(size_t)t * (act.KT / 16) + (eb >> 4)];
+        for (int g = 0; g < 4; ++g) x[g] = act.qs[(size_t)t * (act.KT / 16) + ((e0 + g * F::GROUP_OFF) >> 4)];
+        if (F::PAIRED) {
+            // groups (0,1) and (2,3): one activation block and one weight scale each
+            float d0, d1, s0 = 0.f, s1 = 0.f;
+            if (F::SUM_GRAN == 32) {
+                const float2* h = reinterpret_cast<const float2*>(act.hdr) + (size_t)t * (act.KT / 32) + (e0 >> 5);
+                const float2 h0 = h[0], h1 = h[1];
+                d0 = h0.x; s0 = h0.y; d1 = h1.x; s1 = h1.y;
+            } else {
+                const float* h = reinterpret_cast<const float*>(act.hdr) + (size_t)t * (act.KT / 32) + (e0 >> 5);
+                d0 = h[0]; d1 = h[1];
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                int ia = dot4(un[r].a[0], xa.x, 0);
-                ia = dot4(un[r].a[1], xa.y, ia);
-                ia = dot4(un[r].a[2], xa.z, ia);
-                ia = dot4(un[r].a[3], xa.w, ia);
-                int ib = dot4(un[r].b[0], xb.x, 0);
-                ib = dot4(un[r].b[1], xb.y, ib);
-                ib = dot4(un[r].b[2], xb.z, ib);
-                ib = dot4(un[r].b[3], xb.w, ib);
-                float v = un[r].ca * (da * (float)ia) + un[r].cb * (db * (float)ib);
-                if (F::HAS_MIN) v -= un[r].ma * sa + un[r].mb * sb;
+                const int i0 = dot16(un[r].q[1], x[1], dot16(un[r].q[0], x[0], 0));
+                const int i1 = dot16(un[r].q[3], x[3], dot16(un[r].q[2], x[2], 0));
+                float v = un[r].c[0] * (d0 * (float)i0) + un[r].c[2] * (d1 * (float)i1);
+                if (F::SUM_GRAN == 32) v -= un[r].m[0] * s0 + un[r].m[2] * s1;
+                acc[r][t] += v;
+            }
+        } else {
+            float2 h[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                h[g] = reinterpret_cast<const float2*>(act.hdr)[(size_t)t * (act.KT / 16) + ((e0 + g * F::GROUP_OFF) >> 4)];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float v = 0.f;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int ig = dot16(un[r].q[g], x[g], 0);
+                    v += un[r].c[g] * (h[g].x * (float)ig) - un[r].m[g] * h[g].y;
+                }
                 acc[r][t] += v;
             }
         }
+    }
+}
+
+// Walk one K-tile for R rows: lane `gl` of a G-lane group handles tile-local
+// units gl, gl+G, ...  Full iterations (every lane live) run U at a time with
+// all U*R loads issued before the first use; the ragged rest is predicated.
+// cu[r] must point at unit (tile_first_unit + gl) of row r.  `n_units` counts
+// 64-element units including a trailing half unit (`half_tail`: K % 64 == 32).
+template <class F, int T, int R, int G, int U>
+__device__ __forceinline__ void gemv_rows(const typename F::Cursor (&cu)[R], uint32_t n_units, bool half_tail, uint32_t gl,
+                                          const ActTile& act, float (&acc)[R][T]) {
+    const uint32_t n_whole = half_tail ? n_units - 1 : n_units;
+    const uint32_t full = n_whole / G;
+    uint32_t it = 0;
+    for (; it + U <= full; it += U) {
+        typename F::Raw raw[U][R];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int r = 0; r < R; ++r) raw[u][r] = load_unit<F, G>(cu[r], it + u, false);
+#pragma unroll
+        for (int u = 0; u < U; ++u) gemv_step<F, T, R>(raw[u], cu, gl + (it + u) * G, act, acc);
+    }
+    for (; it * G + gl < n_units; ++it) {
+        typename F::Raw raw[R];
+        const bool half_only = half_tail && (it * G + gl == n_units - 1);
+#pragma unroll
+        for (int r = 0; r < R; ++r) raw[r] = load_unit<F, G>(cu[r], it, half_only);
+        gemv_step<F, T, R>(raw, cu, gl + it * G, act, acc);
     }
 }
 
