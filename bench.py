@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the quantized-matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu] [--no-detail]
+
+Workload (BASELINE.json configs[1]): decode GEMV at Llama-3-8B FFN shapes —
+gate and up 4096->14336, down 14336->4096 — with Q6_K and Q8_0 weights, int-dot
+on q8_1 activations, batch 1.  One step = those six GEMV launches over one set of
+weight matrices; consecutive steps rotate through several distinct weight sets
+(> 1 GB in total) so that neither L2 nor the 256 MB Infinity Cache can serve the
+weights.  Inputs (packed weights, quantized activations) are resident in HBM
+before the timed region.
+
+Prints ONE JSON line: the metric is achieved HBM GB/s on algorithmic bytes
+(weights once + q8 activations + fp16 outputs).  `roofline` prices the dominant
+kernel against the 8 TB/s HBM peak; `cpu_baseline` times the reference's CPU
+path (dequant to fp32 + scalar fp32 dot, restated in oracle/) on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+H, FF = 4096, 14336
+Q81X = 40
+
+
+def gemv_bytes(fmt_row_bytes, K, N, T):
+    """Algorithmic bytes of one GEMV launch: weights once, q8 activations, fp16 outputs."""
+    return N * fmt_row_bytes + T * (K // 32) * Q81X + T * N * 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-detail", action="store_true", help="skip the per-config detail table")
+    ap.add_argument("--sets", type=int, default=4, help="distinct weight sets rotated through (331.7 MB each)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build measures one GPU only (the path is data-parallel over output rows / experts; "
+                         "see DESIGN.md for how it shards); run with --gpus 1\n")
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        sys.exit(3)
+    import machx_inference_engine_amd as mx
+    from machx_inference_engine_amd import synth
+    ops = mx.ops
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    # ---------------------------------------------------------------- inputs, resident in HBM
+    fmts = ("q6_K", "q8_0")
+    shapes = {"gate": (H, FF), "up": (H, FF), "down": (FF, H)}   # (K, N)
+    sets = []
+    for s in range(args.sets):
+        ws = {}
+        for fi, fmt in enumerate(fmts):
+            for ni, (name, (K, N)) in enumerate(shapes.items()):
+                ws[(fmt, name)] = synth.random_weights(fmt, N, K, seed=1000 * s + 10 * fi + ni, device=dev)
+        sets.append(ws)
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    x = torch.randn((1, H), device=dev, generator=g).half()
+    h = torch.randn((1, FF), device=dev, generator=g).half()
+    xq, hq = ops.quantize_q8_1(x), ops.quantize_q8_1(h)
+    y_ff = {(f, n): torch.empty(FF, dtype=torch.float16, device=dev) for f in fmts for n in ("gate", "up")}
+    y_h = {f: torch.empty(H, dtype=torch.float16, device=dev) for f in fmts}
+    # Q8_0 runs through the reference's own entry point for this format, gemv_q8_0_soa_q8: the
+    # load-time split of block_q8_0 into an int8 plane and an fp16 scale plane (same bytes).
+    for ws in sets:
+        for n in shapes:
+            ws[("q8_0_soa", n)] = synth.split_q8_0(ws[("q8_0", n)])
+
+    def gemv(fmt, xq_, ws, name, K, N, y):
+        if fmt == "q6_K":
+            ops.gemv_q6_K_q8(xq_, ws[(fmt, name)], K, N, y)
+        else:
+            qs, d = ws[("q8_0_soa", name)]
+            ops.gemv_q8_0_soa_q8(xq_, qs, d, K, N, y)
+
+    def step(ws):
+        for fmt in fmts:
+            gemv(fmt, xq, ws, "gate", H, FF, y_ff[(fmt, "gate")])
+            gemv(fmt, xq, ws, "up", H, FF, y_ff[(fmt, "up")])
+            gemv(fmt, hq, ws, "down", FF, H, y_h[fmt])
+
+    bytes_per_step = sum(gemv_bytes(synth.row_bytes(f, K), K, N, 1) for f in fmts for (K, N) in shapes.values())
+
+    # ---------------------------------------------------------------- warm-up, graphs
+    for i in range(args.warmup):
+        step(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    graphs = None
+    if not args.no_graph:
+        graphs = []
+        for ws in sets:
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                step(ws)
+            graphs.append(gr)
+        for gr in graphs:
+            gr.replay()
+        torch.cuda.synchronize()
+
+    # ---------------------------------------------------------------- timed region: exactly K steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        if graphs:
+            graphs[i % len(graphs)].replay()
+        else:
+            step(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = bytes_per_step * args.steps / elapsed / 1e9
+
+    # ---------------------------------------------------------------- roofline of the dominant kernel (HIP events)
+    # Dominant by time and bytes: the Q8_0 gate/up GEMV (K=4096, N=14336), 62,390,272 weight bytes per launch.
+    def kernel_avg_us(fn, n_launch):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn(0)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for i in range(n_launch):
+                fn(i)
+        gr.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (5 * n_launch) * 1e3
+
+    mats = [ws[("q8_0_soa", n)] for ws in sets for n in ("gate", "up")]
+    dom_us = kernel_avg_us(lambda i: ops.gemv_q8_0_soa_q8(xq, mats[i % len(mats)][0], mats[i % len(mats)][1], H, FF, y_ff[("q8_0", "gate")]),
+                           4 * len(mats))
+    dom_bytes = gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1)
+    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": "gemv_q8_kernel<FmtQ8Soa,T=1> K=4096 N=14336", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 3)}
+
+    out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
+           "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8 dot, fp32 fold", "data": "synthetic",
+           "config": {"workload": "configs[1]: decode GEMV gate/up 4096->14336 + down 14336->4096, Q6_K and Q8_0, T=1, "
+                                  "6 launches/step, %d rotating weight sets" % len(sets),
+                      "bytes_per_step": bytes_per_step, "hip_graph": bool(graphs), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+           "roofline": roofline}
+
+    # ---------------------------------------------------------------- detail: the other batch sizes and formats
+    if not args.no_detail:
+        detail = {}
+        def soa_batched(xsq_, w, K, N, T, yt_):
+            return ops.gemv_q8_0_soa_q8_batched(xsq_, w[0], w[1], K, N, T, yt_)
+
+        for fmt, fn in (("q6_K", ops.gemv_q6_K_q8_batched), ("q8_0_soa", soa_batched), ("q8_0", ops.gemv_q8_0_q8_batched),
+                        ("q4_K", ops.gemv_q4_K_q8_batched)):
+            for name, (K, N) in (("gate_up", (H, FF)), ("down", (FF, H))):
+                if fmt == "q4_K":
+                    ws_l = [synth.random_weights(fmt, N, K, seed=77 + i, device=dev) for i in range(12)]
+                else:
+                    ws_l = [ws[(fmt, "gate" if name == "gate_up" else "down")] for ws in sets] + \
+                           ([ws[(fmt, "up")] for ws in sets] if name == "gate_up" else [])
+                for T in (1, 2, 4, 8):
+                    xs = torch.randn((T, K), device=dev, generator=g).half()
+                    xsq = ops.quantize_q8_1(xs)
+                    yt = torch.empty((T, N), dtype=torch.float16, device=dev)
+                    us = kernel_avg_us(lambda i: fn(xsq, ws_l[i % len(ws_l)], K, N, T, yt), 3 * len(ws_l))
+                    b = gemv_bytes(synth.row_bytes(fmt.replace("_soa", ""), K), K, N, T)
+                    detail["%s_%s_T%d" % (fmt, name, T)] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1),
+                                                            "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+                del ws_l
+        # BASELINE config 1: Q4_K 4096x4096, fp32 activations, fp32 out (9.4 MB: cache resident unless rotated)
+        w1 = [synth.random_weights("q4_K", 4096, 4096, seed=500 + i, device=dev) for i in range(40)]
+        a32 = torch.randn(4096, device=dev, generator=g)
+        y32 = torch.empty(4096, dtype=torch.float32, device=dev)
+        us = kernel_avg_us(lambda i: ops.gemv_q4_K(a32, w1[i % len(w1)], 4096, 4096, y32), 2 * len(w1))
+        b = 4096 * synth.row_bytes("q4_K", 4096) + 2 * 4096 * 4
+        detail["config1_q4_K_4096x4096_f32"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+        aq = ops.quantize_q8_1(a32)
+        y16 = torch.empty(4096, dtype=torch.float16, device=dev)
+        us = kernel_avg_us(lambda i: ops.gemv_q4_K_q8(aq, w1[i % len(w1)], 4096, 4096, y16), 2 * len(w1))
+        detail["config1_q4_K_4096x4096_q8"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+        out["detail"] = detail
+
+    # ---------------------------------------------------------------- CPU baseline (reported only)
+    if not args.no_cpu:
+        import numpy as np
+        import oracle as O   # the checker, used here only as the timed CPU baseline
+        # Sample: the down projection of both formats plus gate (one step's shapes), T=1, one thread,
+        # exactly the reference's loop: dequant row to fp32, sequential fp32 dot.
+        xh = x.float().cpu().numpy()
+        hh = h.float().cpu().numpy()
+        work = [("q6_K", O.Q6_K, sets[0][("q6_K", "gate")], xh, H, FF), ("q6_K", O.Q6_K, sets[0][("q6_K", "down")], hh, FF, H),
+                ("q8_0", O.Q8_0, sets[0][("q8_0", "gate")], xh, H, FF), ("q8_0", O.Q8_0, sets[0][("q8_0", "down")], hh, FF, H)]
+        host = [(f, w.cpu().numpy(), a, K, N) for (_, f, w, a, K, N) in work]
+        os.environ["OMP_NUM_THREADS"] = "1"
+        tot_b, t_cpu, reps = 0, 0.0, 0
+        try:
+            import ctypes
+            omp = ctypes.CDLL("libgomp.so.1")
+            omp.omp_set_num_threads(1)
+        except OSError:
+            omp = None
+        while t_cpu < 10.0 and reps < 50:
+            for f, w, a, K, N in host:
+                c0 = time.perf_counter()
+                O.gemv_f32chain(f, w, a, K, N)
+                t_cpu += time.perf_counter() - c0
+                tot_b += w.nbytes
+            reps += 1
+        out["cpu_baseline"] = {"value": round(tot_b / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "gate (4096->14336) and down (14336->4096) GEMV in Q6_K and Q8_0, T=1, %d repetitions, "
+                                         "weight bytes / time; dequant-to-fp32 + sequential fp32 dot as in the reference's "
+                                         "tests/unit/gemv_q4k_test.cpp" % reps}
+        if omp is not None:
+            n_thr = min(16, os.cpu_count() or 1)
+            omp.omp_set_num_threads(n_thr)
+            c0 = time.perf_counter()
+            nb = 0
+            for _ in range(3):
+                for f, w, a, K, N in host:
+                    O.gemv_f32chain(f, w, a, K, N)
+                    nb += w.nbytes
+            out["cpu_baseline_mt"] = {"value": round(nb / (time.perf_counter() - c0) / 1e9, 3), "unit": "GB/s", "cores": n_thr,
+                                      "kind": "port", "sample": "same work, rows split over OpenMP threads"}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
