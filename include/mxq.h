@@ -136,6 +136,70 @@ int mx_gemv_q4_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uin
 int mx_gemv_q6_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 
+/* ---------------------------------------------------------------- MoE, expert-indexed GEMV
+ * Q8_0-expert decode kernels (device-resident routing: the expert of token slot
+ * tk = t*K + k is read from topk_idx[tk]; no host round trip):
+ *   moe_gate_up_silu_q8  include/ie/moe_q8.hpp:17-23, src/ops/moe_q8.cpp:45-100
+ *     h_out[tk, n] = half(silu(gate_e . x_t) * (up_e . x_t)); x_q8 = T rows of H/32 blocks
+ *   moe_down_q8          include/ie/moe_q8.hpp:25-31, src/ops/moe_q8.cpp:102-147
+ *     y_packed[tk, n] = half(topk_w[tk] * (down_e . h_tk)); h_q8 = T*K rows of E_ffn/32 blocks
+ *   moe_reduce_q8        include/ie/moe_q8.hpp:33-35, src/ops/moe_q8.cpp:149-158
+ * Expert e of a SoA bank: qs + e*qs_stride (bytes), d + e*d_stride (fp16 entries).  */
+int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
+                           const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx,
+                           uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H, uint32_t E_ffn);
+int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                   uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
+                   uint32_t K, uint32_t E_ffn, uint32_t H);
+int mx_moe_reduce_q8(mx_stream_t s, const uint16_t* y_packed, uint16_t* y, uint32_t T, uint32_t K, uint32_t H);
+/* Expert-grouped form: activation rows are expert-sorted and partitioned by
+ * expert_offsets[E+1]; each expert's weights are streamed once per tile of rows;
+ * experts without rows cost nothing (src/ops/moe_q8.cpp:211).
+ *   moe_prefill_gate_up_silu_q8  include/ie/moe_q8.hpp:51-58, src/ops/moe_q8.cpp:185-275
+ *   moe_prefill_down_q8          include/ie/moe_q8.hpp:65-72, src/ops/moe_q8.cpp:277-366
+ *     out_packed[row, n] = half(sorted_w[row] * acc)
+ *   moe_prefill_reduce_sum       include/ie/moe_q8.hpp:77-80, src/ops/moe_q8.cpp:368-384
+ *   moe_prefill_reduce           include/ie/ops.hpp:1008-1017, src/ops/moe_fused.cpp:1927-1954
+ *     y[t] += sum_k w[row] * out_packed[row], row = tk_to_packed[t*K+k]  (accumulates: caller zeroes y)
+ *   moe_gather_rows              src/ops/moe.cpp:262-282  */
+int mx_moe_prefill_gate_up_silu_q8(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d,
+                                   const int8_t* u_qs, const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride,
+                                   const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn);
+int mx_moe_prefill_down_q8(mx_stream_t s, const void* hq8_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                           uint64_t d_stride, const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed,
+                           uint32_t E, uint32_t H, uint32_t E_ffn);
+int mx_moe_prefill_reduce_sum(mx_stream_t s, const uint16_t* out_packed, const uint32_t* tk_to_packed, uint16_t* y, uint32_t T,
+                              uint32_t K, uint32_t H);
+int mx_moe_prefill_reduce(mx_stream_t s, const uint16_t* out_packed, const uint32_t* tk_to_packed, const uint16_t* weights_packed,
+                          uint16_t* y, uint32_t T, uint32_t K_top, uint32_t H);
+int mx_moe_gather_rows(mx_stream_t s, const uint16_t* x, const int32_t* indices, uint16_t* y_packed, uint32_t n_rows,
+                       uint32_t hidden);
+/* MXFP4-expert (gpt-oss) kernels.  The reference runs this layer as a host loop
+ * over experts of gemv_mxfp4_soa_q8 / add_bias / swiglu_oai launches
+ * (src/model/gptoss.cpp:366-420); these entry points are that loop moved onto the
+ * device, with the same rounding points: h = half(swiglu_oai(half(gate.x + bg),
+ * half(up.x + bu))), out = half(half(down.h) + bd).  Biases fp32 [E][N], may be NULL.
+ * Decode form reads topk_idx; grouped form takes expert-sorted rows +
+ * expert_offsets (total_rows = expert_offsets[E], known to the host from the packing).  */
+int mx_moe_gate_up_oai_mxfp4(mx_stream_t s, const void* x_q8, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs,
+                             const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride, const float* gate_bias,
+                             const float* up_bias, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
+                             uint32_t E_ffn, uint32_t n_experts, float alpha, float limit);
+int mx_moe_down_mxfp4(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
+                      uint64_t e_stride, const float* down_bias, const int32_t* topk_idx, uint16_t* out_packed, uint32_t T,
+                      uint32_t K, uint32_t E_ffn, uint32_t H, uint32_t n_experts);
+int mx_moe_grouped_gate_up_oai_mxfp4(mx_stream_t s, const void* xq8_packed, const uint8_t* g_qs, const uint8_t* g_e,
+                                     const uint8_t* u_qs, const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride,
+                                     const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets,
+                                     uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha,
+                                     float limit);
+int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
+                              uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed,
+                              uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+/* build_moe_packing  src/model/qwen3moe_pack.cpp:5-31 (host pointers): stable counting sort by expert.  */
+int mx_build_moe_packing(const int32_t* topk_ids, const float* topk_w, uint32_t T, uint32_t K, uint32_t E,
+                         uint32_t* expert_offsets, int32_t* sorted_idx, float* weights_packed, int32_t* tk_to_packed);
+
 /* ---------------------------------------------------------------- host repackers (host pointers)
  * MXFP4 AoS -> SoA planes  src/model/gptoss.cpp:180-208
  * Q8_0  AoS -> SoA planes  src/model/qwen35moe_split.cpp:134-144  */

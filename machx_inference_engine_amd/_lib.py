@@ -36,7 +36,7 @@ def parse_header(path=HEADER):
 
 def load():
     if not os.path.exists(LIB_PATH):
-        raise ImportError("libmxq.so is not built (%s): run `python -m machx_inference_engine_amd.build`; "
+        raise ImportError("libmxq.so is not built (%s): run `python machx_inference_engine_amd/build.py`; "
                           "there is no CPU fallback for this path" % LIB_PATH)
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in parse_header().items():

@@ -1,6 +1,6 @@
 """Build recipe for libmxq.so (hipcc, gfx950 only).
 
-    python -m machx_inference_engine_amd.build [--force]
+    python machx_inference_engine_amd/build.py [--force]
 
 Each translation unit under csrc/ is compiled to an object in csrc/build/ and the
 objects are linked into machx_inference_engine_amd/libmxq.so.  The library is

@@ -1,0 +1,420 @@
+// moe.hip — expert-indexed GEMV kernels (MoE decode and small-batch grouped
+// decode) and the row utilities around them.
+//
+// One kernel serves both addressing modes of the reference:
+//   * decode   — blockIdx.y = token slot tk = t*K_top + k; the expert id is read
+//                from the device array topk_idx[tk] (include/ie/moe_q8.hpp:17-33,
+//                src/ops/moe_q8.cpp:45-147): no host round trip, no per-expert
+//                host loop;
+//   * grouped  — blockIdx.y = expert e; its activation rows are the expert-sorted
+//                rows [expert_offsets[e], expert_offsets[e+1]) (moe_q8.hpp:51-72);
+//                the expert's weights are streamed once per tile of up to TT rows,
+//                empty experts return at once (src/ops/moe_q8.cpp:211).
+// The inner loop is the dense GEMV core (mxq_gemv_core.h).  gate and up rows are
+// walked together against one staged activation and fused with the activation
+// function in the epilogue.
+#include "mxq_gemv_core.h"
+#include "mxq_host.h"
+
+namespace mxq {
+
+enum { EPI_SILU = 0, EPI_OAI = 1, EPI_DOWN_WEIGHTED = 2, EPI_DOWN_BIAS = 3 };
+
+struct MoeArgs {
+    const uint8_t* xq8;              // block_q8_1x rows
+    const int32_t* topk_idx;         // decode mode: [n_seg] expert per slot; NULL in grouped mode
+    const uint32_t* expert_offsets;  // grouped mode: [E+1]
+    const float* bias0;              // [E][N] fp32 or NULL (gate bias / down bias)
+    const float* bias1;              // [E][N] fp32 or NULL (up bias)
+    const half_t* route_w;           // [rows] fp16 routing weight per output row (EPI_DOWN_WEIGHTED)
+    half_t* out;                     // [rows][N]
+    float alpha, limit;              // swiglu_oai parameters
+    uint32_t act_div;                // activation row of output row r is r / act_div
+    uint32_t K, N, KT, n_experts;
+};
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
+// src/ops/elementwise.cpp:468-492: x = min(gate, limit), z = clamp(up, -limit, limit), (x * sigmoid(alpha x)) * (z + 1)
+__device__ __forceinline__ float swiglu_oai(float g, float u, float alpha, float limit) {
+    const float x = fminf(g, limit), z = fmaxf(fminf(u, limit), -limit);
+    return (x / (1.f + __expf(alpha * -x))) * (z + 1.f);
+}
+
+// NW = weight rows per output element (2: gate and up, 1: down); R outputs per lane group.
+template <class F, int TT, int NW, int R, int G, int U, int EPI>
+__global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank bank0, typename F::Bank bank1, MoeArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
+    const uint32_t seg = blockIdx.y;
+    uint32_t e, r_begin, r_end;
+    if (a.topk_idx) {
+        e = (uint32_t)a.topk_idx[seg];
+        r_begin = seg;
+        r_end = seg + 1;
+    } else {
+        e = seg;
+        r_begin = a.expert_offsets[seg];
+        r_end = a.expert_offsets[seg + 1];
+    }
+    if (r_begin >= r_end || e >= a.n_experts) return;   // empty expert / invalid id: uniform for the block
+    const typename F::W w0 = F::expert(bank0, e), w1 = F::expert(NW == 2 ? bank1 : bank0, e);
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    const uint32_t K = a.K, N = a.N, KT = a.KT;
+    const size_t q8_row_bytes = (size_t)(K / 32) * kQ81xBytes;
+    const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    const uint32_t n_tiles = (K + KT - 1) / KT;
+    for (uint32_t t0 = r_begin; t0 < r_end; t0 += TT) {
+        const uint32_t nt = (r_end - t0 < (uint32_t)TT) ? r_end - t0 : (uint32_t)TT;
+        auto xrow = [&](uint32_t t) { return a.xq8 + (size_t)((t0 + (t < nt ? t : nt - 1)) / a.act_div) * q8_row_bytes; };
+        ActTile act;
+        bool staged = false;
+        for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
+            const uint32_t n0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
+            float acc[NW * R][TT];
+#pragma unroll
+            for (int r = 0; r < NW * R; ++r)
+#pragma unroll
+                for (int t = 0; t < TT; ++t) acc[r][t] = 0.f;
+            for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+                const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
+                typename F::Cursor cu[NW * R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const uint32_t n = (n0 + r < N) ? n0 + r : N - 1;
+                    cu[NW * r] = F::cursor(w0, n, k0 / 64 + gl);
+                    if (NW == 2) cu[NW * r + 1] = F::cursor(w1, n, k0 / 64 + gl);
+                }
+                if (n_tiles > 1 || !staged) {
+                    __syncthreads();
+                    act = stage_act<F::SUM_GRAN, TT>(lds, xrow, k0, kt, KT);
+                    __syncthreads();
+                    staged = true;
+                }
+                gemv_rows<F, TT, NW * R, G, U>(cu, (kt + 63) / 64, (kt & 63u) != 0, gl, act, acc);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    const float v0 = group_sum<G>(acc[NW * r][t]);
+                    const float v1 = (NW == 2) ? group_sum<G>(acc[NW * r + 1][t]) : 0.f;
+                    const uint32_t n = n0 + r;
+                    if (lane == (uint32_t)group_sum_lane<G>(lane) && n < N && (uint32_t)t < nt) {
+                        const uint32_t row = t0 + t;
+                        float o;
+                        if (EPI == EPI_SILU) {
+                            o = silu_mul(v0, v1);                                   // src/ops/moe_q8.cpp:94-97
+                        } else if (EPI == EPI_OAI) {
+                            // rounding points of the reference chain: half(acc + bias) per projection, then the fp16 activation
+                            const float g = (float)(half_t)(v0 + (a.bias0 ? a.bias0[(size_t)e * N + n] : 0.f));
+                            const float u = (float)(half_t)(v1 + (a.bias1 ? a.bias1[(size_t)e * N + n] : 0.f));
+                            o = swiglu_oai(g, u, a.alpha, a.limit);
+                        } else if (EPI == EPI_DOWN_WEIGHTED) {
+                            o = (float)a.route_w[row] * v0;                        // src/ops/moe_q8.cpp:143-144
+                        } else {
+                            o = (float)(half_t)v0;                                 // gemv out, then add_bias (elementwise.cpp:782-793)
+                            if (a.bias0) o += a.bias0[(size_t)e * N + n];
+                        }
+                        a.out[(size_t)row * N + n] = (half_t)o;
+                    }
+                }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- row utilities
+// moe_gather_rows (src/ops/moe.cpp:262-282): y_packed[i] = x[indices[i]]
+__global__ __launch_bounds__(256) void gather_rows_kernel(const half_t* x, const int32_t* idx, half_t* y, uint32_t n_rows, uint32_t hidden) {
+    const uint32_t row = blockIdx.y;
+    const uint32_t c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (row >= n_rows || c >= hidden) return;
+    const half_t* src = x + (size_t)idx[row] * hidden + c;
+    half_t* dst = y + (size_t)row * hidden + c;
+    if (c + 8 <= hidden && (hidden & 7u) == 0) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+    } else {
+        for (uint32_t i = 0; i < 8 && c + i < hidden; ++i) dst[i] = src[i];
+    }
+}
+
+// moe_reduce_q8 (src/ops/moe_q8.cpp:149-158): y[t] = sum_k y_packed[t*K+k]
+// moe_prefill_reduce_sum (:368-384): y[t] = sum_k out_packed[tk_to_packed[t*K+k]]
+// moe_prefill_reduce (src/ops/moe_fused.cpp:1927-1954): y[t] += sum_k w[row] * out_packed[row]
+template <bool WEIGHTED, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void moe_reduce_kernel(const half_t* packed, const uint32_t* tk_to_packed, const half_t* w, half_t* y,
+                                                         uint32_t T, uint32_t Ktop, uint32_t H) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (uint64_t)T * H) return;
+    const uint32_t t = (uint32_t)(i / H), n = (uint32_t)(i % H);
+    float s = ACCUMULATE ? (float)y[i] : 0.f;
+    for (uint32_t k = 0; k < Ktop; ++k) {
+        const uint32_t row = tk_to_packed ? tk_to_packed[(size_t)t * Ktop + k] : t * Ktop + k;
+        const float v = (float)packed[(size_t)row * H + n];
+        s += WEIGHTED ? (float)w[row] * v : v;
+    }
+    y[i] = (half_t)s;
+}
+
+// ---------------------------------------------------------------- host side
+static int cu_count_moe() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    }
+    return n;
+}
+constexpr uint32_t kMoeLdsBudget = 48 * 1024;
+
+static uint32_t pick_group_moe(uint32_t units) {
+    uint32_t best = 64, waste = (units + 63) / 64 * 64 - units;
+    for (uint32_t g : {32u, 16u}) {
+        const uint32_t w = (units + g - 1) / g * g - units;
+        if (w < waste) { best = g; waste = w; }
+    }
+    return best;
+}
+
+template <class F, int TT, int NW, int G, int EPI>
+static int launch_moe_tg(hipStream_t st, const typename F::Bank& b0, const typename F::Bank& b1, MoeArgs a, uint32_t n_seg) {
+    constexpr int R = (NW == 2) ? 1 : 2;
+    constexpr int U = (TT == 1) ? 2 : 1;
+    constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
+    const uint32_t per32 = 32 + hdr_bytes_per32(F::SUM_GRAN);
+    const uint32_t KT_max = (kMoeLdsBudget / (per32 * TT)) * 32 / 256 * 256;
+    if (KT_max == 0) return MX_ERR_SHAPE;
+    const uint32_t K256 = (a.K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
+    a.KT = (K256 + n_tiles - 1) / n_tiles * 256;
+    const uint32_t n_rg = (a.N + rows_per_wg - 1) / rows_per_wg;
+    uint32_t gx = (uint32_t)cu_count_moe() * 8 / (n_seg ? n_seg : 1);
+    if (gx < 1) gx = 1;
+    if (gx > n_rg) gx = n_rg;
+    if (n_seg > 65535) return MX_ERR_SHAPE;
+    hipLaunchKernelGGL((moe_gemv_kernel<F, TT, NW, R, G, U, EPI>), dim3(gx, n_seg), dim3(kGemvThreads), act_tile_bytes(TT, a.KT, F::SUM_GRAN), st,
+                       b0, b1, a);
+    return launch_status();
+}
+
+template <class F, int NW, int EPI>
+static int launch_moe(mx_stream_t s, const typename F::Bank& b0, const typename F::Bank& b1, const MoeArgs& a, uint32_t n_seg, uint32_t tt) {
+    const uint32_t G = pick_group_moe((a.K + 63) / 64);
+    hipStream_t st = as_stream(s);
+#define MX_MOE_G(TT)                                                                     \
+    (G == 16 ? launch_moe_tg<F, TT, NW, 16, EPI>(st, b0, b1, a, n_seg)                   \
+             : G == 32 ? launch_moe_tg<F, TT, NW, 32, EPI>(st, b0, b1, a, n_seg)         \
+                       : launch_moe_tg<F, TT, NW, 64, EPI>(st, b0, b1, a, n_seg))
+    if (tt == 1) return MX_MOE_G(1);
+    if (tt <= 4) return MX_MOE_G(4);
+    return MX_MOE_G(8);
+#undef MX_MOE_G
+}
+
+// rows per token tile in grouped mode: expected rows per expert, rounded up to 4 or 8
+static uint32_t grouped_tt(uint64_t total_rows, uint32_t E) { return (total_rows <= 4ull * E) ? 4 : 8; }
+
+static int check_moe(const void* x, const void* out, uint32_t K, uint32_t N, uint32_t n_seg) {
+    MX_REQUIRE_PTR(x);
+    MX_REQUIRE_PTR(out);
+    MX_REQUIRE_SHAPE(K > 0 && N > 0 && K % 32 == 0 && n_seg > 0);
+    MX_REQUIRE_ALIGN(x, 8);
+    return MX_OK;
+}
+
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+// ------------------------------------------------------------ Q8_0 SoA experts, decode
+int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d,
+                           uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
+                           uint32_t E_ffn) {
+    const uint32_t n_experts = 0xFFFFFFFFu;   // the reference signature carries no expert count: ids are trusted
+    if (int rc = check_moe(x_q8, h_out, H, E_ffn, T * K)) return rc;
+    MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d); MX_REQUIRE_PTR(topk_idx);
+    MX_REQUIRE_SHAPE(K > 0 && n_experts > 0 && qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(g_qs, 16); MX_REQUIRE_ALIGN(u_qs, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(x_q8); a.topk_idx = topk_idx; a.out = reinterpret_cast<half_t*>(h_out);
+    a.act_div = K; a.K = H; a.N = E_ffn; a.n_experts = n_experts;
+    FmtQ8Soa::Bank bg{g_qs, g_d, qs_stride, d_stride, H}, bu{u_qs, u_d, qs_stride, d_stride, H};
+    return launch_moe<FmtQ8Soa, 2, EPI_SILU>(s, bg, bu, a, T * K, 1);
+}
+int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                   const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
+    const uint32_t n_experts = 0xFFFFFFFFu;
+    if (int rc = check_moe(h_q8, y_packed, E_ffn, H, T * K)) return rc;
+    MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(topk_w);
+    MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(d_qs, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(h_q8); a.topk_idx = topk_idx; a.route_w = reinterpret_cast<const half_t*>(topk_w);
+    a.out = reinterpret_cast<half_t*>(y_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
+    FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
+    return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, T * K, 1);
+}
+// ------------------------------------------------------------ Q8_0 SoA experts, grouped rows, int-dot GEMV form
+static int moe_grouped_gate_up_silu_q8_gemv(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
+                                   const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const uint32_t* expert_offsets,
+                                   uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    if (int rc = check_moe(xq8_packed, h_packed, H, E_ffn, E)) return rc;
+    MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(g_qs, 16); MX_REQUIRE_ALIGN(u_qs, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(xq8_packed); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(h_packed);
+    a.act_div = 1; a.K = H; a.N = E_ffn; a.n_experts = E;
+    FmtQ8Soa::Bank bg{g_qs, g_d, qs_stride, d_stride, H}, bu{u_qs, u_d, qs_stride, d_stride, H};
+    return launch_moe<FmtQ8Soa, 2, EPI_SILU>(s, bg, bu, a, E, grouped_tt(total_rows, E));
+}
+static int moe_grouped_down_q8_gemv(mx_stream_t s, const void* hq8_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                           uint64_t d_stride, const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E,
+                           uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    if (int rc = check_moe(hq8_packed, out_packed, E_ffn, H, E)) return rc;
+    MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(expert_offsets); MX_REQUIRE_PTR(sorted_w);
+    MX_REQUIRE_SHAPE(qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(d_qs, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(hq8_packed); a.expert_offsets = expert_offsets; a.route_w = reinterpret_cast<const half_t*>(sorted_w);
+    a.out = reinterpret_cast<half_t*>(out_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = E;
+    FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
+    return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, E, grouped_tt(total_rows, E));
+}
+
+int mx_moe_prefill_gate_up_silu_q8(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
+                                   const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const uint32_t* expert_offsets,
+                                   uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn) {
+    return moe_grouped_gate_up_silu_q8_gemv(s, xq8_packed, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, h_packed, E, H, E_ffn,
+                                            0xFFFFFFFFu);
+}
+int mx_moe_prefill_down_q8(mx_stream_t s, const void* hq8_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                           const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H,
+                           uint32_t E_ffn) {
+    return moe_grouped_down_q8_gemv(s, hq8_packed, d_qs, d_d, qs_stride, d_stride, expert_offsets, sorted_w, out_packed, E, H, E_ffn, 0xFFFFFFFFu);
+}
+
+// ------------------------------------------------------------ MXFP4 SoA experts (gpt-oss)
+static int moe_mxfp4_gate_up(mx_stream_t s, const void* x_q8, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
+                             uint64_t qs_stride, uint64_t e_stride, const float* gate_bias, const float* up_bias, const int32_t* topk_idx,
+                             const uint32_t* expert_offsets, uint16_t* h_out, uint32_t n_seg, uint32_t act_div, uint32_t H, uint32_t E_ffn,
+                             uint32_t n_experts, float alpha, float limit, uint32_t tt) {
+    if (int rc = check_moe(x_q8, h_out, H, E_ffn, n_seg)) return rc;
+    MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_e); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_e);
+    MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(g_qs, 16); MX_REQUIRE_ALIGN(u_qs, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(x_q8); a.topk_idx = topk_idx; a.expert_offsets = expert_offsets; a.bias0 = gate_bias; a.bias1 = up_bias;
+    a.out = reinterpret_cast<half_t*>(h_out); a.alpha = alpha; a.limit = limit; a.act_div = act_div; a.K = H; a.N = E_ffn; a.n_experts = n_experts;
+    FmtMxfp4Soa::Bank bg{g_qs, g_e, qs_stride, e_stride, H}, bu{u_qs, u_e, qs_stride, e_stride, H};
+    return launch_moe<FmtMxfp4Soa, 2, EPI_OAI>(s, bg, bu, a, n_seg, tt);
+}
+int mx_moe_gate_up_oai_mxfp4(mx_stream_t s, const void* x_q8, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
+                             uint64_t qs_stride, uint64_t e_stride, const float* gate_bias, const float* up_bias, const int32_t* topk_idx,
+                             uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H, uint32_t E_ffn, uint32_t n_experts, float alpha, float limit) {
+    MX_REQUIRE_PTR(topk_idx);
+    MX_REQUIRE_SHAPE(K > 0);
+    return moe_mxfp4_gate_up(s, x_q8, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, topk_idx, nullptr, h_out, T * K, K, H, E_ffn,
+                             n_experts, alpha, limit, 1);
+}
+int mx_moe_grouped_gate_up_oai_mxfp4(mx_stream_t s, const void* xq8_packed, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs,
+                                     const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride, const float* gate_bias, const float* up_bias,
+                                     const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                                     uint32_t total_rows, float alpha, float limit) {
+    MX_REQUIRE_PTR(expert_offsets);
+    return moe_mxfp4_gate_up(s, xq8_packed, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, nullptr, expert_offsets, h_packed, E, 1,
+                             H, E_ffn, E, alpha, limit, grouped_tt(total_rows, E));
+}
+static int moe_mxfp4_down(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
+                          const float* down_bias, const int32_t* topk_idx, const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t n_seg,
+                          uint32_t E_ffn, uint32_t H, uint32_t n_experts, uint32_t tt) {
+    if (int rc = check_moe(h_q8, out_packed, E_ffn, H, n_seg)) return rc;
+    MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_e);
+    MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(d_qs, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(h_q8); a.topk_idx = topk_idx; a.expert_offsets = expert_offsets; a.bias0 = down_bias;
+    a.out = reinterpret_cast<half_t*>(out_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
+    FmtMxfp4Soa::Bank b{d_qs, d_e, qs_stride, e_stride, E_ffn};
+    return launch_moe<FmtMxfp4Soa, 1, EPI_DOWN_BIAS>(s, b, b, a, n_seg, tt);
+}
+int mx_moe_down_mxfp4(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
+                      const float* down_bias, const int32_t* topk_idx, uint16_t* out_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H,
+                      uint32_t n_experts) {
+    MX_REQUIRE_PTR(topk_idx);
+    return moe_mxfp4_down(s, h_q8, d_qs, d_e, qs_stride, e_stride, down_bias, topk_idx, nullptr, out_packed, T * K, E_ffn, H, n_experts, 1);
+}
+int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
+                              uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E,
+                              uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    MX_REQUIRE_PTR(expert_offsets);
+    return moe_mxfp4_down(s, hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
+                          grouped_tt(total_rows, E));
+}
+
+// ------------------------------------------------------------ row utilities
+int mx_moe_gather_rows(mx_stream_t s, const uint16_t* x, const int32_t* indices, uint16_t* y_packed, uint32_t n_rows, uint32_t hidden) {
+    MX_REQUIRE_PTR(x); MX_REQUIRE_PTR(indices); MX_REQUIRE_PTR(y_packed);
+    MX_REQUIRE_SHAPE(n_rows > 0 && hidden > 0 && n_rows <= 65535);
+    MX_REQUIRE_ALIGN(x, 16); MX_REQUIRE_ALIGN(y_packed, 16);
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((hidden + 2047) / 2048, n_rows), dim3(256), 0, as_stream(s), reinterpret_cast<const half_t*>(x),
+                       indices, reinterpret_cast<half_t*>(y_packed), n_rows, hidden);
+    return launch_status();
+}
+static int reduce_common(const void* packed, const void* y, uint32_t T, uint32_t K, uint32_t H) {
+    MX_REQUIRE_PTR(packed); MX_REQUIRE_PTR(y);
+    MX_REQUIRE_SHAPE(T > 0 && K > 0 && H > 0);
+    return MX_OK;
+}
+int mx_moe_reduce_q8(mx_stream_t s, const uint16_t* y_packed, uint16_t* y, uint32_t T, uint32_t K, uint32_t H) {
+    if (int rc = reduce_common(y_packed, y, T, K, H)) return rc;
+    hipLaunchKernelGGL((moe_reduce_kernel<false, false>), dim3((uint32_t)(((uint64_t)T * H + 255) / 256)), dim3(256), 0, as_stream(s),
+                       reinterpret_cast<const half_t*>(y_packed), nullptr, nullptr, reinterpret_cast<half_t*>(y), T, K, H);
+    return launch_status();
+}
+int mx_moe_prefill_reduce_sum(mx_stream_t s, const uint16_t* out_packed, const uint32_t* tk_to_packed, uint16_t* y, uint32_t T, uint32_t K,
+                              uint32_t H) {
+    if (int rc = reduce_common(out_packed, y, T, K, H)) return rc;
+    MX_REQUIRE_PTR(tk_to_packed);
+    hipLaunchKernelGGL((moe_reduce_kernel<false, false>), dim3((uint32_t)(((uint64_t)T * H + 255) / 256)), dim3(256), 0, as_stream(s),
+                       reinterpret_cast<const half_t*>(out_packed), tk_to_packed, nullptr, reinterpret_cast<half_t*>(y), T, K, H);
+    return launch_status();
+}
+int mx_moe_prefill_reduce(mx_stream_t s, const uint16_t* out_packed, const uint32_t* tk_to_packed, const uint16_t* weights_packed, uint16_t* y,
+                          uint32_t T, uint32_t K_top, uint32_t H) {
+    if (int rc = reduce_common(out_packed, y, T, K_top, H)) return rc;
+    MX_REQUIRE_PTR(tk_to_packed); MX_REQUIRE_PTR(weights_packed);
+    hipLaunchKernelGGL((moe_reduce_kernel<true, true>), dim3((uint32_t)(((uint64_t)T * H + 255) / 256)), dim3(256), 0, as_stream(s),
+                       reinterpret_cast<const half_t*>(out_packed), tk_to_packed, reinterpret_cast<const half_t*>(weights_packed),
+                       reinterpret_cast<half_t*>(y), T, K_top, H);
+    return launch_status();
+}
+
+// build_moe_packing (src/model/qwen3moe_pack.cpp:5-31), host pointers: stable counting sort of the
+// T*K (token, slot) pairs by expert id.
+int mx_build_moe_packing(const int32_t* topk_ids, const float* topk_w, uint32_t T, uint32_t K, uint32_t E, uint32_t* expert_offsets,
+                         int32_t* sorted_idx, float* weights_packed, int32_t* tk_to_packed) {
+    if (!topk_ids || !topk_w || !expert_offsets || !sorted_idx || !weights_packed || !tk_to_packed) return MX_ERR_NULL;
+    if (!T || !K || !E) return MX_ERR_SHAPE;
+    for (uint32_t i = 0; i <= E; ++i) expert_offsets[i] = 0;
+    for (uint64_t i = 0; i < (uint64_t)T * K; ++i) {
+        if (topk_ids[i] < 0 || (uint32_t)topk_ids[i] >= E) return MX_ERR_SHAPE;
+        ++expert_offsets[topk_ids[i] + 1];
+    }
+    for (uint32_t e = 0; e < E; ++e) expert_offsets[e + 1] += expert_offsets[e];
+    uint32_t* cur = new uint32_t[E];
+    for (uint32_t e = 0; e < E; ++e) cur[e] = expert_offsets[e];
+    for (uint32_t t = 0; t < T; ++t)
+        for (uint32_t k = 0; k < K; ++k) {
+            const uint32_t pos = cur[topk_ids[(size_t)t * K + k]]++;
+            sorted_idx[pos] = (int32_t)t;
+            weights_packed[pos] = topk_w[(size_t)t * K + k];
+            tk_to_packed[(size_t)t * K + k] = (int32_t)pos;
+        }
+    delete[] cur;
+    return MX_OK;
+}
+
+}  // extern "C"

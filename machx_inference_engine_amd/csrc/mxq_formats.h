@@ -66,6 +66,13 @@ struct FmtQ4K {
     struct Raw {
         uint4 hdr, q0, q1;
     };
+    // expert bank: expert e at base + e * expert_stride_bytes (include/ie/ops.hpp:1027-1029)
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
     static constexpr int SUM_GRAN = 32;
     static constexpr bool PAIRED = true;
     static constexpr uint32_t GROUP_OFF = 16;
@@ -125,6 +132,12 @@ struct FmtQ6K {
         uint2 sc;             // scales[8h .. 8h+8)
         uint32_t d;
     };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
     static constexpr int SUM_GRAN = 16;
     static constexpr bool PAIRED = false;
     static constexpr uint32_t GROUP_OFF = 32;
@@ -178,6 +191,14 @@ struct FmtQ8Soa {
         const uint16_t* d;
         uint32_t K;
     };
+    // expert e: qs + e*qs_stride (elements), d + e*d_stride (fp16 entries) (include/ie/moe_q8.hpp:8-10)
+    struct Bank {
+        const int8_t* qs;
+        const uint16_t* d;
+        uint64_t qs_stride, d_stride;
+        uint32_t K;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.qs + (size_t)e * b.qs_stride, b.d + (size_t)e * b.d_stride, b.K}; }
     struct Cursor {
         const uint4* qs;
         const uint8_t* d;
@@ -277,6 +298,14 @@ struct FmtMxfp4Soa {
         const uint8_t* e;
         uint32_t K;
     };
+    // expert x: qs + x*qs_stride, e + x*e_stride bytes (src/model/gptoss.cpp:183-195)
+    struct Bank {
+        const uint8_t* qs;
+        const uint8_t* e;
+        uint64_t qs_stride, e_stride;
+        uint32_t K;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t x) { return {b.qs + (size_t)x * b.qs_stride, b.e + (size_t)x * b.e_stride, b.K}; }
     struct Cursor {
         const uint4* qs;
         const uint8_t* e;

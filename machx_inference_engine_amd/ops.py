@@ -180,3 +180,100 @@ def gemv_mxfp4_soa_f16(A, qs_plane, e_plane, K, N, y=None):
     y = _out(y, (N,), torch.float16, A)
     _call("mx_gemv_mxfp4_soa_f16", _f16(A), _u8(qs_plane), _u8(e_plane), _ptr(y), K, N)
     return y
+
+
+# ---------------------------------------------------------------- MoE, expert-indexed GEMV
+def moe_gate_up_silu_q8(x_q8, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, topk_idx, T, K, H, E_ffn, h_out=None):
+    h_out = _out(h_out, (T * K, E_ffn), torch.float16, x_q8)
+    _call("mx_moe_gate_up_silu_q8", _u8(x_q8), _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d), qs_stride, d_stride, _ptr(topk_idx),
+          _ptr(h_out), T, K, H, E_ffn)
+    return h_out
+
+
+def moe_down_q8(h_q8, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_ffn, H, y_packed=None):
+    y_packed = _out(y_packed, (T * K, H), torch.float16, h_q8)
+    _call("mx_moe_down_q8", _u8(h_q8), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(topk_idx), _f16(topk_w), _ptr(y_packed),
+          T, K, E_ffn, H)
+    return y_packed
+
+
+def moe_reduce_q8(y_packed, T, K, H, y=None):
+    y = _out(y, (T, H), torch.float16, y_packed)
+    _call("mx_moe_reduce_q8", _f16(y_packed), _ptr(y), T, K, H)
+    return y
+
+
+def moe_prefill_gate_up_silu_q8(xq8_packed, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, TK, E, H, E_ffn, h_packed=None):
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8_packed)
+    _call("mx_moe_prefill_gate_up_silu_q8", _u8(xq8_packed), _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d), qs_stride, d_stride,
+          _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn)
+    return h_packed
+
+
+def moe_prefill_down_q8(hq8_packed, d_qs, d_d, qs_stride, d_stride, expert_offsets, sorted_w, TK, E, H, E_ffn, out_packed=None):
+    out_packed = _out(out_packed, (TK, H), torch.float16, hq8_packed)
+    _call("mx_moe_prefill_down_q8", _u8(hq8_packed), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(expert_offsets), _f16(sorted_w),
+          _ptr(out_packed), E, H, E_ffn)
+    return out_packed
+
+
+def moe_prefill_reduce_sum(out_packed, tk_to_packed, T, K, H, y=None):
+    y = _out(y, (T, H), torch.float16, out_packed)
+    _call("mx_moe_prefill_reduce_sum", _f16(out_packed), _ptr(tk_to_packed), _ptr(y), T, K, H)
+    return y
+
+
+def moe_prefill_reduce(out_packed, tk_to_packed, weights_packed, y, T, K_top, H):
+    """y[t] += sum_k w[row] * out_packed[row]; accumulates into y (the caller zeroes it)."""
+    _call("mx_moe_prefill_reduce", _f16(out_packed), _ptr(tk_to_packed), _f16(weights_packed), _f16(y), T, K_top, H)
+    return y
+
+
+def moe_gather_rows(x, indices, n_rows, hidden, y_packed=None):
+    y_packed = _out(y_packed, (n_rows, hidden), torch.float16, x)
+    _call("mx_moe_gather_rows", _f16(x), _ptr(indices), _ptr(y_packed), n_rows, hidden)
+    return y_packed
+
+
+def moe_gate_up_oai_mxfp4(x_q8, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, topk_idx, T, K, H, E_ffn, n_experts,
+                          alpha=1.702, limit=7.0, h_out=None):
+    h_out = _out(h_out, (T * K, E_ffn), torch.float16, x_q8)
+    _call("mx_moe_gate_up_oai_mxfp4", _u8(x_q8), _u8(g_qs), _u8(g_e), _u8(u_qs), _u8(u_e), qs_stride, e_stride, _ptr(gate_bias),
+          _ptr(up_bias), _ptr(topk_idx), _ptr(h_out), T, K, H, E_ffn, n_experts, alpha, limit)
+    return h_out
+
+
+def moe_down_mxfp4(h_q8, d_qs, d_e, qs_stride, e_stride, down_bias, topk_idx, T, K, E_ffn, H, n_experts, out_packed=None):
+    out_packed = _out(out_packed, (T * K, H), torch.float16, h_q8)
+    _call("mx_moe_down_mxfp4", _u8(h_q8), _u8(d_qs), _u8(d_e), qs_stride, e_stride, _ptr(down_bias), _ptr(topk_idx), _ptr(out_packed),
+          T, K, E_ffn, H, n_experts)
+    return out_packed
+
+
+def moe_grouped_gate_up_oai_mxfp4(xq8_packed, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, expert_offsets, TK, E, H,
+                                  E_ffn, alpha=1.702, limit=7.0, h_packed=None):
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8_packed)
+    _call("mx_moe_grouped_gate_up_oai_mxfp4", _u8(xq8_packed), _u8(g_qs), _u8(g_e), _u8(u_qs), _u8(u_e), qs_stride, e_stride,
+          _ptr(gate_bias), _ptr(up_bias), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn, TK, alpha, limit)
+    return h_packed
+
+
+def moe_grouped_down_mxfp4(hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias, expert_offsets, TK, E, H, E_ffn, out_packed=None):
+    out_packed = _out(out_packed, (TK, H), torch.float16, hq8_packed)
+    _call("mx_moe_grouped_down_mxfp4", _u8(hq8_packed), _u8(d_qs), _u8(d_e), qs_stride, e_stride, _ptr(down_bias), _ptr(expert_offsets),
+          _ptr(out_packed), E, H, E_ffn, TK)
+    return out_packed
+
+
+def build_moe_packing(topk_ids, topk_w, E):
+    """Host counting sort (numpy in, numpy out): expert_offsets[E+1], sorted_idx, weights_packed, tk_to_packed."""
+    import numpy as np
+    ids = np.ascontiguousarray(topk_ids, np.int32)
+    w = np.ascontiguousarray(topk_w, np.float32)
+    T, K = ids.shape
+    off, si = np.empty(E + 1, np.uint32), np.empty(T * K, np.int32)
+    wp, t2p = np.empty(T * K, np.float32), np.empty(T * K, np.int32)
+    rc = lib.mx_build_moe_packing(ids.ctypes.data, w.ctypes.data, T, K, E, off.ctypes.data, si.ctypes.data, wp.ctypes.data, t2p.ctypes.data)
+    if rc != 0:
+        raise MxError("mx_build_moe_packing", rc)
+    return off, si, wp, t2p

@@ -1,0 +1,191 @@
+"""GPU parity: expert-indexed GEMV kernels (MoE decode with device-side expert ids
+and the expert-grouped form) for MXFP4 experts (gpt-oss shape family, BASELINE
+config 4) and Q8_0 SoA experts, stage by stage against the oracle, and the whole
+layer against a per-token per-expert brute-force loop."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import check, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+def make_experts(fmt, seed, E, N, K):
+    """E experts of [N, K] weights -> (AoS blocks [E, N, row_bytes], SoA planes)."""
+    W = np.stack([O.quantize(fmt, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
+    if fmt == O.MXFP4:
+        qs, sc = O.repack_mxfp4_to_soa(W)
+        return W, qs, sc, N * K // 2, N * K // 32
+    qs, sc = O.repack_q8_0_to_soa(W)
+    return W, qs, sc, N * K, N * K // 32
+
+
+def route(seed, T, E, k):
+    ids, w = O.route_from_logits(O.normal(seed, (T, E)), k)
+    return ids, w
+
+
+def f16(a):
+    return O.round_fp16(np.asarray(a, np.float32))
+
+
+def check_rows(a, b, what):
+    """Two fp16 results of the same arithmetic: equal up to a few fp16 ulps where fp32 noise crosses a
+    rounding boundary (and is then re-quantised downstream)."""
+    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+    rms = float(np.sqrt(np.mean(b32 * b32)))
+    frac_equal = float(np.mean(a == b))
+    err = float(np.abs(a32 - b32).max() / rms)
+    print("%s: %.4f bit-equal, max_abs/rms=%.2e" % (what, frac_equal, err), flush=True)
+    assert frac_equal > 0.98 and err < 1e-2, what
+
+
+# Stages that mirror the reference's chain of fp16 roundings (half(acc + bias), then the fp16
+# activation or bias add) can land one fp16 ulp (2^-10 relative) away from the fp64 evaluation
+# when an intermediate value sits next to a rounding boundary; their gate is 2 fp16 ulps.
+CHAIN_GATE = 2e-3
+
+
+def ref_gate_up_oai(Wg, Wu, bg, bu, e, xq_row, K, N):
+    """-> (lo, hi) envelope of half(swiglu_oai(g16, u16)) over the admissible roundings of the two
+    intermediates: the fp32 device sums may sit on the other side of an fp16 rounding boundary than
+    the fp64 oracle sums, and swiglu_oai's (up + 1) factor can amplify that ulp without bound in
+    relative terms, so the stage is checked against the set of results the reference chain can
+    produce when g16 / u16 move by at most one fp16 ulp."""
+    g = f16(O.gemv_q8chain(O.MXFP4, Wg[e], xq_row, K, N)[0] + bg[e]).astype(np.float16)
+    u = f16(O.gemv_q8chain(O.MXFP4, Wu[e], xq_row, K, N)[0] + bu[e]).astype(np.float16)
+    inf = np.float16(np.inf)
+    outs = [f16(O.swiglu_oai_np(gg.astype(np.float32), uu.astype(np.float32)))
+            for gg in (np.nextafter(g, -inf), g, np.nextafter(g, inf)) for uu in (np.nextafter(u, -inf), u, np.nextafter(u, inf))]
+    return np.min(outs, axis=0), np.max(outs, axis=0)
+
+
+def check_envelope(got, lo, hi, what):
+    got16 = got.astype(np.float16)
+    inf = np.float16(np.inf)
+    ok = (got16 >= np.nextafter(lo.astype(np.float16), -inf)) & (got16 <= np.nextafter(hi.astype(np.float16), inf))
+    print("%s: %d / %d inside the 1-ulp envelope" % (what, ok.sum(), ok.size), flush=True)
+    assert ok.all(), (what, np.argwhere(~ok)[:5], got[~ok][:5], lo[~ok][:5], hi[~ok][:5])
+
+
+@pytest.mark.parametrize("T,H,EF,E,Kt", [(1, 2880, 2880, 32, 4), (3, 512, 320, 6, 2), (32, 704, 384, 8, 4)])
+def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
+    """gpt-oss style layer: gate/up (+bias, swiglu_oai) -> quantize -> down (+bias) -> weighted reduce.
+    T=1, H=EF=2880, E=32, top-4 is BASELINE config 4's decode case at full size."""
+    ops = mx.ops
+    Wg, gq, ge, qs_st, e_st = make_experts(O.MXFP4, 100, E, EF, H)
+    Wu, uq, ue, _, _ = make_experts(O.MXFP4, 200, E, EF, H)
+    Wd, dq, de, dqs_st, de_st = make_experts(O.MXFP4, 300, E, H, EF)
+    bg, bu, bd = O.normal(1, (E, EF)), O.normal(2, (E, EF)), O.normal(3, (E, H))
+    x = f16(O.normal(4, (T, H)))
+    ids, w = route(5, T, E, Kt)
+    xq = O.quantize_q8_1(x)
+    rb = H // 32 * 40
+    D = dict(gq=dev(gq), ge=dev(ge), uq=dev(uq), ue=dev(ue), dq=dev(dq), de=dev(de), bg=dev(bg), bu=dev(bu), bd=dev(bd))
+    # ---- decode form: expert ids stay on the device
+    h = ops.moe_gate_up_oai_mxfp4(dev(xq), D["gq"], D["ge"], D["uq"], D["ue"], qs_st, e_st, D["bg"], D["bu"], dev(ids.ravel()), T, Kt, H, EF, E)
+    h_h = host(h).astype(np.float32)
+    env = [ref_gate_up_oai(Wg, Wu, bg, bu, ids[t, k], xq[t * rb:(t + 1) * rb], H, EF) for t in range(T) for k in range(Kt)]
+    check_envelope(h_h, np.stack([e[0] for e in env]), np.stack([e[1] for e in env]), "moe gate_up swiglu_oai (decode) T=%d" % T)
+    check(h_h, np.stack([(e[0] + e[1]) / 2 for e in env]), "  ... and against the envelope centre", max_rel=1.0, cos=0.99999)
+    hq = ops.quantize_q8_1(h)
+    hq_h = host(hq)
+    assert np.array_equal(hq_h, O.quantize_q8_1(h_h))
+    out = ops.moe_down_mxfp4(hq, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(ids.ravel()), T, Kt, EF, H, E)
+    out_h = host(out).astype(np.float32)
+    hrb = EF // 32 * 40
+    inf = np.float16(np.inf)
+    lo, hi = [], []
+    for s_ in range(T * Kt):   # out = half(half(acc) + bias): envelope over half(acc) moving by one ulp (the sum can cancel)
+        a16 = f16(O.gemv_q8chain(O.MXFP4, Wd[ids.ravel()[s_]], hq_h[s_ * hrb:(s_ + 1) * hrb], EF, H)[0]).astype(np.float16)
+        c = [f16(v.astype(np.float32) + bd[ids.ravel()[s_]]) for v in (np.nextafter(a16, -inf), a16, np.nextafter(a16, inf))]
+        lo.append(np.min(c, axis=0))
+        hi.append(np.max(c, axis=0))
+    check_envelope(out_h, np.stack(lo), np.stack(hi), "moe down + bias (decode)")
+    y = torch.zeros((T, H), dtype=torch.float16, device="cuda")
+    ident = dev(np.arange(T * Kt, dtype=np.uint32))
+    ops.moe_prefill_reduce(out, ident, dev(w.ravel()).half(), y, T, Kt, H)
+    w16 = f16(w)
+    y_ref = f16((w16[:, :, None] * out_h.reshape(T, Kt, H)).sum(axis=1))
+    check(host(y).astype(np.float32), y_ref, "moe weighted reduce")
+    # ---- grouped form: host packing, expert-sorted rows, every expert's weights streamed once
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    assert all(np.array_equal(a, b) for a, b in zip((off, si, wp, t2p), O.build_moe_packing(ids, w, E)))
+    TK = T * Kt
+    xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
+    assert np.array_equal(host(xp), x[si].astype(np.float16))
+    xpq = ops.quantize_q8_1(xp)
+    hp = ops.moe_grouped_gate_up_oai_mxfp4(xpq, D["gq"], D["ge"], D["uq"], D["ue"], qs_st, e_st, D["bg"], D["bu"], dev(off), TK, E, H, EF)
+    # same products per (token, expert); only the compiler's fma grouping may differ between the
+    # 1-row and the tiled instantiation, so rows agree to fp16 rounding of an fp32-noise difference
+    check_rows(host(hp)[t2p], host(h), "grouped gate_up == decode rows")
+    hpq = ops.quantize_q8_1(hp)
+    op = ops.moe_grouped_down_mxfp4(hpq, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(off), TK, E, H, EF)
+    check_rows(host(op)[t2p], host(out), "grouped down == decode rows")
+    y2 = torch.zeros((T, H), dtype=torch.float16, device="cuda")
+    ops.moe_prefill_reduce(op, dev(t2p.astype(np.uint32)), dev(wp).half(), y2, T, Kt, H)
+    check_rows(host(y2), host(y), "grouped layer output == decode layer output")
+
+
+@pytest.mark.parametrize("T,H,EF,E,Kt", [(1, 2048, 768, 16, 8), (5, 512, 256, 8, 2), (40, 256, 128, 4, 2)])
+def test_moe_q8_0_decode_and_grouped(mx, T, H, EF, E, Kt):
+    """Q8_0 SoA experts (include/ie/moe_q8.hpp): silu(gate)*up, route weight folded into down, plain-sum reduce."""
+    ops = mx.ops
+    Wg, gq, gd, qs_st, d_st = make_experts(O.Q8_0, 400, E, EF, H)
+    Wu, uq, ud, _, _ = make_experts(O.Q8_0, 500, E, EF, H)
+    Wd, dq, dd, dqs_st, dd_st = make_experts(O.Q8_0, 600, E, H, EF)
+    x = f16(O.normal(7, (T, H)))
+    ids, w = route(8, T, E, Kt)
+    xq = O.quantize_q8_1(x)
+    rb, hrb = H // 32 * 40, EF // 32 * 40
+    idsd = dev(ids.ravel())
+    h = ops.moe_gate_up_silu_q8(dev(xq), dev(gq), dev(gd), dev(uq), dev(ud), qs_st, d_st, idsd, T, Kt, H, EF)
+    h_h = host(h).astype(np.float32)
+    h_ref = np.stack([O.swiglu_np(O.gemv_q8chain(O.Q8_0, Wg[ids[t, k]], xq[t * rb:(t + 1) * rb], H, EF)[0].astype(np.float32),
+                                  O.gemv_q8chain(O.Q8_0, Wu[ids[t, k]], xq[t * rb:(t + 1) * rb], H, EF)[0].astype(np.float32))
+                      for t in range(T) for k in range(Kt)])
+    check(h_h, h_ref, "moe_gate_up_silu_q8 T=%d" % T)
+    hq = ops.quantize_q8_1(h)
+    hq_h = host(hq)
+    w16 = dev(w.ravel()).half()
+    yp = ops.moe_down_q8(hq, dev(dq), dev(dd), dqs_st, dd_st, idsd, w16, T, Kt, EF, H)
+    yp_ref = np.stack([f16(w.ravel()[s]) * O.gemv_q8chain(O.Q8_0, Wd[ids.ravel()[s]], hq_h[s * hrb:(s + 1) * hrb], EF, H)[0]
+                       for s in range(T * Kt)])
+    check(host(yp).astype(np.float32), yp_ref, "moe_down_q8")
+    y = ops.moe_reduce_q8(yp, T, Kt, H)
+    check(host(y).astype(np.float32), host(yp).astype(np.float32).reshape(T, Kt, H).sum(axis=1), "moe_reduce_q8")
+    # grouped form == decode form, row for row
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    TK = T * Kt
+    xpq = ops.quantize_q8_1(ops.moe_gather_rows(dev(x).half(), dev(si), TK, H))
+    hp = ops.moe_prefill_gate_up_silu_q8(xpq, dev(gq), dev(gd), dev(uq), dev(ud), qs_st, d_st, dev(off), TK, E, H, EF)
+    check_rows(host(hp)[t2p], host(h), "grouped gate_up == decode rows")
+    op = ops.moe_prefill_down_q8(ops.quantize_q8_1(hp), dev(dq), dev(dd), dqs_st, dd_st, dev(off), dev(wp).half(), TK, E, H, EF)
+    check_rows(host(op)[t2p], host(yp), "grouped down == decode rows")
+    y2 = ops.moe_prefill_reduce_sum(op, dev(t2p.astype(np.uint32)), T, Kt, H)
+    check_rows(host(y2), host(y), "grouped layer output == decode layer output")
+
+
+def test_moe_grouped_skips_empty_and_single_row_experts(mx):
+    """Experts with 0 rows write nothing; 1-row experts are exact (the reference notes
+    wrong rows for tiny per-expert batches on its dense-GEMM route, gptoss_tp.cpp:702-765)."""
+    ops = mx.ops
+    E, H, EF = 6, 256, 128
+    Wg, gq, gd, qs_st, d_st = make_experts(O.Q8_0, 700, E, EF, H)
+    Wu, uq, ud, _, _ = make_experts(O.Q8_0, 800, E, EF, H)
+    ids = np.array([[1], [1], [4], [1], [5], [1], [1], [1], [1], [1], [1]], np.int32)   # expert 1: 9 rows (two tiles), 4 and 5: one row
+    w = np.ones(ids.shape, np.float32)
+    x = f16(O.normal(9, (ids.shape[0], H)))
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    assert off.tolist() == [0, 0, 9, 9, 9, 10, 11]
+    xpq = ops.quantize_q8_1(ops.moe_gather_rows(dev(x).half(), dev(si), 11, H))
+    hp = torch.full((11, EF), 7.0, dtype=torch.float16, device="cuda")
+    ops.moe_prefill_gate_up_silu_q8(xpq, dev(gq), dev(gd), dev(uq), dev(ud), qs_st, d_st, dev(off), 11, E, H, EF, h_packed=hp)
+    xq_h = host(xpq)
+    rb = H // 32 * 40
+    ref = np.stack([O.swiglu_np(O.gemv_q8chain(O.Q8_0, Wg[ids[si[r], 0]], xq_h[r * rb:(r + 1) * rb], H, EF)[0].astype(np.float32),
+                                O.gemv_q8chain(O.Q8_0, Wu[ids[si[r], 0]], xq_h[r * rb:(r + 1) * rb], H, EF)[0].astype(np.float32))
+                    for r in range(11)])
+    check(host(hp).astype(np.float32), ref, "grouped with empty experts")
