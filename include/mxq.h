@@ -136,6 +136,32 @@ int mx_gemv_q4_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uin
 int mx_gemv_q6_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 
+/* ---------------------------------------------------------------- prefill quant-GEMM (matrix cores)
+ * y[M,N] = A[M,K] . half(deq(W))[N,K]^T, fp16 x fp16 MFMA, fp32 accumulate, fp16 out; any M.
+ * Replaces the 16-row XMX launches and the dequant + dense-GEMM route:
+ *   gemm_q4_K_xmx / gemm_q4_K_esimd / gemm_q4_K  include/ie/ops.hpp:607-611, src/ops/gemm_q4k_xmx.cpp:115-234
+ *   dequant_q4_K_to_Bt + gemm_fp16(_onednn)      src/model/dense_dispatch.hpp:658-693
+ * K % 256 == 0 (Q4_K), K % 128 == 0 (Q8_0 planes); A and W 16-byte aligned.
+ * mx_gemm_q8_0_soa takes the SoA planes of gemv_q8_0_soa_q8 (the reference runs Q8_0 prefill
+ * as dequant_q8_0_soa_to_Bt + gemm_fp16, src/model/qwen35_dense.cpp:811-831).  */
+int mx_gemm_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M,
+                     uint32_t K, uint32_t N);
+/* Expert-grouped GEMM over expert-sorted fp16 rows (Q8_0 SoA expert banks): the matrix-core
+ * form of moe_prefill_gate_up_silu_q8 / moe_prefill_down_q8 (include/ie/moe_q8.hpp:51-72) for
+ * fp16 activations — same arguments except that the activation rows are fp16 instead of
+ * block_q8_1x and the host passes total_rows = expert_offsets[E] (known from the packing).
+ *   h_packed[row, n]   = half(silu(gate_e . x_row) * (up_e . x_row))
+ *   out_packed[row, n] = half(sorted_w[row] * (down_e . h_row))
+ * H % 128 == 0 and E_ffn % 128 == 0.  */
+int mx_moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x_packed, const int8_t* g_qs, const uint16_t* g_d,
+                                const int8_t* u_qs, const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride,
+                                const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                                uint32_t total_rows);
+int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                        uint64_t d_stride, const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed,
+                        uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+
 /* ---------------------------------------------------------------- MoE, expert-indexed GEMV
  * Q8_0-expert decode kernels (device-resident routing: the expert of token slot
  * tk = t*K + k is read from topk_idx[tk]; no host round trip):

@@ -277,3 +277,30 @@ def build_moe_packing(topk_ids, topk_w, E):
     if rc != 0:
         raise MxError("mx_build_moe_packing", rc)
     return off, si, wp, t2p
+
+
+# ---------------------------------------------------------------- prefill GEMM (MFMA)
+def gemm_q4_K(A, W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_q4_K", _f16(A), _u8(W), _ptr(y), M, K, N)
+    return y
+
+
+def gemm_q8_0_soa(A, qs_W, d_W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_q8_0_soa", _f16(A), _u8(qs_W), _ptr(d_W), _ptr(y), M, K, N)
+    return y
+
+
+def moe_gemm_gate_up_silu_q8(x_packed, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, TK, E, H, E_ffn, h_packed=None):
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
+    _call("mx_moe_gemm_gate_up_silu_q8", _f16(x_packed), _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d), qs_stride, d_stride,
+          _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn, TK)
+    return h_packed
+
+
+def moe_gemm_down_q8(h_packed, d_qs, d_d, qs_stride, d_stride, expert_offsets, sorted_w, TK, E, H, E_ffn, out_packed=None):
+    out_packed = _out(out_packed, (TK, H), torch.float16, h_packed)
+    _call("mx_moe_gemm_down_q8", _f16(h_packed), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(expert_offsets), _f16(sorted_w),
+          _ptr(out_packed), E, H, E_ffn, TK)
+    return out_packed

@@ -291,8 +291,12 @@ def load_ref():
 
 
 # ---------------------------------------------------------------- parity metrics
-def parity(got, ref):
+def parity(got, ref, abs_floor=0.0):
     """Metrics used by every parity test.
+
+    abs_floor : extra absolute floor of the denominator; fp16 outputs use 2^-14 (the
+              smallest normal half): below it the output format itself has absolute,
+              not relative, precision.
 
     max_rel : max_i |g-r| / max(|r_i|, 1e-2*rms(r))  -- elementwise relative error
               with a floor at 1 % of the signal RMS (outputs that cancel to ~0 carry
@@ -308,6 +312,6 @@ def parity(got, ref):
     if rms == 0.0:
         return {"max_rel": float(np.max(np.abs(g))) if g.size else 0.0, "cos": 1.0, "max_abs_over_rms": 0.0, "rms": 0.0}
     err = np.abs(g - r)
-    return {"max_rel": float(np.max(err / np.maximum(np.abs(r), 1e-2 * rms))),
+    return {"max_rel": float(np.max(err / np.maximum(np.abs(r), max(1e-2 * rms, abs_floor)))),
             "cos": float(np.dot(g, r) / (np.linalg.norm(g) * np.linalg.norm(r) + 1e-300)),
             "max_abs_over_rms": float(err.max() / rms), "rms": rms}

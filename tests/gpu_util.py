@@ -28,8 +28,9 @@ def weights(fmt, seed, N, K, std=0.02):
     return O.quantize(fmt, O.normal(seed, (N, K), 0.0, std))
 
 
-def check(got, ref, what, max_rel=GATE_MAX_REL, cos=GATE_COS):
-    p = O.parity(got, ref)
+def check(got, ref, what, max_rel=GATE_MAX_REL, cos=GATE_COS, abs_floor=2.0 ** -14):
+    """abs_floor: 2^-14 for fp16 outputs (default; subnormal halfs carry absolute precision), 0 for fp32 outputs."""
+    p = O.parity(got, ref, abs_floor)
     msg = "%s: max_rel=%.3e cos=%.7f max_abs/rms=%.3e" % (what, p["max_rel"], p["cos"], p["max_abs_over_rms"])
     print(msg, flush=True)
     assert np.isfinite(np.asarray(got, np.float64)).all(), what + ": non-finite output"
