@@ -193,7 +193,7 @@ __device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const
 }
 
 template <class QF, int MODE>
-__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     half_t* lds = reinterpret_cast<half_t*>(lds_raw);
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
@@ -263,24 +263,54 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(typename QF::Bank ba
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    typename QF::Raw raw[2], nxt[2];
-    uint4 areg[8];
+    // Software pipeline over K chunks: the weight words and the A rows of chunk c+1 are
+    // fetched from global while chunk c is multiplied; the A rows go through registers in
+    // two halves (rows 0..63 during steps 0-3, rows 64..127 during steps 4-7) into the
+    // other LDS buffer.  The last chunk is peeled so the loop body has no conditionals.
+    typename QF::Raw raw[2];
     raw[0] = QF::load(w0, wrow[0], 0, h);
     raw[1] = QF::load(w1, wrow[1], 0, h);
+    {
+        uint4 a0[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const uint4*>(a_src[i]);
+        for (int i = 0; i < 8; ++i) a0[i] = *reinterpret_cast<const uint4*>(a_src[i]);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(lds + (size_t)(a_row + 16 * i) * kPitch + a_col) = areg[i];
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(lds + (size_t)(a_row + 16 * i) * kPitch + a_col) = a0[i];
+    }
     __syncthreads();
 
-    for (uint32_t c = 0; c < n_chunks; ++c) {
-        const bool more = c + 1 < n_chunks;
-        if (more) {
-            nxt[0] = QF::load(w0, wrow[0], c + 1, h);
-            nxt[1] = QF::load(w1, wrow[1], c + 1, h);
+    for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
+        typename QF::Raw nxt[2];
+        nxt[0] = QF::load(w0, wrow[0], c + 1, h);
+        nxt[1] = QF::load(w1, wrow[1], c + 1, h);
+        uint4 alo[4], ahi[4];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const uint4*>(a_src[i] + (size_t)(c + 1) * kBK);
-        }
+        for (int i = 0; i < 4; ++i) alo[i] = *reinterpret_cast<const uint4*>(a_src[i] + (size_t)(c + 1) * kBK);
+        typename QF::Dec dec[2];
+        dec[0] = QF::prepare(raw[0], c, h);
+        dec[1] = QF::prepare(raw[1], c, h);
+        const half_t* a_lds = lds + (size_t)(c & 1u) * (kBM * kPitch);
+        half_t* dst = lds + (size_t)((c + 1) & 1u) * (kBM * kPitch);
+        mma_step<0, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<1, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<2, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<3, QF>(raw, dec, a_lds, r, h, acc);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * i) * kPitch + a_col) = alo[i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ahi[i] = *reinterpret_cast<const uint4*>(a_src[4 + i] + (size_t)(c + 1) * kBK);
+        mma_step<4, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<5, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<6, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<7, QF>(raw, dec, a_lds, r, h, acc);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * (4 + i)) * kPitch + a_col) = ahi[i];
+        raw[0] = nxt[0];
+        raw[1] = nxt[1];
+        __syncthreads();
+    }
+    {
+        const uint32_t c = n_chunks - 1;
         typename QF::Dec dec[2];
         dec[0] = QF::prepare(raw[0], c, h);
         dec[1] = QF::prepare(raw[1], c, h);
@@ -293,14 +323,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(typename QF::Bank ba
         mma_step<5, QF>(raw, dec, a_lds, r, h, acc);
         mma_step<6, QF>(raw, dec, a_lds, r, h, acc);
         mma_step<7, QF>(raw, dec, a_lds, r, h, acc);
-        if (more) {
-            half_t* dst = lds + (size_t)((c + 1) & 1u) * (kBM * kPitch);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * i) * kPitch + a_col) = areg[i];
-            raw[0] = nxt[0];
-            raw[1] = nxt[1];
-        }
-        __syncthreads();
     }
 
     // ---- epilogue.  MFMA C layout: lane holds column n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4.
