@@ -197,6 +197,89 @@ def main():
         y16 = torch.empty(4096, dtype=torch.float16, device=dev)
         us = kernel_avg_us(lambda i: ops.gemv_q4_K_q8(aq, w1[i % len(w1)], 4096, 4096, y16), 2 * len(w1))
         detail["config1_q4_K_4096x4096_q8"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del w1
+        # BASELINE config 3: prefill quant-GEMM, Q4_K, fp16 MFMA (peak 2.5 PFLOP/s dense fp16)
+        MFMA_PEAK = 2500.0
+        for (K, N) in ((H, FF), (FF, H)):
+            wq = synth.random_weights("q4_K", N, K, seed=900, device=dev)
+            for T in (512, 2048, 4096):
+                a16 = torch.randn((T, K), device=dev, generator=g).half()
+                yg = torch.empty((T, N), dtype=torch.float16, device=dev)
+                us = kernel_avg_us(lambda i: ops.gemm_q4_K(a16, wq, T, K, N, yg), 4)
+                tf = 2.0 * T * N * K / us / 1e6
+                detail["config3_gemm_q4_K_T%d_K%d_N%d" % (T, K, N)] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
+                del a16, yg
+            del wq
+        # BASELINE config 4: MXFP4 MoE decode at gpt-oss-20b shape (E=32, top-4, H=EF=2880), T=1 and T=32
+        import numpy as np
+        E4, K4, H4 = 32, 4, 2880
+        nrep = 6   # rotate expert banks so a decode step cannot live in the Infinity Cache
+        banks = []
+        for i in range(nrep):
+            gq, ge = synth.split_mxfp4(synth.random_weights("mxfp4", E4 * H4, H4, seed=3000 + i, device=dev))
+            uq, ue = synth.split_mxfp4(synth.random_weights("mxfp4", E4 * H4, H4, seed=3100 + i, device=dev))
+            dq, de = synth.split_mxfp4(synth.random_weights("mxfp4", E4 * H4, H4, seed=3200 + i, device=dev))
+            banks.append((gq, ge, uq, ue, dq, de))
+        qs_st, e_st = H4 * H4 // 2, H4 * H4 // 32
+        per_expert = 3 * (qs_st + e_st)
+        rng = np.random.default_rng(4)
+        for T in (1, 32):
+            logits = rng.standard_normal((T, E4)).astype(np.float32)
+            ids = np.sort(np.argsort(-logits, axis=1)[:, :K4], axis=1).astype(np.int32)
+            wts = np.full((T, K4), 0.25, np.float32)
+            off, si, wp, t2p = ops.build_moe_packing(ids, wts, E4)
+            n_distinct = int((np.diff(off.astype(np.int64)) > 0).sum())
+            xt = torch.randn((T, H4), device=dev, generator=g).half()
+            TK = T * K4
+            offd, sid = torch.from_numpy(off).to(dev), torch.from_numpy(si).to(dev)
+            idsd = torch.from_numpy(ids.ravel().copy()).to(dev)
+            hbuf = torch.empty((TK, H4), dtype=torch.float16, device=dev)
+            obuf = torch.empty((TK, H4), dtype=torch.float16, device=dev)
+            xq8 = ops.quantize_q8_1(xt)
+            xpq = ops.quantize_q8_1(ops.moe_gather_rows(xt, sid, TK, H4))
+            hq8 = ops.quantize_q8_1(hbuf)
+
+            def layer(i):
+                b = banks[i % nrep]
+                if T == 1:    # device-side expert ids, one launch per stage
+                    ops.moe_gate_up_oai_mxfp4(xq8, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, idsd, T, K4, H4, H4, E4, h_out=hbuf)
+                    ops.quantize_q8_1(hbuf, hq8)
+                    ops.moe_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
+                else:         # expert-grouped rows, each routed expert streamed once
+                    ops.moe_grouped_gate_up_oai_mxfp4(xpq, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, offd, TK, E4, H4, H4, h_packed=hbuf)
+                    ops.quantize_q8_1(hbuf, hq8)
+                    ops.moe_grouped_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, offd, TK, E4, H4, H4, out_packed=obuf)
+
+            us = kernel_avg_us(layer, 2 * nrep)
+            bts = n_distinct * per_expert
+            detail["config4_moe_mxfp4_T%d" % T] = {"us": round(us, 1), "distinct_experts": n_distinct, "GBps": round(bts / us / 1e3, 1),
+                                                   "frac_hbm": round(bts / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del banks
+        # BASELINE config 5: Qwen3-MoE style grouped GEMM, E=128 top-8 H=2048 EF=768, 2048 tokens, Zipf(1.1), Q8_0 experts
+        E5, K5, H5, EF5, T5 = 128, 8, 2048, 768, 2048
+        gq5, gd5 = synth.split_q8_0(synth.random_weights("q8_0", E5 * EF5, H5, seed=5000, device=dev))
+        uq5, ud5 = synth.split_q8_0(synth.random_weights("q8_0", E5 * EF5, H5, seed=5001, device=dev))
+        dq5, dd5 = synth.split_q8_0(synth.random_weights("q8_0", E5 * H5, EF5, seed=5002, device=dev))
+        pz = np.arange(1, E5 + 1, dtype=np.float64) ** -1.1
+        pz = pz[rng.permutation(E5)]
+        pz /= pz.sum()
+        ids5 = np.stack([np.sort(rng.choice(E5, size=K5, replace=False, p=pz)) for _ in range(T5)]).astype(np.int32)
+        w5 = np.full(ids5.shape, 1.0 / K5, np.float32)
+        off5, si5, wp5, t2p5 = ops.build_moe_packing(ids5, w5, E5)
+        TK5 = T5 * K5
+        x5 = torch.randn((T5, H5), device=dev, generator=g).half()
+        off5d, wp5d = torch.from_numpy(off5).to(dev), torch.from_numpy(wp5).to(dev).half()
+        xp5 = ops.moe_gather_rows(x5[:, :].contiguous(), torch.from_numpy(si5).to(dev), TK5, H5) if TK5 <= 65535 else None
+        h5 = torch.empty((TK5, EF5), dtype=torch.float16, device=dev)
+        o5 = torch.empty((TK5, H5), dtype=torch.float16, device=dev)
+
+        def layer5(i):
+            ops.moe_gemm_gate_up_silu_q8(xp5, gq5, gd5, uq5, ud5, EF5 * H5, EF5 * H5 // 32, off5d, TK5, E5, H5, EF5, h5)
+            ops.moe_gemm_down_q8(h5, dq5, dd5, H5 * EF5, H5 * EF5 // 32, off5d, wp5d, TK5, E5, H5, EF5, o5)
+
+        us = kernel_avg_us(layer5, 3)
+        tf = 2.0 * TK5 * H5 * EF5 * 3 / us / 1e6
+        detail["config5_moe_grouped_gemm_q8_0"] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
         out["detail"] = detail
 
     # ---------------------------------------------------------------- CPU baseline (reported only)

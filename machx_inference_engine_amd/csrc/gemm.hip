@@ -177,12 +177,25 @@ struct GemmArgs {
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
 
-template <int S, class QF>
+// `mi` = number of live 32-token tiles of this workgroup tile (4 unless PARTIAL: expert-grouped
+// tiles are often mostly empty, and their dead token tiles skip both the LDS reads and the MFMAs).
+template <int S, class QF, bool PARTIAL>
 __device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const half_t* a_lds, uint32_t r,
-                                         uint32_t h, float16_t (&acc)[4][2]) {
+                                         uint32_t h, float16_t (&acc)[4][2], uint32_t mi) {
     Frag bf[2];
     QF::template frag<S>(raw[0], dec[0], bf[0]);
     QF::template frag<S>(raw[1], dec[1], bf[1]);
+    if (PARTIAL) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if ((uint32_t)i < mi) {
+                Frag af;
+                af.q = *reinterpret_cast<const uint4*>(a_lds + (size_t)(32 * i + r) * kPitch + 64 * h + 8 * S);
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af.v, bf[0].v, acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af.v, bf[1].v, acc[i][1], 0, 0, 0);
+            }
+        return;
+    }
     Frag af[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) af[i].q = *reinterpret_cast<const uint4*>(a_lds + (size_t)(32 * i + r) * kPitch + 64 * h + 8 * S);
@@ -215,21 +228,39 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
     }
     uint32_t e = 0, row_lo = 0, row_hi = g.M;
     if (MODE != GEMM_DENSE) {
-        // tm-th 128-row tile over all experts: walk the offsets
-        uint32_t t = tm;
-        bool found = false;
-        for (e = 0; e < g.E; ++e) {
-            const uint32_t lo = g.expert_offsets[e], hi = g.expert_offsets[e + 1];
-            const uint32_t nt = (hi - lo + kBM - 1) / kBM;
-            if (t < nt) {
-                row_lo = lo + t * kBM;
-                row_hi = hi;
-                found = true;
-                break;
+        // tm-th 128-row tile over all experts: wave 0 scans the per-expert tile counts, 64 experts at a time
+        __shared__ uint32_t s_tile[3];
+        const uint32_t ln = threadIdx.x & 63u;
+        if (threadIdx.x < 64) {
+            uint32_t base = 0;
+            bool found = false;
+            for (uint32_t e0 = 0; e0 < g.E && !found; e0 += 64) {
+                const uint32_t ee = e0 + ln;
+                const uint32_t lo = ee < g.E ? g.expert_offsets[ee] : 0u, hi = ee < g.E ? g.expert_offsets[ee + 1] : 0u;
+                const uint32_t nt = (hi - lo + kBM - 1) / kBM;
+                uint32_t incl = nt;
+#pragma unroll
+                for (int d = 1; d < 64; d <<= 1) {
+                    const uint32_t v = (uint32_t)__shfl_up((int)incl, d);
+                    if (ln >= (uint32_t)d) incl += v;
+                }
+                const uint32_t excl = base + incl - nt;
+                const bool hit = tm >= excl && tm < excl + nt;
+                if (hit) {
+                    s_tile[0] = ee;
+                    s_tile[1] = lo + (tm - excl) * kBM;
+                    s_tile[2] = hi;
+                }
+                found = __ballot(hit) != 0ull;
+                base += (uint32_t)__shfl((int)incl, 63);
             }
-            t -= nt;
+            if (!found && ln == 0) s_tile[0] = 0xFFFFFFFFu;
         }
-        if (!found) return;
+        __syncthreads();
+        e = s_tile[0];
+        if (e == 0xFFFFFFFFu) return;
+        row_lo = s_tile[1];
+        row_hi = s_tile[2];
     } else {
         row_lo = tm * kBM;
     }
@@ -254,6 +285,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         a_src[i] = g.A + (size_t)row * g.K + a_col;
     }
     const uint32_t n_chunks = g.K / kBK;
+    constexpr bool PARTIAL = MODE != GEMM_DENSE;
+    const uint32_t live_rows = row_hi - row_lo;
+    const uint32_t mi = live_rows >= (uint32_t)kBM ? 4u : (live_rows + 31u) / 32u;
 
     float16_t acc[4][2];
 #pragma unroll
@@ -291,18 +325,18 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         dec[1] = QF::prepare(raw[1], c, h);
         const half_t* a_lds = lds + (size_t)(c & 1u) * (kBM * kPitch);
         half_t* dst = lds + (size_t)((c + 1) & 1u) * (kBM * kPitch);
-        mma_step<0, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<1, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<2, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<3, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<0, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<1, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<2, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<3, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
 #pragma unroll
         for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * i) * kPitch + a_col) = alo[i];
 #pragma unroll
         for (int i = 0; i < 4; ++i) ahi[i] = *reinterpret_cast<const uint4*>(a_src[4 + i] + (size_t)(c + 1) * kBK);
-        mma_step<4, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<5, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<6, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<7, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<4, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<5, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<6, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<7, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
 #pragma unroll
         for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * (4 + i)) * kPitch + a_col) = ahi[i];
         raw[0] = nxt[0];
@@ -315,14 +349,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         dec[0] = QF::prepare(raw[0], c, h);
         dec[1] = QF::prepare(raw[1], c, h);
         const half_t* a_lds = lds + (size_t)(c & 1u) * (kBM * kPitch);
-        mma_step<0, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<1, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<2, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<3, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<4, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<5, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<6, QF>(raw, dec, a_lds, r, h, acc);
-        mma_step<7, QF>(raw, dec, a_lds, r, h, acc);
+        mma_step<0, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<1, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<2, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<3, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<4, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<5, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<6, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_step<7, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
     }
 
     // ---- epilogue.  MFMA C layout: lane holds column n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4.
