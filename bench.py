@@ -44,6 +44,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-detail", action="store_true", help="skip the per-config detail table")
     ap.add_argument("--sets", type=int, default=4, help="distinct weight sets rotated through (331.7 MB each)")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter probe for `rocprofv3 --pmc`: a few launches of the dominant kernels and of a plain copy of known size, no timing")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures one GPU only (the path is data-parallel over output rows / experts; "
@@ -97,6 +99,22 @@ def main():
             gemv(fmt, hq, ws, "down", FF, H, y_h[fmt])
 
     bytes_per_step = sum(gemv_bytes(synth.row_bytes(f, K), K, N, 1) for f in fmts for (K, N) in shapes.values())
+
+    if args.probe:
+        # plain copy of known size first (the scale for FETCH_SIZE / WRITE_SIZE), then the kernels under study
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        for i in range(8):
+            step(sets[i % len(sets)])
+        wq = synth.random_weights("q4_K", FF, H, seed=900, device=dev)
+        a16 = torch.randn((2048, H), device=dev, generator=g).half()
+        for _ in range(4):
+            ops.gemm_q4_K(a16, wq, 2048, H, FF)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy 268435456 B x4; 8 decode steps; gemm_q4_K T=2048 K=4096 N=14336 x4"}))
+        return
 
     # ---------------------------------------------------------------- warm-up, graphs
     for i in range(args.warmup):
@@ -152,7 +170,9 @@ def main():
     dom_bytes = gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": "gemv_q8_kernel<FmtQ8Soa,T=1> K=4096 N=14336", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt)
+                "traffic": 62483456 + 114790,
                 "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 3)}
 
     out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
