@@ -36,15 +36,29 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 constexpr int kBM = 128;            // tokens per workgroup tile
 constexpr int kBK = 128;            // K chunk
 constexpr int kWaveN = 64;          // weight rows per wave (2 MFMA tiles)
-constexpr int kPitch = kBK + 8;     // LDS row pitch in halfs (272 B)
 constexpr int kGemmThreads = 256;
-constexpr uint32_t kGemmLds = 2u * kBM * kPitch * 2u;
+constexpr uint32_t kABuf = kBM * kBK * 2u;   // one A chunk in LDS: 128 rows x 256 B, unpadded, 16-byte columns XOR-swizzled by row
+constexpr uint32_t kGemmLds = 2u * kABuf;
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     const float2_t f = {a, b};
     const half2_t h = __builtin_convertvector(f, half2_t);   // v_cvt_pk_f16_f32, RNE
     return __builtin_bit_cast(uint32_t, h);
 }
+
+// Two consecutive weights of a fragment from integer codes held as fp16 subnormals: the bits
+// 0x0000 | u (u < 1024) read as fp16 are exactly u * 2^-24, so half(fma(u * 2^-24, scale * 2^24, off))
+// is the dequantized weight with the integer -> float conversion folded into the operand
+// (v_fma_mixlo/mixhi_f16: fp16 source, fp32 scale/offset, fused fp32 multiply-add, one RNE to
+// fp16).  The power-of-two rescale of `scale` is exact, so the value is bit-identical to
+// converting the code to float first.
+__device__ __forceinline__ uint32_t mix_pair(_Float16 x0, _Float16 x1, float scale, float off) {
+    half2_t o;
+    o.x = (_Float16)__builtin_fmaf((float)x0, scale, off);
+    o.y = (_Float16)__builtin_fmaf((float)x1, scale, off);
+    return __builtin_bit_cast(uint32_t, o);
+}
+__device__ __forceinline__ half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 
 union Frag {
     half8_t v;
@@ -55,8 +69,9 @@ union Frag {
 // ---------------------------------------------------------------- weight fragment producers
 // Q4_K: chunk kc of a row = half c = kc%2 of block kc/2; lane half h owns the 32 bytes
 // qs[32g, 32g+32), g = 2c + h: low nibbles = sub-block 2g, high = sub-block 2g+1.
-// value = half(fma(d*sc, q, -(dmin*m))): the products are exact in fp32 so this is
-// the single fp32 rounding of the reference expression, then one RNE to fp16.
+// value = half(fma(d*sc, q, -(dmin*m))): the products are exact in fp32, so this is the single
+// fp32 rounding of the reference expression followed by one RNE to fp16.  A low nibble is the
+// subnormal q * 2^-24, a high nibble stays in place as q * 2^-20.
 struct GemmQ4K {
     struct W {
         const uint8_t* base;
@@ -72,7 +87,7 @@ struct GemmQ4K {
         uint4 hdr, q0, q1;
     };
     struct Dec {
-        float d1[2], m1[2];
+        float d1[2], c1[2];
     };
     static constexpr uint32_t K_ALIGN = 256;
     __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
@@ -89,10 +104,10 @@ struct GemmQ4K {
         q4k_scale_pair(r.hdr.y, r.hdr.z, r.hdr.w, (int)(2u * (kc & 1u) + h), sc, mn);
         const float d = h2f(r.hdr.x & 0xFFFFu), dmin = h2f(r.hdr.x >> 16);
         Dec o;
-        o.d1[0] = d * (float)(sc & 0xFFu);
-        o.d1[1] = d * (float)(sc >> 8);
-        o.m1[0] = -(dmin * (float)(mn & 0xFFu));
-        o.m1[1] = -(dmin * (float)(mn >> 8));
+        o.d1[0] = d * (float)(sc & 0xFFu) * 16777216.f;   // x 2^24
+        o.d1[1] = d * (float)(sc >> 8) * 1048576.f;       // x 2^20
+        o.c1[0] = -(dmin * (float)(mn & 0xFFu));
+        o.c1[1] = -(dmin * (float)(mn >> 8));
         return o;
     }
     template <int S>
@@ -100,20 +115,21 @@ struct GemmQ4K {
         constexpr int sub = S / 4, p = S % 4;
         const uint32_t w0 = p == 0 ? r.q0.x : p == 1 ? r.q0.z : p == 2 ? r.q1.x : r.q1.z;
         const uint32_t w1 = p == 0 ? r.q0.y : p == 1 ? r.q0.w : p == 2 ? r.q1.y : r.q1.w;
-        const uint32_t n0 = sub ? (w0 >> 4) & 0x0F0F0F0Fu : w0 & 0x0F0F0F0Fu;
-        const uint32_t n1 = sub ? (w1 >> 4) & 0x0F0F0F0Fu : w1 & 0x0F0F0F0Fu;
-        const float d1 = dc.d1[sub], m1 = dc.m1[sub];
-        f.u[0] = pack_h2(__builtin_fmaf(d1, (float)(n0 & 0xFFu), m1), __builtin_fmaf(d1, (float)((n0 >> 8) & 0xFFu), m1));
-        f.u[1] = pack_h2(__builtin_fmaf(d1, (float)((n0 >> 16) & 0xFFu), m1), __builtin_fmaf(d1, (float)(n0 >> 24), m1));
-        f.u[2] = pack_h2(__builtin_fmaf(d1, (float)(n1 & 0xFFu), m1), __builtin_fmaf(d1, (float)((n1 >> 8) & 0xFFu), m1));
-        f.u[3] = pack_h2(__builtin_fmaf(d1, (float)((n1 >> 16) & 0xFFu), m1), __builtin_fmaf(d1, (float)(n1 >> 24), m1));
+        constexpr uint32_t mask = sub ? 0x00F000F0u : 0x000F000Fu;
+        const half2_t e0 = as_h2(w0 & mask), o0 = as_h2((w0 >> 8) & mask);   // bytes (0,2), (1,3)
+        const half2_t e1 = as_h2(w1 & mask), o1 = as_h2((w1 >> 8) & mask);
+        const float d1 = dc.d1[sub], c1 = dc.c1[sub];
+        f.u[0] = mix_pair(e0.x, o0.x, d1, c1);
+        f.u[1] = mix_pair(e0.y, o0.y, d1, c1);
+        f.u[2] = mix_pair(e1.x, o1.x, d1, c1);
+        f.u[3] = mix_pair(e1.y, o1.y, d1, c1);
     }
 };
 
 // Q8_0 SoA planes: lane half h owns quants [128 kc + 64h, +64) of the row and the two
 // block scales.  value = half(d * q) (exact product, one RNE to fp16), computed as
-// fma(d, q + 128, -128 d) on the bias-flipped byte so that the conversion is a
-// single v_cvt_f32_ubyte.
+// fma((q ^ 0x80) * 2^-24, d * 2^24, -128 d): the bias-flipped byte is zero-extended into an
+// fp16 subnormal operand.
 struct GemmQ8Soa {
     struct W {
         const int8_t* qs;
@@ -149,6 +165,8 @@ struct GemmQ8Soa {
         o.d[1] = h2f(r.d2 >> 16);
         o.o[0] = -128.f * o.d[0];
         o.o[1] = -128.f * o.d[1];
+        o.d[0] *= 16777216.f;
+        o.d[1] *= 16777216.f;
         return o;
     }
     template <int S>
@@ -156,10 +174,12 @@ struct GemmQ8Soa {
         constexpr int blk = S / 4, i = (S * 2) / 4, e = (S * 2) % 4;
         const uint32_t a = (e == 0 ? r.q[i].x : r.q[i].z) ^ 0x80808080u, b = (e == 0 ? r.q[i].y : r.q[i].w) ^ 0x80808080u;
         const float d = dc.d[blk], o = dc.o[blk];
-        f.u[0] = pack_h2(__builtin_fmaf(d, (float)(a & 0xFFu), o), __builtin_fmaf(d, (float)((a >> 8) & 0xFFu), o));
-        f.u[1] = pack_h2(__builtin_fmaf(d, (float)((a >> 16) & 0xFFu), o), __builtin_fmaf(d, (float)(a >> 24), o));
-        f.u[2] = pack_h2(__builtin_fmaf(d, (float)(b & 0xFFu), o), __builtin_fmaf(d, (float)((b >> 8) & 0xFFu), o));
-        f.u[3] = pack_h2(__builtin_fmaf(d, (float)((b >> 16) & 0xFFu), o), __builtin_fmaf(d, (float)(b >> 24), o));
+        const half2_t a01 = as_h2(__builtin_amdgcn_perm(0u, a, 0x0C010C00u)), a23 = as_h2(__builtin_amdgcn_perm(0u, a, 0x0C030C02u));
+        const half2_t b01 = as_h2(__builtin_amdgcn_perm(0u, b, 0x0C010C00u)), b23 = as_h2(__builtin_amdgcn_perm(0u, b, 0x0C030C02u));
+        f.u[0] = mix_pair(a01.x, a01.y, d, o);
+        f.u[1] = mix_pair(a23.x, a23.y, d, o);
+        f.u[2] = mix_pair(b01.x, b01.y, d, o);
+        f.u[3] = mix_pair(b23.x, b23.y, d, o);
     }
 };
 
@@ -177,38 +197,60 @@ struct GemmArgs {
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
 
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// 16 bytes per lane from global memory straight into LDS, no registers in between
+// (global_load_lds_dwordx4: lane L of the wave lands at lds_addr + 16 L).  `base` and
+// `lds_addr` are wave-uniform.  The load counts on vmcnt like any other global load; the
+// data is visible in LDS once vmcnt has drained, so every consumer sits behind an explicit
+// vmcnt(0) + workgroup barrier.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // m0 is a reserved register; naming it as clobbered is the intent
+__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t byte_off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(base), "v"(byte_off), "s"(lds_addr) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+// One K chunk = 8 MFMA steps.  A fragment (token row R, 16-byte column c) sits at
+// R * 256 + ((c ^ (R & 15)) << 4): the 16 lanes of a quarter wave then hit 16 different
+// columns, i.e. all 64 banks once.  For step S the column is 8h + S, so the address is the
+// lane's step-0 address with bits 4-6 XOR-ed by S.
 // `mi` = number of live 32-token tiles of this workgroup tile (4 unless PARTIAL: expert-grouped
 // tiles are often mostly empty, and their dead token tiles skip both the LDS reads and the MFMAs).
 template <int S, class QF, bool PARTIAL>
-__device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const half_t* a_lds, uint32_t r,
-                                         uint32_t h, float16_t (&acc)[4][2], uint32_t mi) {
-    Frag bf[2];
-    QF::template frag<S>(raw[0], dec[0], bf[0]);
-    QF::template frag<S>(raw[1], dec[1], bf[1]);
-    if (PARTIAL) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if ((uint32_t)i < mi) {
-                Frag af;
-                af.q = *reinterpret_cast<const uint4*>(a_lds + (size_t)(32 * i + r) * kPitch + 64 * h + 8 * S);
-                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af.v, bf[0].v, acc[i][0], 0, 0, 0);
-                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af.v, bf[1].v, acc[i][1], 0, 0, 0);
-            }
-        return;
-    }
-    Frag af[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) af[i].q = *reinterpret_cast<const uint4*>(a_lds + (size_t)(32 * i + r) * kPitch + 64 * h + 8 * S);
+__device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
+                                         float16_t (&acc)[4][2], uint32_t mi) {
+    Frag af[4], bf[2];
+    const uint32_t a_s = a_frag0 ^ (uint32_t)(S << 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
+        if (!PARTIAL || (uint32_t)i < mi) af[i].q = *reinterpret_cast<const uint4*>(lds + a_s + i * 8192);
+    QF::template frag<S>(raw[0], dec[0], bf[0]);
+    QF::template frag<S>(raw[1], dec[1], bf[1]);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[j].v, acc[i][j], 0, 0, 0);
+    for (int i = 0; i < 4; ++i)
+        if (!PARTIAL || (uint32_t)i < mi) {
+            acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[0].v, acc[i][0], 0, 0, 0);
+            acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[1].v, acc[i][1], 0, 0, 0);
+        }
+}
+
+template <class QF, bool PARTIAL>
+__device__ __forceinline__ void mma_chunk(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
+                                          float16_t (&acc)[4][2], uint32_t mi) {
+    mma_step<0, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<1, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<2, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<3, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<4, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<5, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<6, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    mma_step<7, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
 }
 
 template <class QF, int MODE>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
-    half_t* lds = reinterpret_cast<half_t*>(lds_raw);
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
     constexpr uint32_t BN = GATE_UP ? 4 * 32 : 4 * kWaveN;   // output columns per workgroup
 
@@ -257,16 +299,17 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
             if (!found && ln == 0) s_tile[0] = 0xFFFFFFFFu;
         }
         __syncthreads();
-        e = s_tile[0];
+        e = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[0]);
         if (e == 0xFFFFFFFFu) return;
-        row_lo = s_tile[1];
-        row_hi = s_tile[2];
+        row_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[1]);
+        row_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[2]);
     } else {
         row_lo = tm * kBM;
     }
     const typename QF::W w0 = QF::expert(bank0, e), w1 = QF::expert(GATE_UP ? bank1 : bank0, e);
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, r = lane & 31u, h = lane >> 5;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 31u, h = lane >> 5;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_base = tn * BN + wave * (GATE_UP ? 32 : kWaveN);
     // weight rows of the two MFMA column tiles of this wave (gate/up: same row in two matrices)
     uint32_t wrow[2];
@@ -275,19 +318,26 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
     if (wrow[0] >= g.N) wrow[0] = g.N - 1;
     if (wrow[1] >= g.N) wrow[1] = g.N - 1;
 
-    // A staging: thread loads 8 x 16 B: rows (tid/16) + 16 i, 16-byte column tid%16
-    const uint32_t a_col = (tid & 15u) * 8u, a_row = tid >> 4;
-    const half_t* a_src[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        uint32_t row = row_lo + a_row + 16 * i;
-        if (row >= row_hi) row = row_hi - 1;
-        a_src[i] = g.A + (size_t)row * g.K + a_col;
-    }
     const uint32_t n_chunks = g.K / kBK;
     constexpr bool PARTIAL = MODE != GEMM_DENSE;
-    const uint32_t live_rows = row_hi - row_lo;
-    const uint32_t mi = live_rows >= (uint32_t)kBM ? 4u : (live_rows + 31u) / 32u;
+    const uint32_t live_rows = (row_hi - row_lo) >= (uint32_t)kBM ? (uint32_t)kBM : row_hi - row_lo;
+    const uint32_t mi = (live_rows + 31u) / 32u;
+
+    // A staging: wave w brings rows 32w .. 32w+31 of the chunk, 4 rows (1 KB) per load; lane L
+    // fills LDS slot (row 4j + L/16, column L%16) of that 1 KB with global column
+    // (L%16) ^ (row & 15).  Rows past the end of the tile re-read its last row (never used).
+    uint32_t a_off[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t R = 32u * wave + 4u * j + (lane >> 4);
+        const uint32_t Rc = R < live_rows ? R : live_rows - 1u;
+        a_off[j] = Rc * (g.K * 2u) + (((lane & 15u) ^ (R & 15u)) << 4);
+    }
+    const uint8_t* a_glb = reinterpret_cast<const uint8_t*>(g.A + (size_t)row_lo * g.K);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds_raw;
+    const uint32_t a_dst = lds_base + wave * 8192u;   // this wave's 32 rows inside an A buffer
+    // step-0 fragment address of this lane inside an A buffer
+    const uint32_t frag0 = r * 256u + (((8u * h) ^ (r & 15u)) << 4);
 
     float16_t acc[4][2];
 #pragma unroll
@@ -297,50 +347,34 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // Software pipeline over K chunks: the weight words and the A rows of chunk c+1 are
-    // fetched from global while chunk c is multiplied; the A rows go through registers in
-    // two halves (rows 0..63 during steps 0-3, rows 64..127 during steps 4-7) into the
-    // other LDS buffer.  The last chunk is peeled so the loop body has no conditionals.
+    // Software pipeline over K chunks: at the top of chunk c the A rows of chunk c+1 start
+    // their way into the other LDS buffer and the weight words of chunk c+1 into registers;
+    // both have the whole chunk (64 MFMAs per wave) to arrive.  The A rows are requested
+    // first: memory returns in order, and they come from L2 while the weights come from HBM.
     typename QF::Raw raw[2];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) load_to_lds16(a_glb, a_off[j], a_dst + 1024u * j);
     raw[0] = QF::load(w0, wrow[0], 0, h);
     raw[1] = QF::load(w1, wrow[1], 0, h);
-    {
-        uint4 a0[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) a0[i] = *reinterpret_cast<const uint4*>(a_src[i]);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(lds + (size_t)(a_row + 16 * i) * kPitch + a_col) = a0[i];
-    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
     __syncthreads();
 
     for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
+        const uint8_t* a_next = a_glb + (size_t)(c + 1) * (kBK * 2u);
+        const uint32_t dst = a_dst + ((c + 1) & 1u) * kABuf;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
         typename QF::Raw nxt[2];
         nxt[0] = QF::load(w0, wrow[0], c + 1, h);
         nxt[1] = QF::load(w1, wrow[1], c + 1, h);
-        uint4 alo[4], ahi[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) alo[i] = *reinterpret_cast<const uint4*>(a_src[i] + (size_t)(c + 1) * kBK);
+        __builtin_amdgcn_sched_barrier(0);   // the scheduler must not sink these loads towards their uses
         typename QF::Dec dec[2];
         dec[0] = QF::prepare(raw[0], c, h);
         dec[1] = QF::prepare(raw[1], c, h);
-        const half_t* a_lds = lds + (size_t)(c & 1u) * (kBM * kPitch);
-        half_t* dst = lds + (size_t)((c + 1) & 1u) * (kBM * kPitch);
-        mma_step<0, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<1, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<2, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<3, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * i) * kPitch + a_col) = alo[i];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) ahi[i] = *reinterpret_cast<const uint4*>(a_src[4 + i] + (size_t)(c + 1) * kBK);
-        mma_step<4, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<5, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<6, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<7, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(dst + (size_t)(a_row + 16 * (4 + i)) * kPitch + a_col) = ahi[i];
+        mma_chunk<QF, PARTIAL>(raw, dec, lds_raw, (c & 1u) * kABuf + frag0, acc, mi);
         raw[0] = nxt[0];
         raw[1] = nxt[1];
+        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): A rows of chunk c+1 are in LDS
         __syncthreads();
     }
     {
@@ -348,15 +382,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         typename QF::Dec dec[2];
         dec[0] = QF::prepare(raw[0], c, h);
         dec[1] = QF::prepare(raw[1], c, h);
-        const half_t* a_lds = lds + (size_t)(c & 1u) * (kBM * kPitch);
-        mma_step<0, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<1, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<2, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<3, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<4, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<5, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<6, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
-        mma_step<7, QF, PARTIAL>(raw, dec, a_lds, r, h, acc, mi);
+        mma_chunk<QF, PARTIAL>(raw, dec, lds_raw, (c & 1u) * kABuf + frag0, acc, mi);
     }
 
     // ---- epilogue.  MFMA C layout: lane holds column n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4.
@@ -468,3 +494,12 @@ int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d
 }
 
 }  // extern "C"
+
+// Resident workgroups per CU of the dense Q4_K GEMM kernel at its launch configuration
+// (diagnostic; negative = HIP error).
+extern "C" int mx_debug_gemm_occupancy(void) {
+    int n = 0;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mxq::gemm_kernel<mxq::GemmQ4K, mxq::GEMM_DENSE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)mxq::kGemmLds);
+    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mxq::gemm_kernel<mxq::GemmQ4K, mxq::GEMM_DENSE>, mxq::kGemmThreads, mxq::kGemmLds);
+    return e == hipSuccess ? n : -(int)e;
+}
