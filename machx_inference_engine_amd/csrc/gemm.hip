@@ -110,19 +110,22 @@ struct GemmQ4K {
         o.c1[1] = -(dmin * (float)(mn >> 8));
         return o;
     }
+    // Half HF of the fragment of step S: elements 4 HF .. 4 HF + 3 (words u[2 HF], u[2 HF + 1]).
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int sub = S / 4, p = S % 4;
+        const uint32_t w = HF == 0 ? (p == 0 ? r.q0.x : p == 1 ? r.q0.z : p == 2 ? r.q1.x : r.q1.z)
+                                   : (p == 0 ? r.q0.y : p == 1 ? r.q0.w : p == 2 ? r.q1.y : r.q1.w);
+        constexpr uint32_t mask = sub ? 0x00F000F0u : 0x000F000Fu;
+        const half2_t ev = as_h2(w & mask), od = as_h2((w >> 8) & mask);   // bytes (0,2), (1,3)
+        const float d1 = dc.d1[sub], c1 = dc.c1[sub];
+        f.u[2 * HF] = mix_pair(ev.x, od.x, d1, c1);
+        f.u[2 * HF + 1] = mix_pair(ev.y, od.y, d1, c1);
+    }
     template <int S>
     __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
-        constexpr int sub = S / 4, p = S % 4;
-        const uint32_t w0 = p == 0 ? r.q0.x : p == 1 ? r.q0.z : p == 2 ? r.q1.x : r.q1.z;
-        const uint32_t w1 = p == 0 ? r.q0.y : p == 1 ? r.q0.w : p == 2 ? r.q1.y : r.q1.w;
-        constexpr uint32_t mask = sub ? 0x00F000F0u : 0x000F000Fu;
-        const half2_t e0 = as_h2(w0 & mask), o0 = as_h2((w0 >> 8) & mask);   // bytes (0,2), (1,3)
-        const half2_t e1 = as_h2(w1 & mask), o1 = as_h2((w1 >> 8) & mask);
-        const float d1 = dc.d1[sub], c1 = dc.c1[sub];
-        f.u[0] = mix_pair(e0.x, o0.x, d1, c1);
-        f.u[1] = mix_pair(e0.y, o0.y, d1, c1);
-        f.u[2] = mix_pair(e1.x, o1.x, d1, c1);
-        f.u[3] = mix_pair(e1.y, o1.y, d1, c1);
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
     }
 };
 
@@ -169,17 +172,19 @@ struct GemmQ8Soa {
         o.d[1] *= 16777216.f;
         return o;
     }
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int blk = S / 4, i = (S * 2) / 4, e = (S * 2) % 4;
+        const uint32_t w = (HF == 0 ? (e == 0 ? r.q[i].x : r.q[i].z) : (e == 0 ? r.q[i].y : r.q[i].w)) ^ 0x80808080u;
+        const float d = dc.d[blk], o = dc.o[blk];
+        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C030C02u));
+        f.u[2 * HF] = mix_pair(w01.x, w01.y, d, o);
+        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, d, o);
+    }
     template <int S>
     __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
-        constexpr int blk = S / 4, i = (S * 2) / 4, e = (S * 2) % 4;
-        const uint32_t a = (e == 0 ? r.q[i].x : r.q[i].z) ^ 0x80808080u, b = (e == 0 ? r.q[i].y : r.q[i].w) ^ 0x80808080u;
-        const float d = dc.d[blk], o = dc.o[blk];
-        const half2_t a01 = as_h2(__builtin_amdgcn_perm(0u, a, 0x0C010C00u)), a23 = as_h2(__builtin_amdgcn_perm(0u, a, 0x0C030C02u));
-        const half2_t b01 = as_h2(__builtin_amdgcn_perm(0u, b, 0x0C010C00u)), b23 = as_h2(__builtin_amdgcn_perm(0u, b, 0x0C030C02u));
-        f.u[0] = mix_pair(a01.x, a01.y, d, o);
-        f.u[1] = mix_pair(a23.x, a23.y, d, o);
-        f.u[2] = mix_pair(b01.x, b01.y, d, o);
-        f.u[3] = mix_pair(b23.x, b23.y, d, o);
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
     }
 };
 
@@ -235,17 +240,56 @@ __device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const
         }
 }
 
+// Full tiles: the chunk as one software pipeline.  A step is cut into four segments, one per
+// token tile: its 2 MFMAs, the LDS read that refills that A fragment for step S+1 (first use
+// 6 MFMAs later), and a quarter of the dequantisation of the weight fragments of step S+1 into
+// the other fragment pair.  The scheduling fences between segments keep that interleaving, so
+// neither the VALU work nor the LDS latency ends up between two clusters of MFMAs.
+template <int S, class QF>
+__device__ __forceinline__ void mma_pipe(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
+                                         float16_t (&acc)[4][2], Frag (&af)[4], Frag (&bf)[2][2]) {
+    if constexpr (S < 8) {
+        constexpr int cur = S & 1, nxt = cur ^ 1, SN = (S + 1) & 7;
+        constexpr bool more = S + 1 < 8;
+        const uint32_t a_n = a_frag0 ^ (uint32_t)(SN << 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[cur][0].v, acc[i][0], 0, 0, 0);
+            acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[cur][1].v, acc[i][1], 0, 0, 0);
+            if (more) {
+                af[i].q = *reinterpret_cast<const uint4*>(lds + a_n + i * 8192);
+                if (i == 0) QF::template frag_half<SN, 0>(raw[0], dec[0], bf[nxt][0]);
+                if (i == 1) QF::template frag_half<SN, 1>(raw[0], dec[0], bf[nxt][0]);
+                if (i == 2) QF::template frag_half<SN, 0>(raw[1], dec[1], bf[nxt][1]);
+                if (i == 3) QF::template frag_half<SN, 1>(raw[1], dec[1], bf[nxt][1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        mma_pipe<S + 1, QF>(raw, dec, lds, a_frag0, acc, af, bf);
+    }
+}
+
 template <class QF, bool PARTIAL>
 __device__ __forceinline__ void mma_chunk(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
                                           float16_t (&acc)[4][2], uint32_t mi) {
-    mma_step<0, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<1, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<2, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<3, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<4, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<5, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<6, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-    mma_step<7, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    if constexpr (!PARTIAL) {
+        Frag af[4], bf[2][2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i].q = *reinterpret_cast<const uint4*>(lds + a_frag0 + i * 8192);
+        QF::template frag<0>(raw[0], dec[0], bf[0][0]);
+        QF::template frag<0>(raw[1], dec[1], bf[0][1]);
+        __builtin_amdgcn_sched_barrier(0);   // prologue stays ahead of the pipelined steps
+        mma_pipe<0, QF>(raw, dec, lds, a_frag0, acc, af, bf);
+    } else {
+        mma_step<0, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<1, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<2, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<3, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<4, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<5, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<6, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<7, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+    }
 }
 
 template <class QF, int MODE>
