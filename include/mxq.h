@@ -147,6 +147,12 @@ int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uin
 int mx_gemm_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M,
                      uint32_t K, uint32_t N);
+/* Q6_K and AoS Q8_0 weights through the same kernel:
+ *   gemm_q6_K_xmx / gemm_q6_K   include/ie/ops.hpp (gemm_q6_K_xmx), src/ops/gemm_q4k_xmx.cpp:284-387, src/ops/gemv_q6k.cpp:655-748
+ *   dequant_q6_K_to_Bt / dequant_q8_0_to_Bt + gemm_fp16   src/ops/dequant_kernels.cpp:392-431,611-632
+ * K % 256 == 0 (Q6_K), K % 128 == 0 (Q8_0); W is the GGUF block stream, 2-byte aligned.  */
+int mx_gemm_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 /* Expert-grouped GEMM over expert-sorted fp16 rows (Q8_0 SoA expert banks): the matrix-core
  * form of moe_prefill_gate_up_silu_q8 / moe_prefill_down_q8 (include/ie/moe_q8.hpp:51-72) for
  * fp16 activations — same arguments except that the activation rows are fp16 instead of
@@ -161,6 +167,23 @@ int mx_moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x_packed, const i
 int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
                         uint64_t d_stride, const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed,
                         uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+/* The same for AoS K-quant expert banks (expert e at W + e*expert_stride_bytes, include/ie/ops.hpp:1027-1029):
+ *   moe_prefill_gate_up_silu_q4k (fp16 x_packed) / _q4k_xmx   include/ie/ops.hpp:922-929, src/ops/moe_fused.cpp:727-901,
+ *                                                             src/ops/gemm_q4k_xmx.cpp:662-847
+ *   moe_prefill_down_packed_q4k / _q6k (and _v2)              include/ie/ops.hpp:968-983, src/ops/moe_fused.cpp:1090-1572
+ * sorted_w may be NULL: the rows are then written unweighted, as the reference's packed down
+ * kernels do (the weights are applied by moe_prefill_reduce); with sorted_w the product
+ * half(sorted_w[row] * acc) is folded into the store.  H % 256 == 0 and E_ffn % 256 == 0;
+ * the reference's `soa` flag (per-expert SoA views) is not taken: AoS banks only.  */
+int mx_moe_gemm_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x_packed, const void* gate_W, const void* up_W,
+                                 const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                                 uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
+                         const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                         uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
+                         const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                         uint64_t expert_stride_bytes, uint32_t total_rows);
 
 /* ---------------------------------------------------------------- MoE, expert-indexed GEMV
  * Q8_0-expert decode kernels (device-resident routing: the expert of token slot

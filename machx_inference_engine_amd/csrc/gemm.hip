@@ -23,7 +23,7 @@
 //               trip and no redundant dequantisation inside a workgroup.
 // The k order inside a chunk is (lanes 0-31: 8s.., lanes 32-63: 64+8s..); the
 // A fragments are read from LDS with the same order, so the products pair up.
-#include "mxq_device.h"
+#include "mxq_formats.h"
 #include "mxq_host.h"
 
 namespace mxq {
@@ -90,6 +90,8 @@ struct GemmQ4K {
         float d1[2], c1[2];
     };
     static constexpr uint32_t K_ALIGN = 256;
+    static constexpr uint32_t H_COL = 8;                                   // 16-byte A column of lane half h at step 0
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)S; }   // A column offset of step S
     __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
         const uint8_t* blk = w.base + (size_t)n * w.row_bytes + (size_t)(kc >> 1) * kQ4KBytes;
         const uint4* q = reinterpret_cast<const uint4*>(blk + 16 + (2u * (kc & 1u) + h) * 32u);
@@ -154,6 +156,8 @@ struct GemmQ8Soa {
         float d[2], o[2];
     };
     static constexpr uint32_t K_ALIGN = 128;
+    static constexpr uint32_t H_COL = 8;
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)S; }
     __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
         const uint4* p = reinterpret_cast<const uint4*>(w.qs + (size_t)n * w.K + (size_t)kc * 128u + 64u * h);
         Raw r;
@@ -188,6 +192,150 @@ struct GemmQ8Soa {
     }
 };
 
+// Q8_0 AoS GGUF blocks (34 B: fp16 d, 32 int8): lane half h owns blocks 4 kc + 2h and + 1, 68
+// contiguous bytes at a 2-byte aligned address, fetched as 17 dwords.  The quants of the first
+// block start 2 bytes into a dword and are realigned with one byte-align per word; those of
+// the second block (byte 36) are dword aligned.  Same arithmetic as the SoA planes.
+struct GemmQ8Aos {
+    struct W {
+        const uint8_t* base;
+        uint32_t row_bytes;
+    };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
+    struct Raw {
+        uint32_t w[17];
+    };
+    struct Dec {
+        float d[2], o[2];
+    };
+    static constexpr uint32_t K_ALIGN = 128;
+    static constexpr uint32_t H_COL = 8;
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)S; }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
+        const uint8_t* p = w.base + (size_t)n * w.row_bytes + (size_t)(4u * kc + 2u * h) * kQ8_0Bytes;
+        Raw r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint4 v = load_u4_a2(p + 16 * i);
+            r.w[4 * i] = v.x; r.w[4 * i + 1] = v.y; r.w[4 * i + 2] = v.z; r.w[4 * i + 3] = v.w;
+        }
+        r.w[16] = load_u1_a2(p + 64);
+        return r;
+    }
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t, uint32_t) {
+        Dec o;
+        o.d[0] = h2f(r.w[0] & 0xFFFFu);
+        o.d[1] = h2f(r.w[8] >> 16);
+        o.o[0] = -128.f * o.d[0];
+        o.o[1] = -128.f * o.d[1];
+        o.d[0] *= 16777216.f;
+        o.d[1] *= 16777216.f;
+        return o;
+    }
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int blk = S / 4, j = 2 * (S % 4) + HF;   // word j of the block's 8 quant words
+        uint32_t w;
+        if (blk == 0) w = __builtin_amdgcn_alignbyte(r.w[j + 1], r.w[j], 2);   // bytes 2 + 4j .. 5 + 4j
+        else w = r.w[9 + j];
+        w ^= 0x80808080u;
+        const float d = dc.d[blk], o = dc.o[blk];
+        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C030C02u));
+        f.u[2 * HF] = mix_pair(w01.x, w01.y, d, o);
+        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, d, o);
+    }
+    template <int S>
+    __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
+    }
+};
+
+// Q6_K (210-byte AoS blocks, 2-byte aligned): chunk kc = 128-element half c = kc%2 of block
+// kc/2.  Lane half j = lane/32 owns the 16 "l" positions 16j .. 16j+15 of that half, i.e. the
+// four 16-element groups 32s + 16j + [0,16), s = 0..3 (include/ie/dequant_ref.hpp:78-96):
+// ql[64c + 16j + ..] (groups 0 and 2 in its low / high nibbles), ql[64c + 32 + 16j + ..]
+// (groups 1 and 3), qh[32c + 16j + ..] (the 2-bit tops of all four) and the scales
+// scales[8c + 2s + j].  Step S covers group S/2, elements 8 (S%2) .. +7 of it, so the A column
+// of a step is 4 (S/2) + 2j + S%2.
+// value = half((d*sc) * (code - 32)): every product is exact in fp32; evaluated as
+// fma(code * 2^-24, d*sc * 2^24, -32 d*sc) on the 6-bit code held as an fp16 subnormal.
+struct GemmQ6K {
+    struct W {
+        const uint8_t* base;
+        uint32_t row_bytes;
+    };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
+    struct Raw {
+        uint4 qla, qlb, qh;
+        uint2 sc;
+        uint32_t d;
+    };
+    struct Dec {
+        float c[4], o[4];
+    };
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr uint32_t H_COL = 2;
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)(((S >> 1) << 2) | (S & 1)); }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t j) {
+        const uint8_t* blk = w.base + (size_t)n * w.row_bytes + (size_t)(kc >> 1) * kQ6KBytes;
+        const uint32_t c = kc & 1u;
+        Raw r;
+        r.qla = load_u4_a2(blk + 64u * c + 16u * j);
+        r.qlb = load_u4_a2(blk + 64u * c + 32u + 16u * j);
+        r.qh = load_u4_a2(blk + 128u + 32u * c + 16u * j);
+        r.sc = load_u2_a2(blk + 192u + 8u * c);
+        r.d = *reinterpret_cast<const uint16_t*>(blk + 208);
+        return r;
+    }
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t, uint32_t j) {
+        const float d = h2f(r.d);
+        const uint32_t j8 = j * 8u;
+        Dec o;
+        o.c[0] = d * (float)(int)(int8_t)(r.sc.x >> j8);
+        o.c[1] = d * (float)(int)(int8_t)(r.sc.x >> (16u + j8));
+        o.c[2] = d * (float)(int)(int8_t)(r.sc.y >> j8);
+        o.c[3] = d * (float)(int)(int8_t)(r.sc.y >> (16u + j8));
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            o.o[s] = -32.f * o.c[s];
+            o.c[s] *= 16777216.f;
+        }
+        return o;
+    }
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int s = S / 2, i = 2 * (S % 2) + HF;   // group, dword of the 16-byte slices
+        const uint32_t la = i == 0 ? r.qla.x : i == 1 ? r.qla.y : i == 2 ? r.qla.z : r.qla.w;
+        const uint32_t lb = i == 0 ? r.qlb.x : i == 1 ? r.qlb.y : i == 2 ? r.qlb.z : r.qlb.w;
+        const uint32_t qh = i == 0 ? r.qh.x : i == 1 ? r.qh.y : i == 2 ? r.qh.z : r.qh.w;
+        uint32_t code;
+        if (s == 0) code = (la & 0x0F0F0F0Fu) | ((qh << 4) & 0x30303030u);
+        else if (s == 1) code = (lb & 0x0F0F0F0Fu) | ((qh << 2) & 0x30303030u);
+        else if (s == 2) code = ((la >> 4) & 0x0F0F0F0Fu) | (qh & 0x30303030u);
+        else code = ((lb >> 4) & 0x0F0F0F0Fu) | ((qh >> 2) & 0x30303030u);
+        const float c = dc.c[s], o = dc.o[s];
+        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, code, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, code, 0x0C030C02u));
+        f.u[2 * HF] = mix_pair(w01.x, w01.y, c, o);
+        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, c, o);
+    }
+    template <int S>
+    __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
+    }
+};
+
 // ---------------------------------------------------------------- kernel
 enum { GEMM_DENSE = 0, GEMM_MOE_GATE_UP_SILU = 1, GEMM_MOE_DOWN = 2 };
 
@@ -195,7 +343,7 @@ struct GemmArgs {
     const half_t* A;                  // [M, K] fp16 (dense) or expert-sorted rows [TK, K]
     half_t* Y;                        // [M, N]
     const uint32_t* expert_offsets;   // grouped: [E+1]
-    const half_t* route_w;            // GEMM_MOE_DOWN: [TK] fp16
+    const half_t* route_w;            // GEMM_MOE_DOWN: [TK] fp16 row weights, or NULL for unweighted rows
     uint32_t M, K, N, E;
     uint32_t tiles_m, tiles_n;        // dense tile grid; grouped: tiles_m is an upper bound
 };
@@ -218,15 +366,15 @@ __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t byte_of
 
 // One K chunk = 8 MFMA steps.  A fragment (token row R, 16-byte column c) sits at
 // R * 256 + ((c ^ (R & 15)) << 4): the 16 lanes of a quarter wave then hit 16 different
-// columns, i.e. all 64 banks once.  For step S the column is 8h + S, so the address is the
-// lane's step-0 address with bits 4-6 XOR-ed by S.
+// columns, i.e. all 64 banks once.  For step S the column is QF::H_COL * h + QF::step_col(S),
+// so the address is the lane's step-0 address XOR-ed with step_col(S) << 4.
 // `mi` = number of live 32-token tiles of this workgroup tile (4 unless PARTIAL: expert-grouped
 // tiles are often mostly empty, and their dead token tiles skip both the LDS reads and the MFMAs).
 template <int S, class QF, bool PARTIAL>
 __device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
                                          float16_t (&acc)[4][2], uint32_t mi) {
     Frag af[4], bf[2];
-    const uint32_t a_s = a_frag0 ^ (uint32_t)(S << 4);
+    const uint32_t a_s = a_frag0 ^ (QF::step_col(S) << 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         if (!PARTIAL || (uint32_t)i < mi) af[i].q = *reinterpret_cast<const uint4*>(lds + a_s + i * 8192);
@@ -251,7 +399,7 @@ __device__ __forceinline__ void mma_pipe(const typename QF::Raw (&raw)[2], const
     if constexpr (S < 8) {
         constexpr int cur = S & 1, nxt = cur ^ 1, SN = (S + 1) & 7;
         constexpr bool more = S + 1 < 8;
-        const uint32_t a_n = a_frag0 ^ (uint32_t)(SN << 4);
+        const uint32_t a_n = a_frag0 ^ (QF::step_col(SN) << 4);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[cur][0].v, acc[i][0], 0, 0, 0);
@@ -381,7 +529,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds_raw;
     const uint32_t a_dst = lds_base + wave * 8192u;   // this wave's 32 rows inside an A buffer
     // step-0 fragment address of this lane inside an A buffer
-    const uint32_t frag0 = r * 256u + (((8u * h) ^ (r & 15u)) << 4);
+    const uint32_t frag0 = r * 256u + (((QF::H_COL * h) ^ (r & 15u)) << 4);
 
     float16_t acc[4][2];
 #pragma unroll
@@ -445,7 +593,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
                     const uint32_t n = n_base + 32 * j + r;
                     if (n >= g.N) continue;
                     float o = acc[i][j][v];
-                    if (MODE == GEMM_MOE_DOWN) o *= (float)g.route_w[row];
+                    if (MODE == GEMM_MOE_DOWN && g.route_w) o *= (float)g.route_w[row];
                     g.Y[(size_t)row * g.N + n] = (half_t)o;
                 }
             }
@@ -475,14 +623,31 @@ static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typenam
     return launch_status();
 }
 
-static int check_gemm(const void* A, const void* W, const void* y, uint32_t M, uint32_t K, uint32_t N, uint32_t k_align) {
+static int check_gemm(const void* A, const void* W, const void* y, uint32_t M, uint32_t K, uint32_t N, uint32_t k_align, uint32_t w_align = 16) {
     MX_REQUIRE_PTR(A);
     MX_REQUIRE_PTR(W);
     MX_REQUIRE_PTR(y);
-    MX_REQUIRE_SHAPE(M > 0 && N > 0 && K > 0 && K % k_align == 0);
+    MX_REQUIRE_SHAPE(M > 0 && N > 0 && K > 0 && K % k_align == 0 && K <= (1u << 22));   // a 128-row A tile is addressed with 32-bit byte offsets
     MX_REQUIRE_ALIGN(A, 16);
-    MX_REQUIRE_ALIGN(W, 16);
+    MX_REQUIRE_ALIGN(W, w_align);
     return MX_OK;
+}
+
+// AoS expert bank entry points (Q4_K, Q6_K): shared argument checks and GemmArgs
+template <class QF, int MODE>
+static int moe_gemm_aos(mx_stream_t s, const uint16_t* rows, const void* W0, const void* W1, uint64_t expert_stride_bytes, const uint32_t* expert_offsets,
+                        const uint16_t* sorted_w, uint16_t* out, uint32_t E, uint32_t K, uint32_t N, uint32_t total_rows, uint32_t block_bytes,
+                        uint32_t w_align) {
+    if (int rc = check_gemm(rows, W0, out, total_rows, K, N, 256, w_align)) return rc;
+    MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(E > 0 && expert_stride_bytes % w_align == 0);
+    MX_REQUIRE_ALIGN(W1, w_align);
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(rows); g.Y = reinterpret_cast<half_t*>(out); g.expert_offsets = expert_offsets;
+    g.route_w = reinterpret_cast<const half_t*>(sorted_w); g.M = total_rows; g.K = K; g.N = N; g.E = E;
+    const uint32_t row_bytes = K / 256 * block_bytes;
+    typename QF::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
+    return launch_gemm<QF, MODE>(s, b0, b1, g, total_rows);
 }
 
 }  // namespace mxq
@@ -497,6 +662,22 @@ int mx_gemm_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, u
     g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
     GemmQ4K::Bank b{static_cast<const uint8_t*>(W), 0, K / 256 * (uint32_t)kQ4KBytes};
     return launch_gemm<GemmQ4K, GEMM_DENSE>(s, b, b, g, M);
+}
+
+int mx_gemm_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    if (int rc = check_gemm(A, W, y, M, K, N, 256, 2)) return rc;
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
+    GemmQ6K::Bank b{static_cast<const uint8_t*>(W), 0, K / 256 * (uint32_t)kQ6KBytes};
+    return launch_gemm<GemmQ6K, GEMM_DENSE>(s, b, b, g, M);
+}
+
+int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    if (int rc = check_gemm(A, W, y, M, K, N, 128, 2)) return rc;
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
+    GemmQ8Aos::Bank b{static_cast<const uint8_t*>(W), 0, K / 32 * (uint32_t)kQ8_0Bytes};
+    return launch_gemm<GemmQ8Aos, GEMM_DENSE>(s, b, b, g, M);
 }
 
 int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
@@ -537,13 +718,22 @@ int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d
     return launch_gemm<GemmQ8Soa, GEMM_MOE_DOWN>(s, b, b, g, total_rows);
 }
 
-}  // extern "C"
-
-// Resident workgroups per CU of the dense Q4_K GEMM kernel at its launch configuration
-// (diagnostic; negative = HIP error).
-extern "C" int mx_debug_gemm_occupancy(void) {
-    int n = 0;
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mxq::gemm_kernel<mxq::GemmQ4K, mxq::GEMM_DENSE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)mxq::kGemmLds);
-    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mxq::gemm_kernel<mxq::GemmQ4K, mxq::GEMM_DENSE>, mxq::kGemmThreads, mxq::kGemmLds);
-    return e == hipSuccess ? n : -(int)e;
+int mx_moe_gemm_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
+                                 uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_gemm_aos<GemmQ4K, GEMM_MOE_GATE_UP_SILU>(s, x_packed, gate_W, up_W, expert_stride_bytes, expert_offsets, nullptr, h_packed, E, H, E_ffn,
+                                                        total_rows, kQ4KBytes, 16);
 }
+
+int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const uint16_t* sorted_w,
+                         uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_gemm_aos<GemmQ4K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
+                                                total_rows, kQ4KBytes, 16);
+}
+
+int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const uint16_t* sorted_w,
+                         uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_gemm_aos<GemmQ6K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
+                                                total_rows, kQ6KBytes, 2);
+}
+
+}  // extern "C"

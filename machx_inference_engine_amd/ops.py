@@ -286,6 +286,33 @@ def gemm_q4_K(A, W, M, K, N, y=None):
     return y
 
 
+def gemm_q6_K(A, W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_q6_K", _f16(A), _u8(W), _ptr(y), M, K, N)
+    return y
+
+
+def gemm_q8_0(A, W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_q8_0", _f16(A), _u8(W), _ptr(y), M, K, N)
+    return y
+
+
+def moe_gemm_gate_up_silu_q4k(x_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None):
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
+    _call("mx_moe_gemm_gate_up_silu_q4k", _f16(x_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
+          expert_stride_bytes, TK)
+    return h_packed
+
+
+def moe_gemm_down_kquant(fmt, h_packed, down_W, expert_offsets, sorted_w, TK, E, H, E_ffn, expert_stride_bytes, out_packed=None):
+    """fmt in ('q4k', 'q6k'); sorted_w None -> unweighted packed rows."""
+    out_packed = _out(out_packed, (TK, H), torch.float16, h_packed)
+    _call("mx_moe_gemm_down_%s" % fmt, _f16(h_packed), _u8(down_W), _ptr(expert_offsets), _f16(sorted_w) if sorted_w is not None else None,
+          _ptr(out_packed), E, H, E_ffn, expert_stride_bytes, TK)
+    return out_packed
+
+
 def gemm_q8_0_soa(A, qs_W, d_W, M, K, N, y=None):
     y = _out(y, (M, N), torch.float16, A)
     _call("mx_gemm_q8_0_soa", _f16(A), _u8(qs_W), _ptr(d_W), _ptr(y), M, K, N)

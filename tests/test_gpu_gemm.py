@@ -41,6 +41,57 @@ def test_gemm_q8_0_soa(mx, M, K, N):
     check(got, ref, "gemm_q8_0_soa M=%d K=%d N=%d" % (M, K, N))
 
 
+def onehot_weights_through_gemm(gemm, K, N):
+    """A = rows of the identity: Y[t, n] is the kernel's own fp16 weight W16[n, k0 + t]."""
+    out = np.zeros((N, K), np.float32)
+    for k0 in range(0, K, 128):
+        A = np.zeros((128, K), np.float32)
+        A[np.arange(128), k0 + np.arange(128)] = 1.0
+        out[:, k0:k0 + 128] = host(gemm(dev(A).half())).astype(np.float32).T
+    return out
+
+
+@pytest.mark.parametrize("fmt,K", [("q4_K", 512), ("q6_K", 512), ("q8_0", 256)])
+def test_gemm_weight_fragments_bit_exact(mx, fmt, K):
+    """The fp16 weights the GEMM multiplies by equal half(reference dequant) element for element
+    (include/ie/dequant_ref.hpp), read back through one-hot activations."""
+    F = {"q4_K": O.Q4_K, "q6_K": O.Q6_K, "q8_0": O.Q8_0}[fmt]
+    N = 256
+    W = weights(F, 2300, N, K)
+    ref = f16(O.dequant(F, W, N * K).reshape(N, K))
+    fn = {"q4_K": mx.ops.gemm_q4_K, "q6_K": mx.ops.gemm_q6_K, "q8_0": mx.ops.gemm_q8_0}[fmt]
+    got = onehot_weights_through_gemm(lambda A: fn(A, dev(W), 128, K, N), K, N)
+    # value equality: a zero weight may come out as +0 where the reference expression gives -0
+    # (Q6_K code 32 under a negative scale); the sign of a zero cannot change a dot product
+    n_bad = int((got != ref.astype(np.float32)).sum())
+    assert n_bad == 0, "%d of %d weights differ" % (n_bad, got.size)
+    if fmt == "q8_0":
+        qs, d = O.repack_q8_0_to_soa(W)
+        got = onehot_weights_through_gemm(lambda A: mx.ops.gemm_q8_0_soa(A, dev(qs), dev(d), 128, K, N), K, N)
+        assert np.array_equal(got, ref.astype(np.float32))
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 256, 256), (1, 512, 64), (300, 1024, 520), (129, 768, 33), (512, 4096, 1024)])
+def test_gemm_q6_K(mx, M, K, N):
+    W = weights(O.Q6_K, 2200 + N, N, K)
+    A = f16(O.normal(2201 + M, (M, K)))
+    ref = O.gemv_f64(O.Q6_K, W, A, K, N, round_w_fp16=True)
+    got = host(mx.ops.gemm_q6_K(dev(A).half(), dev(W), M, K, N)).astype(np.float32)
+    check(got, ref, "gemm_q6_K M=%d K=%d N=%d" % (M, K, N))
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 128, 256), (260, 768, 2048), (77, 2048, 768)])
+def test_gemm_q8_0_aos(mx, M, K, N):
+    W = weights(O.Q8_0, 2100 + N, N, K)
+    A = f16(O.normal(2101 + M, (M, K)))
+    ref = O.gemv_f64(O.Q8_0, W, A, K, N, round_w_fp16=True)
+    got = host(mx.ops.gemm_q8_0(dev(A).half(), dev(W), M, K, N)).astype(np.float32)
+    check(got, ref, "gemm_q8_0 M=%d K=%d N=%d" % (M, K, N))
+    qs, d = O.repack_q8_0_to_soa(W)
+    soa = host(mx.ops.gemm_q8_0_soa(dev(A).half(), dev(qs), dev(d), M, K, N)).astype(np.float32)
+    assert np.array_equal(got, soa), "AoS and SoA entry points multiply the same fp16 weights in the same order"
+
+
 def test_gemm_rejects_bad_shapes(mx):
     A = torch.zeros((4, 300), dtype=torch.float16, device="cuda")
     W = torch.zeros(1024, dtype=torch.uint8, device="cuda")
@@ -104,3 +155,45 @@ def test_moe_grouped_gemm_q8(mx, T, E, Kt, H, EF):
     hq = ops.moe_prefill_gate_up_silu_q8(ops.quantize_q8_1(xp), dev(gq), dev(gd), dev(uq), dev(ud), EF * H, EF * H // 32, dev(off), TK, E, H, EF)
     a, b = host(hq).astype(np.float64), hp_h.astype(np.float64)
     assert np.abs(a - b).max() / np.sqrt(np.mean(b * b)) < 0.2   # q8 activation noise through silu(g)*u
+
+
+@pytest.mark.parametrize("T,E,Kt,H,EF", [(64, 8, 2, 256, 256), (300, 16, 4, 512, 256)])
+def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
+    """Q4_K gate/up + Q4_K or Q6_K down expert banks (AoS, expert-major) through the grouped GEMM
+    (moe_prefill_gate_up_silu_q4k, moe_prefill_down_packed_q4k/_q6k, include/ie/ops.hpp:922-983)."""
+    ops = mx.ops
+    mk = lambda F, seed, N, K: np.stack([O.quantize(F, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
+    Wg, Wu = mk(O.Q4_K, 3100, EF, H), mk(O.Q4_K, 4100, EF, H)
+    x = f16(O.normal(6100, (T, H)))
+    ids, w = zipf_routing(7100, T, E, Kt)
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    TK = T * Kt
+    counts = np.diff(off.astype(np.int64))
+    xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
+    stride_gu = Wg[0].size
+    hp = ops.moe_gemm_gate_up_silu_q4k(xp, dev(Wg), dev(Wu), dev(off), TK, E, H, EF, stride_gu)
+    hp_h = host(hp).astype(np.float32)
+    xs = x[si]
+    h_ref = np.zeros((TK, EF), np.float32)
+    for e in range(E):
+        if counts[e]:
+            rows = slice(off[e], off[e + 1])
+            g = O.gemv_f64(O.Q4_K, Wg[e], xs[rows], H, EF, round_w_fp16=True)
+            u = O.gemv_f64(O.Q4_K, Wu[e], xs[rows], H, EF, round_w_fp16=True)
+            h_ref[rows] = O.swiglu_np(g.astype(np.float32), u.astype(np.float32))
+    check(hp_h, h_ref, "moe grouped gate_up silu q4k (MFMA)")
+    for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
+        Wd = mk(F, 5100, H, EF)
+        o_ref = np.zeros((TK, H), np.float64)
+        for e in range(E):
+            if counts[e]:
+                rows = slice(off[e], off[e + 1])
+                o_ref[rows] = O.gemv_f64(F, Wd[e], hp_h[rows], EF, H, round_w_fp16=True)
+        op = ops.moe_gemm_down_kquant(fmt, hp, dev(Wd), dev(off), None, TK, E, H, EF, Wd[0].size)
+        check(host(op).astype(np.float32), o_ref, "moe grouped down %s unweighted (MFMA)" % fmt)
+        opw = ops.moe_gemm_down_kquant(fmt, hp, dev(Wd), dev(off), dev(wp).half(), TK, E, H, EF, Wd[0].size)
+        check(host(opw).astype(np.float32), o_ref * f16(wp)[:, None], "moe grouped down %s weighted (MFMA)" % fmt)
+        # unweighted rows + moe_prefill_reduce (weights applied there) == the reference's two-step path
+        y = ops.moe_prefill_reduce(op, dev(t2p.astype(np.uint32)), dev(wp).half(), torch.zeros((T, H), dtype=torch.float16, device="cuda"), T, Kt, H)
+        y_ref = (host(op).astype(np.float32) * f16(wp)[:, None])[t2p].reshape(T, Kt, H).sum(axis=1)
+        check(host(y).astype(np.float32), y_ref, "prefill_reduce over %s rows" % fmt, max_rel=2e-3)
