@@ -201,6 +201,24 @@ int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const ui
                    uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
                    uint32_t K, uint32_t E_ffn, uint32_t H);
 int mx_moe_reduce_q8(mx_stream_t s, const uint16_t* y_packed, uint16_t* y, uint32_t T, uint32_t K, uint32_t H);
+/* K-quant (AoS, expert-major) expert banks with fp16 activations, decode — the reference's fused
+ * Q4_K / Q6_K expert kernels; fp32 fold acc += (d*sc)*sum(a*q) - (dmin*m)*sum(a):
+ *   moe_decode_gate_up_silu_q4k  include/ie/ops.hpp:1034-1041, src/ops/moe_fused.cpp:82-211
+ *     h_out[t*K_top + k, n] = half(silu(gate_e . x_t) * (up_e . x_t)),  e = topk_idx[t*K_top + k]
+ *   moe_decode_down_q4k / _q6k   include/ie/ops.hpp:1078-1095, src/ops/moe_fused.cpp:224-330,352-522
+ *     y_out[t, n] = half(sum_k topk_w[t*K_top + k] * (down_e . h[t*K_top + k])); written, not accumulated
+ * The reference signatures are single-token; T (last argument) generalises them to T tokens per
+ * launch, T = 1 being the reference call.  H % 256 == 0, E_ffn % 256 == 0; the `soa` flag of the
+ * reference (per-expert SoA views) is not taken: AoS banks only.  */
+int mx_moe_decode_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x, const void* gate_W, const void* up_W,
+                                   const int32_t* topk_idx, uint16_t* h_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
+                                   uint64_t expert_stride_bytes, uint32_t T);
+int mx_moe_decode_down_q4k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx,
+                           const uint16_t* topk_w, uint16_t* y_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
+                           uint64_t expert_stride_bytes, uint32_t T);
+int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx,
+                           const uint16_t* topk_w, uint16_t* y_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
+                           uint64_t expert_stride_bytes, uint32_t T);
 /* Expert-grouped form: activation rows are expert-sorted and partitioned by
  * expert_offsets[E+1]; each expert's weights are streamed once per tile of rows;
  * experts without rows cost nothing (src/ops/moe_q8.cpp:211).

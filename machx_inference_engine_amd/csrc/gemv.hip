@@ -71,12 +71,6 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
 // ---------------------------------------------------------------- float activations (T = 1)
 // Same unit walk; activations staged as fp32 plus per-16 sums; the fold is the
 // reference's acc += (d*sc) * sum(a*q) - (dmin*m) * sum(a)  (src/ops/gemv_q4k.cpp:119-146).
-template <bool UNSIGNED>
-__device__ __forceinline__ float code_to_f(uint32_t w, int j) {
-    if (UNSIGNED) return (float)((w >> (8 * j)) & 0xFFu);
-    return (float)(int)(int8_t)(w >> (8 * j));
-}
-
 template <class F, int R, int G, class ActT, class OutT>
 __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w, const ActT* A, OutT* y, uint32_t K, uint32_t N, uint32_t KT) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -98,16 +92,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
             const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
             if (n_tiles > 1 || !staged) {
                 __syncthreads();
-                for (uint32_t i = threadIdx.x; i < (kt + 63) / 64 * 4; i += blockDim.x) {
-                    float s = 0.f;
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        const float v = (i * 16 < kt) ? load_act(A + k0 + i * 16 + j) : 0.f;
-                        xa[i * 16 + j] = v;
-                        s += v;
-                    }
-                    s16[i] = s;
-                }
+                stage_fact(xa, s16, A + k0, kt);
                 __syncthreads();
                 staged = true;
             }
@@ -123,23 +108,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
                 for (int r = 0; r < R; ++r) raw[r] = load_unit<F, G>(cu[r], it, half_tail && ul == n_units - 1);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    Unit un;
-                    F::decode(raw[r], cu[r], un);
-                    float v = 0.f;
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const uint32_t eg = e0 + g * F::GROUP_OFF;
-                        float dq = 0.f;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float4 x = *reinterpret_cast<const float4*>(xa + eg + 4 * i);
-                            dq += x.x * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 0) + x.y * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 1) +
-                                  x.z * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 2) + x.w * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 3);
-                        }
-                        v += un.c[g] * dq;
-                        if (F::SUM_GRAN != 0) v -= un.m[g] * s16[eg >> 4];
-                    }
-                    acc[r] += v;
+                    acc[r] += fact_unit<F>(raw[r], cu[r], xa, s16, e0);
                 }
             }
         }

@@ -124,6 +124,83 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
     }
 }
 
+// ---------------------------------------------------------------- fp16-activation decode (K-quant expert banks)
+// The reference's decode kernels for Q4_K / Q6_K experts take fp16 activations and fold in fp32
+// (src/ops/moe_fused.cpp:82-211, 224-330, 352-522).  Same unit walk as the float-activation GEMV.
+//   FACT_GATE_UP: grid (x, slot tk): h_out[tk, n] = half(silu(gate_e . x_t) * (up_e . x_t)), t = tk / K_top
+//   FACT_DOWN   : grid (x, token t): y[t, n] = half(sum_k w[t,k] * (down_e(t,k) . h[t*K_top + k])),
+//                 the K_top products summed in fp32 before the single rounding (moe_fused.cpp:268-318);
+//                 all K_top activation rows of the token are staged side by side.
+enum { FACT_GATE_UP = 0, FACT_DOWN = 1 };
+
+struct MoeFactArgs {
+    const half_t* act;          // gate/up: x [T, K]; down: h [T*K_top, K]
+    const int32_t* topk_idx;    // [T*K_top]
+    const half_t* topk_w;       // down: [T*K_top]
+    half_t* out;                // gate/up: [T*K_top, N]; down: [T, N]
+    uint32_t K, N, KT, K_top;
+};
+
+template <class F, int G, int MODE>
+__global__ __launch_bounds__(kGemvThreads) void moe_fact_kernel(typename F::Bank bank0, typename F::Bank bank1, MoeFactArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS;
+    constexpr int NW = (MODE == FACT_GATE_UP) ? 2 : 1;
+    const uint32_t K = a.K, N = a.N, KT = a.KT;
+    const uint32_t n_act = (MODE == FACT_DOWN) ? a.K_top : 1u;   // activation rows staged together
+    float* xa = reinterpret_cast<float*>(lds);                    // [n_act][KT]
+    float* s16 = xa + (size_t)n_act * KT;                         // [n_act][KT/16]
+    const uint32_t seg = blockIdx.y;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    const uint32_t n_tiles = (K + KT - 1) / KT;
+    const half_t* act0 = (MODE == FACT_DOWN) ? a.act + (size_t)seg * a.K_top * K : a.act + (size_t)(seg / a.K_top) * K;
+    bool staged = false;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
+        const uint32_t n0 = rg * ROWS_PER_WG + wave * GROUPS + grp;
+        const uint32_t n = n0 < N ? n0 : N - 1;
+        float tot0 = 0.f, tot1 = 0.f;
+        for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+            const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
+            if (n_tiles > 1 || !staged) {
+                __syncthreads();
+                for (uint32_t j = 0; j < n_act; ++j) stage_fact(xa + (size_t)j * KT, s16 + (size_t)j * (KT / 16), act0 + (size_t)j * K + k0, kt);
+                __syncthreads();
+                staged = true;
+            }
+            const uint32_t n_units = (kt + 63) / 64;
+            const bool half_tail = (kt & 63u) != 0;
+            for (uint32_t j = 0; j < n_act; ++j) {
+                const uint32_t slot = (MODE == FACT_DOWN) ? seg * a.K_top + j : seg;
+                const uint32_t e = (uint32_t)a.topk_idx[slot];
+                const typename F::W w0 = F::expert(bank0, e), w1 = F::expert(NW == 2 ? bank1 : bank0, e);
+                typename F::Cursor c0 = F::cursor(w0, n, k0 / 64 + gl), c1 = F::cursor(w1, n, k0 / 64 + gl);
+                const float* xj = xa + (size_t)j * KT;
+                const float* sj = s16 + (size_t)j * (KT / 16);
+                float acc0 = 0.f, acc1 = 0.f;
+                for (uint32_t it = 0; it * G + gl < n_units; ++it) {
+                    const uint32_t ul = it * G + gl, e0 = F::elem_off(ul);
+                    const bool tail = half_tail && ul == n_units - 1;
+                    const typename F::Raw r0 = load_unit<F, G>(c0, it, tail);
+                    if (NW == 2) {
+                        const typename F::Raw r1 = load_unit<F, G>(c1, it, tail);
+                        acc1 += fact_unit<F>(r1, c1, xj, sj, e0);
+                    }
+                    acc0 += fact_unit<F>(r0, c0, xj, sj, e0);
+                }
+                if (MODE == FACT_DOWN) tot0 += (float)a.topk_w[slot] * acc0;
+                else { tot0 += acc0; tot1 += acc1; }
+            }
+        }
+        const float v0 = group_sum<G>(tot0);
+        const float v1 = (NW == 2) ? group_sum<G>(tot1) : 0.f;
+        if (lane == (uint32_t)group_sum_lane<G>(lane) && n0 < N)
+            a.out[(size_t)seg * N + n0] = (half_t)((MODE == FACT_GATE_UP) ? silu_mul(v0, v1) : v0);
+    }
+}
+
 // ---------------------------------------------------------------- row utilities
 // moe_gather_rows (src/ops/moe.cpp:262-282): y_packed[i] = x[indices[i]]
 __global__ __launch_bounds__(256) void gather_rows_kernel(const half_t* x, const int32_t* idx, half_t* y, uint32_t n_rows, uint32_t hidden) {
@@ -167,6 +244,7 @@ static int cu_count_moe() {
     return n;
 }
 constexpr uint32_t kMoeLdsBudget = 48 * 1024;
+constexpr uint32_t kMoeFactLds = 60 * 1024;   // staged fp32 activations of the fp16-activation decode kernels
 
 static uint32_t pick_group_moe(uint32_t units) {
     uint32_t best = 64, waste = (units + 63) / 64 * 64 - units;
@@ -214,6 +292,49 @@ static int launch_moe(mx_stream_t s, const typename F::Bank& b0, const typename 
 // rows per token tile in grouped mode: expected rows per expert, rounded up to 4 or 8
 static uint32_t grouped_tt(uint64_t total_rows, uint32_t E) { return (total_rows <= 4ull * E) ? 4 : 8; }
 
+template <class F, int MODE>
+static int launch_moe_fact(mx_stream_t s, const typename F::Bank& b0, const typename F::Bank& b1, MoeFactArgs a, uint32_t n_seg) {
+    const uint32_t n_act = (MODE == FACT_DOWN) ? a.K_top : 1u;
+    const uint32_t K256 = (a.K + 255) / 256 * 256;
+    uint32_t KT = K256;                                           // whole rows if they fit, else balanced K tiles
+    const uint32_t kt_max = (kMoeFactLds / (n_act * 17u)) * 4u / 256u * 256u;   // 4.25 bytes per staged element
+    if (kt_max == 0) return MX_ERR_SHAPE;
+    if (KT > kt_max) {
+        const uint32_t n_tiles = (K256 + kt_max - 1) / kt_max;
+        KT = (K256 / 256 + n_tiles - 1) / n_tiles * 256;
+    }
+    a.KT = KT;
+    const uint32_t lds = n_act * (KT * 4 + KT / 16 * 4);
+    const uint32_t G = pick_group_moe((a.K + 63) / 64);
+    const uint32_t rows_per_wg = kGemvWaves * (64 / G);
+    const uint32_t n_rg = (a.N + rows_per_wg - 1) / rows_per_wg;
+    uint32_t gx = (uint32_t)cu_count_moe() * 8 / n_seg;
+    if (gx < 1) gx = 1;
+    if (gx > n_rg) gx = n_rg;
+    if (n_seg > 65535) return MX_ERR_SHAPE;
+    hipStream_t st = as_stream(s);
+    if (G == 16) hipLaunchKernelGGL((moe_fact_kernel<F, 16, MODE>), dim3(gx, n_seg), dim3(kGemvThreads), lds, st, b0, b1, a);
+    else if (G == 32) hipLaunchKernelGGL((moe_fact_kernel<F, 32, MODE>), dim3(gx, n_seg), dim3(kGemvThreads), lds, st, b0, b1, a);
+    else hipLaunchKernelGGL((moe_fact_kernel<F, 64, MODE>), dim3(gx, n_seg), dim3(kGemvThreads), lds, st, b0, b1, a);
+    return launch_status();
+}
+
+template <class F, int MODE>
+static int moe_decode_fact(mx_stream_t s, const uint16_t* act, const void* W0, const void* W1, const int32_t* topk_idx, const uint16_t* topk_w,
+                           uint16_t* out, uint32_t K, uint32_t N, uint32_t K_top, uint32_t T, uint64_t expert_stride_bytes, uint32_t block_bytes,
+                           uint32_t w_align) {
+    MX_REQUIRE_PTR(act); MX_REQUIRE_PTR(W0); MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(out);
+    if (MODE == FACT_DOWN) MX_REQUIRE_PTR(topk_w);
+    MX_REQUIRE_SHAPE(K > 0 && N > 0 && K % 256 == 0 && K_top > 0 && T > 0 && expert_stride_bytes % w_align == 0);
+    MX_REQUIRE_ALIGN(W0, w_align); MX_REQUIRE_ALIGN(W1, w_align);
+    MoeFactArgs a{};
+    a.act = reinterpret_cast<const half_t*>(act); a.topk_idx = topk_idx; a.topk_w = reinterpret_cast<const half_t*>(topk_w);
+    a.out = reinterpret_cast<half_t*>(out); a.K = K; a.N = N; a.K_top = K_top;
+    const uint32_t row_bytes = K / 256 * block_bytes;
+    typename F::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
+    return launch_moe_fact<F, MODE>(s, b0, b1, a, MODE == FACT_DOWN ? T : T * K_top);
+}
+
 static int check_moe(const void* x, const void* out, uint32_t K, uint32_t N, uint32_t n_seg) {
     MX_REQUIRE_PTR(x);
     MX_REQUIRE_PTR(out);
@@ -255,6 +376,19 @@ int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const ui
     a.out = reinterpret_cast<half_t*>(y_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
     FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
     return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, T * K, 1);
+}
+// ------------------------------------------------------------ K-quant AoS experts, fp16 activations, decode
+int mx_moe_decode_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x, const void* gate_W, const void* up_W, const int32_t* topk_idx, uint16_t* h_out,
+                                   uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
+    return moe_decode_fact<FmtQ4K, FACT_GATE_UP>(s, x, gate_W, up_W, topk_idx, nullptr, h_out, H, E_ffn, K_top, T, expert_stride_bytes, kQ4KBytes, 16);
+}
+int mx_moe_decode_down_q4k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_out,
+                           uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
+    return moe_decode_fact<FmtQ4K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes, kQ4KBytes, 16);
+}
+int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_out,
+                           uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
+    return moe_decode_fact<FmtQ6K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes, kQ6KBytes, 2);
 }
 // ------------------------------------------------------------ Q8_0 SoA experts, grouped rows, int-dot GEMV form
 static int moe_grouped_gate_up_silu_q8_gemv(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,

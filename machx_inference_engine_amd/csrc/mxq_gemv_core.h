@@ -161,4 +161,49 @@ __device__ __forceinline__ void gemv_rows(const typename F::Cursor (&cu)[R], uin
     }
 }
 
+// ---------------------------------------------------------------- float activations
+// Activations staged in LDS as fp32 plus per-16 sums; one unit folds as the reference's
+//   acc += (d*sc) * sum(a*q) - (dmin*m) * sum(a)      (src/ops/gemv_q4k.cpp:119-146).
+template <bool UNSIGNED>
+__device__ __forceinline__ float code_to_f(uint32_t w, int j) {
+    if (UNSIGNED) return (float)((w >> (8 * j)) & 0xFFu);
+    return (float)(int)(int8_t)(w >> (8 * j));
+}
+
+// kt activations from A (zero up to the next multiple of 64) -> xa[], sums of 16 -> s16[]
+template <class ActT>
+__device__ __forceinline__ void stage_fact(float* xa, float* s16, const ActT* A, uint32_t kt) {
+    for (uint32_t i = threadIdx.x; i < (kt + 63) / 64 * 4; i += blockDim.x) {
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float v = (i * 16 < kt) ? load_act(A + i * 16 + j) : 0.f;
+            xa[i * 16 + j] = v;
+            s += v;
+        }
+        s16[i] = s;
+    }
+}
+
+template <class F>
+__device__ __forceinline__ float fact_unit(const typename F::Raw& raw, const typename F::Cursor& cu, const float* xa, const float* s16, uint32_t e0) {
+    Unit un;
+    F::decode(raw, cu, un);
+    float v = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t eg = e0 + g * F::GROUP_OFF;
+        float dq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 x = *reinterpret_cast<const float4*>(xa + eg + 4 * i);
+            dq += x.x * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 0) + x.y * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 1) +
+                  x.z * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 2) + x.w * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 3);
+        }
+        v += un.c[g] * dq;
+        if (F::SUM_GRAN != 0) v -= un.m[g] * s16[eg >> 4];
+    }
+    return v;
+}
+
 }  // namespace mxq

@@ -229,6 +229,19 @@ def moe_prefill_reduce(out_packed, tk_to_packed, weights_packed, y, T, K_top, H)
     return y
 
 
+def moe_decode_gate_up_silu_q4k(x, gate_W, up_W, topk_idx, H, E_ffn, K_top, expert_stride_bytes, T=1, h_out=None):
+    h_out = _out(h_out, (T * K_top, E_ffn), torch.float16, x)
+    _call("mx_moe_decode_gate_up_silu_q4k", _f16(x), _u8(gate_W), _u8(up_W), _ptr(topk_idx), _ptr(h_out), H, E_ffn, K_top, expert_stride_bytes, T)
+    return h_out
+
+
+def moe_decode_down_kquant(fmt, h, down_W, topk_idx, topk_w, H, E_ffn, K_top, expert_stride_bytes, T=1, y_out=None):
+    """fmt in ('q4k', 'q6k')."""
+    y_out = _out(y_out, (T, H), torch.float16, h)
+    _call("mx_moe_decode_down_%s" % fmt, _f16(h), _u8(down_W), _ptr(topk_idx), _f16(topk_w), _ptr(y_out), H, E_ffn, K_top, expert_stride_bytes, T)
+    return y_out
+
+
 def moe_gather_rows(x, indices, n_rows, hidden, y_packed=None):
     y_packed = _out(y_packed, (n_rows, hidden), torch.float16, x)
     _call("mx_moe_gather_rows", _f16(x), _ptr(indices), _ptr(y_packed), n_rows, hidden)

@@ -189,3 +189,36 @@ def test_moe_grouped_skips_empty_and_single_row_experts(mx):
                                 O.gemv_q8chain(O.Q8_0, Wu[ids[si[r], 0]], xq_h[r * rb:(r + 1) * rb], H, EF)[0].astype(np.float32))
                     for r in range(11)])
     check(host(hp).astype(np.float32), ref, "grouped with empty experts")
+
+
+@pytest.mark.parametrize("T,E,Kt,H,EF", [(1, 16, 8, 2048, 512), (3, 8, 4, 512, 768), (1, 4, 2, 256, 256)])
+def test_moe_decode_kquant_fp16_activations(mx, T, E, Kt, H, EF):
+    """moe_decode_gate_up_silu_q4k / moe_decode_down_q4k / _q6k (include/ie/ops.hpp:1034-1095): fp16
+    activations, AoS expert banks, device-resident expert ids; against the float-activation oracle,
+    expert by expert (the per-token per-expert loop of tests/unit/moe_test.cpp:62-169)."""
+    ops = mx.ops
+    mk = lambda F, seed, N, K: np.stack([O.quantize(F, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
+    Wg, Wu = mk(O.Q4_K, 8100, EF, H), mk(O.Q4_K, 8200, EF, H)
+    x = f16(O.normal(8300, (T, H)))
+    ids, w = route(8400, T, E, Kt)
+    w16 = f16(w)
+    idd = dev(ids.astype(np.int32).reshape(-1))
+    h = ops.moe_decode_gate_up_silu_q4k(dev(x).half(), dev(Wg), dev(Wu), idd, H, EF, Kt, Wg[0].size, T)
+    h_h = host(h).astype(np.float32)
+    h_ref = np.zeros((T * Kt, EF), np.float32)
+    for t in range(T):
+        for k in range(Kt):
+            e = int(ids[t, k])
+            g = O.gemv_f64(O.Q4_K, Wg[e], x[t:t + 1], H, EF)[0]
+            u = O.gemv_f64(O.Q4_K, Wu[e], x[t:t + 1], H, EF)[0]
+            h_ref[t * Kt + k] = O.swiglu_np(g.astype(np.float32), u.astype(np.float32))
+    check(h_h, h_ref, "moe decode gate_up silu q4k")
+    for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
+        Wd = mk(F, 8500, H, EF)
+        y = ops.moe_decode_down_kquant(fmt, h, dev(Wd), idd, dev(w16.reshape(-1)).half(), H, EF, Kt, Wd[0].size, T)
+        y_ref = np.zeros((T, H), np.float64)
+        for t in range(T):
+            for k in range(Kt):
+                e = int(ids[t, k])
+                y_ref[t] += float(w16[t, k]) * O.gemv_f64(F, Wd[e], h_h[t * Kt + k:t * Kt + k + 1], EF, H)[0]
+        check(host(y).astype(np.float32), y_ref, "moe decode down %s" % fmt)
