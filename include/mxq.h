@@ -263,6 +263,38 @@ int mx_moe_grouped_gate_up_oai_mxfp4(mx_stream_t s, const void* xq8_packed, cons
 int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
                               uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed,
                               uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+/* ---------------------------------------------------------------- MoE routing and packing on the device
+ *   moe_router             include/ie/ops.hpp:780-786, src/ops/moe.cpp:22-216
+ *     logits = W_gate[E,H] (fp32) . x_t, softmax, top-k, renormalise, ascending expert id; any
+ *     E <= 1024, k <= 64 (the reference handles E = 256, k = 8 only).  logits_ws: caller-owned
+ *     workspace of n_tokens*n_experts floats (the reference keeps a static per-device buffer).
+ *   moe_topk_from_logits   include/ie/ops.hpp:790-793, src/ops/moe.cpp:366-412   (fp16 logits, n_tokens rows)
+ *   moe_build_pack_decode  include/ie/ops.hpp:797-802, src/ops/moe.cpp:423-446   (one token)
+ *   mx_moe_build_packing_device: the arrays of build_moe_packing (src/model/qwen3moe_pack.cpp:5-31)
+ *     for T tokens without leaving the device: stable counting sort of the T*K slots by expert.
+ * An exact probability tie goes to the higher expert id, as in the reference.  */
+int mx_moe_router(mx_stream_t s, const uint16_t* x, const float* W_gate, int32_t* topk_idx, uint16_t* topk_w,
+                  uint32_t n_tokens, uint32_t hidden, uint32_t n_experts, uint32_t k, float* logits_ws);
+int mx_moe_topk_from_logits(mx_stream_t s, const uint16_t* logits, int32_t* topk_idx, uint16_t* topk_w, uint32_t E,
+                            uint32_t K, uint32_t n_tokens);
+int mx_moe_build_pack_decode(mx_stream_t s, const int32_t* topk_idx, const uint16_t* topk_w, uint32_t* expert_offsets,
+                             int32_t* sorted_idx, int32_t* tk_to_packed, uint16_t* weights_packed, uint32_t E, uint32_t K);
+int mx_moe_build_packing_device(mx_stream_t s, const int32_t* topk_idx, const uint16_t* topk_w, uint32_t T, uint32_t K,
+                                uint32_t E, uint32_t* expert_offsets, int32_t* sorted_idx, uint16_t* weights_packed,
+                                int32_t* tk_to_packed);
+
+/* ---------------------------------------------------------------- producers of the q8 activation stream
+ * Normalisation fused with block_q8_1x emission; the quantizer sees the rounded fp16 outputs, so
+ * q8_out equals quantize_q8_1(y) bit for bit.  hidden % 32 == 0.
+ *   rms_norm_f32w_q8   include/ie/ops.hpp:51-56, src/ops/elementwise.cpp:136-191
+ *     y = half((x * rsqrt(mean(x^2) + eps)) * w), x fp16, w fp32
+ *   gated_rms_norm_q8  include/ie/ops.hpp:367-372, src/ops/deltanet.cpp:73-130
+ *     y = half((w * (x * r)) * silu(z)), x fp32, z and w fp16  */
+int mx_rms_norm_f32w_q8(mx_stream_t s, const uint16_t* x, const float* w, uint16_t* y, void* q8_out, uint32_t n_rows,
+                        uint32_t hidden, float eps);
+int mx_gated_rms_norm_q8(mx_stream_t s, const float* x, const uint16_t* z, const uint16_t* weight, uint16_t* y,
+                         void* q8_out, uint32_t n_rows, uint32_t hidden, float eps);
+
 /* build_moe_packing  src/model/qwen3moe_pack.cpp:5-31 (host pointers): stable counting sort by expert.  */
 int mx_build_moe_packing(const int32_t* topk_ids, const float* topk_w, uint32_t T, uint32_t K, uint32_t E,
                          uint32_t* expert_offsets, int32_t* sorted_idx, float* weights_packed, int32_t* tk_to_packed);

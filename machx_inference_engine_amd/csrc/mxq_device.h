@@ -90,6 +90,26 @@ __device__ __forceinline__ int group_sum8_i(int v) {
     return v;
 }
 
+// ---------------------------------------------------------------- block_q8_1x emission
+// 8 lanes per 32-element block, 4 consecutive elements per lane (v), l8 = lane % 8.  All 8
+// lanes of a group must call.  d = amax/127, inv = 127/amax (0 for a zero block),
+// q = round-half-away(v*inv), s = d*float(sum q)  (src/ops/gemv_q8dot.cpp:94-124).
+__device__ __forceinline__ void emit_q8_1x(const float (&v)[4], uint32_t l8, bool live, uint8_t* blk) {
+    const float amax = group_max8(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+    const float d = amax / 127.0f, inv = amax > 0.f ? 127.0f / amax : 0.f;
+    int q[4], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        q[i] = (int)roundf(v[i] * inv);
+        sum += q[i];
+    }
+    const uint32_t packed = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) | ((uint32_t)(q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
+    const int tot = group_sum8_i(sum);
+    if (!live) return;
+    reinterpret_cast<uint32_t*>(blk + 8)[l8] = packed;
+    if (l8 == 0) *reinterpret_cast<float2*>(blk) = make_float2(d, d * (float)tot);
+}
+
 // ---------------------------------------------------------------- scales
 // The 8 six-bit (scale, min) pairs of a Q4_K block live in 12 bytes
 // (include/ie/dequant_ref.hpp:20-29).  For the 64-element group g the two

@@ -292,6 +292,61 @@ def build_moe_packing(topk_ids, topk_w, E):
     return off, si, wp, t2p
 
 
+# ---------------------------------------------------------------- routing / packing on the device
+def moe_router(x, W_gate, n_experts, k):
+    """x fp16 [T, H], W_gate fp32 [E, H] -> (topk_idx int32 [T, k] ascending, topk_w fp16 [T, k])."""
+    T, H = x.shape
+    idx = torch.empty((T, k), dtype=torch.int32, device=x.device)
+    w = torch.empty((T, k), dtype=torch.float16, device=x.device)
+    ws = torch.empty((T, n_experts), dtype=torch.float32, device=x.device)
+    assert W_gate.dtype == torch.float32
+    _call("mx_moe_router", _f16(x), _ptr(W_gate), _ptr(idx), _ptr(w), T, H, n_experts, k, _ptr(ws))
+    return idx, w
+
+
+def moe_topk_from_logits(logits, k):
+    T, E = logits.shape
+    idx = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, k), dtype=torch.float16, device=logits.device)
+    _call("mx_moe_topk_from_logits", _f16(logits), _ptr(idx), _ptr(w), E, k, T)
+    return idx, w
+
+
+def moe_build_packing_device(topk_idx, topk_w, E, decode=False):
+    """Device arrays (expert_offsets uint32-as-int32 [E+1], sorted_idx, weights_packed fp16, tk_to_packed)."""
+    T, K = topk_idx.shape
+    dev = topk_idx.device
+    off = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    si = torch.empty(T * K, dtype=torch.int32, device=dev)
+    wp = torch.empty(T * K, dtype=torch.float16, device=dev)
+    t2p = torch.empty(T * K, dtype=torch.int32, device=dev)
+    if decode:
+        assert T == 1
+        _call("mx_moe_build_pack_decode", _ptr(topk_idx), _f16(topk_w), _ptr(off), _ptr(si), _ptr(t2p), _ptr(wp), E, K)
+    else:
+        _call("mx_moe_build_packing_device", _ptr(topk_idx), _f16(topk_w), T, K, E, _ptr(off), _ptr(si), _ptr(wp), _ptr(t2p))
+    return off, si, wp, t2p
+
+
+# ---------------------------------------------------------------- fused norm -> q8 producers
+def rms_norm_f32w_q8(x, w, eps):
+    n_rows, hidden = x.shape
+    y = torch.empty_like(x)
+    q8 = torch.empty(n_rows * hidden // 32 * Q81X_BYTES, dtype=torch.uint8, device=x.device)
+    assert w.dtype == torch.float32
+    _call("mx_rms_norm_f32w_q8", _f16(x), _ptr(w), _ptr(y), _ptr(q8), n_rows, hidden, float(eps))
+    return y, q8
+
+
+def gated_rms_norm_q8(x, z, weight, eps):
+    n_rows, hidden = x.shape
+    assert x.dtype == torch.float32
+    y = torch.empty((n_rows, hidden), dtype=torch.float16, device=x.device)
+    q8 = torch.empty(n_rows * hidden // 32 * Q81X_BYTES, dtype=torch.uint8, device=x.device)
+    _call("mx_gated_rms_norm_q8", _ptr(x), _f16(z), _f16(weight), _ptr(y), _ptr(q8), n_rows, hidden, float(eps))
+    return y, q8
+
+
 # ---------------------------------------------------------------- prefill GEMM (MFMA)
 def gemm_q4_K(A, W, M, K, N, y=None):
     y = _out(y, (M, N), torch.float16, A)
