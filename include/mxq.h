@@ -110,6 +110,13 @@ int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x_q8, const uint8_t* gate
  * Q8_0 / MXFP4 batched have no reference counterpart (T >= 2 falls to dequant +
  * GEMM there, src/model/qwen35_dense.cpp:811-831).  */
 int mx_gemv_q4_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* gemv_q4_K_q8s_batched  include/ie/ops.hpp (gemv_q4_K_q8s_batched), src/ops/gemv_q8dot.cpp:483-597: the
+ * activation rows are block_q8_1s (48 B, stored half sums s0/s1; 16-byte aligned) from
+ * mx_quantize_q8_1s.  Q4_K folds the min term with s0 + s1 (one more fp32 rounding than the
+ * block_q8_1x form's d*float(sum32)).  The Q6_K form has no counterpart in the reference: its
+ * per-16 sums are exactly s0 / s1, so it is bit-identical to mx_gemv_q6_K_q8_batched.  */
+int mx_gemv_q4_K_q8s_batched(mx_stream_t s, const void* x_q8s, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_q6_K_q8s_batched(mx_stream_t s, const void* x_q8s, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W,
@@ -219,6 +226,27 @@ int mx_moe_decode_down_q4k(mx_stream_t s, const uint16_t* h, const void* down_W,
 int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx,
                            const uint16_t* topk_w, uint16_t* y_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
                            uint64_t expert_stride_bytes, uint32_t T);
+/* Int-dot grouped kernels for K-quant (AoS) expert banks, expert-sorted rows partitioned by
+ * expert_offsets[E+1] (total_rows = expert_offsets[E], known to the host from the packing):
+ *   moe_prefill_gate_up_silu_q4k_q8       include/ie/ops.hpp:912-919, src/ops/moe_fused.cpp:546-725   block_q8_1x rows
+ *   moe_prefill_gate_up_silu_q6k_q8       src/ops/moe_qwen3.cpp:52-551 (include/ie/moe_qwen3.hpp)      block_q8_1x rows
+ *   moe_prefill_down_packed_q4k_q8/_q6k_q8, moe_prefill_down_q{4,6}k_q8_gen
+ *                                         include/ie/ops.hpp:993-1006, src/ops/moe_fused.cpp:1603-1924  block_q8_1s rows
+ *     out_packed[row, n] = half(down_e . h_row), unweighted (moe_prefill_reduce applies the weights);
+ *     any E_ffn % 256 == 0 (the reference's register-resident variant needs E_ffn == 512).
+ * The `soa` flag of the reference is not taken: AoS banks only.  */
+int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W,
+                                       const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
+                                       uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W,
+                                       const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
+                                       uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_prefill_down_packed_q4k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W,
+                                      const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t H,
+                                      uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_prefill_down_packed_q6k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W,
+                                      const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t H,
+                                      uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
 /* Expert-grouped form: activation rows are expert-sorted and partitioned by
  * expert_offsets[E+1]; each expert's weights are streamed once per tile of rows;
  * experts without rows cost nothing (src/ops/moe_q8.cpp:211).

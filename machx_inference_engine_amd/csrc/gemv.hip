@@ -20,14 +20,14 @@ struct GemvSeg {
 // the activation is staged once per workgroup.
 template <class F, int T, int R, int G, int U, class OutT>
 __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> seg0, GemvSeg<F, OutT> seg1, const uint8_t* xq8,
-                                                                uint32_t K, uint32_t N, uint32_t KT, uint32_t T_real) {
+                                                                uint32_t K, uint32_t N, uint32_t KT, uint32_t T_real, uint32_t q8_split) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int GROUPS = 64 / G;
     constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
     const GemvSeg<F, OutT>& seg = blockIdx.y ? seg1 : seg0;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t grp = lane / G, gl = lane % G;
-    const size_t q8_row_bytes = (size_t)(K / 32) * kQ81xBytes;
+    const size_t q8_row_bytes = (size_t)(K / 32) * (q8_split ? kQ81sBytes : kQ81xBytes);
     auto xrow = [&](uint32_t t) { return xq8 + (size_t)(t < T_real ? t : T_real - 1) * q8_row_bytes; };
     const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
     const uint32_t n_tiles = (K + KT - 1) / KT;
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
             const bool half_tail = (kt & 63u) != 0;
             if (n_tiles > 1 || !staged) {
                 __syncthreads();
-                act = stage_act<F::SUM_GRAN, T>(lds, xrow, k0, kt, KT);
+                act = stage_act<F::SUM_GRAN, T>(lds, xrow, k0, kt, KT, q8_split != 0);
                 __syncthreads();
                 staged = true;
             }
@@ -149,7 +149,7 @@ static uint32_t pick_group(uint32_t units) {
 
 template <class F, int T, int G, class OutT>
 static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8,
-                        uint32_t K, uint32_t N, uint32_t T_real) {
+                        uint32_t K, uint32_t N, uint32_t T_real, bool split) {
     constexpr int R = GemvShape<T>::R, U = GemvShape<T>::U;
     constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
     const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);   // LDS bytes per 32 activation elements
@@ -162,29 +162,30 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t per = (n_rg + cap - 1) / cap;                // row groups per workgroup
     dim3 grid((n_rg + per - 1) / per, nseg);
     const uint32_t lds = act_tile_bytes(T, KT, F::SUM_GRAN);
-    hipLaunchKernelGGL((gemv_q8_kernel<F, T, R, G, U, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real);
+    hipLaunchKernelGGL((gemv_q8_kernel<F, T, R, G, U, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real, split ? 1u : 0u);
     return launch_status();
 }
 
 template <class F, int G, class OutT>
 static int launch_q8_g(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8, uint32_t K,
-                       uint32_t N, uint32_t T) {
+                       uint32_t N, uint32_t T, bool split) {
     switch (T) {
-        case 1: return launch_q8_tg<F, 1, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
-        case 2: return launch_q8_tg<F, 2, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
-        case 3: return launch_q8_tg<F, 3, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
-        case 4: return launch_q8_tg<F, 4, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 1: return launch_q8_tg<F, 1, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
+        case 2: return launch_q8_tg<F, 2, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
+        case 3: return launch_q8_tg<F, 3, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
+        case 4: return launch_q8_tg<F, 4, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
         case 5:
-        case 6: return launch_q8_tg<F, 6, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 6: return launch_q8_tg<F, 6, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
         case 7:
-        case 8: return launch_q8_tg<F, 8, G, OutT>(st, s0, s1, nseg, xq8, K, N, T);
+        case 8: return launch_q8_tg<F, 8, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
     }
     return MX_ERR_SHAPE;
 }
 
 // T up to 16: passes of at most 8 tokens.
 template <class F, class OutT>
-static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, int nseg, const void* xq8, uint32_t K, uint32_t N, uint32_t T) {
+static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, int nseg, const void* xq8, uint32_t K, uint32_t N, uint32_t T,
+                     bool split = false) {
     const uint8_t* x = static_cast<const uint8_t*>(xq8);
     const uint32_t G = pick_group((K + 63) / 64);
     for (uint32_t t0 = 0; t0 < T; t0 += 8) {
@@ -192,10 +193,10 @@ static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, in
         GemvSeg<F, OutT> a = s0, b = s1;
         a.y = s0.y + (size_t)t0 * N;
         if (nseg > 1) b.y = s1.y + (size_t)t0 * N;
-        const uint8_t* xt = x + (size_t)t0 * (K / 32) * kQ81xBytes;
-        const int rc = (G == 16)   ? launch_q8_g<F, 16, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn)
-                       : (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn)
-                                   : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn);
+        const uint8_t* xt = x + (size_t)t0 * (K / 32) * (split ? kQ81sBytes : kQ81xBytes);
+        const int rc = (G == 16)   ? launch_q8_g<F, 16, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split)
+                       : (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split)
+                                   : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split);
         if (rc != MX_OK) return rc;
     }
     return MX_OK;
@@ -210,23 +211,23 @@ static int check_common(const void* x, const void* y, uint32_t K, uint32_t N, ui
 }
 
 template <class OutT>
-static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, OutT* y, uint32_t K, uint32_t N, uint32_t T) {
+static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, OutT* y, uint32_t K, uint32_t N, uint32_t T, bool split = false) {
     const uint32_t k_align = fmt == 0 ? 32 : 256;
     if (int rc = check_common(xq8, y, K, N, T, k_align)) return rc;
     MX_REQUIRE_PTR(W);
-    MX_REQUIRE_ALIGN(xq8, 8);
+    MX_REQUIRE_ALIGN(xq8, split ? 16 : 8);
     MX_REQUIRE_ALIGN(W, fmt == 1 ? 16 : 2);
     const uint8_t* base = static_cast<const uint8_t*>(W);
     if (fmt == 1) {
         GemvSeg<FmtQ4K, OutT> g{{base, K / 256 * (uint32_t)kQ4KBytes}, y, nullptr};
-        return launch_q8<FmtQ4K, OutT>(s, g, g, 1, xq8, K, N, T);
+        return launch_q8<FmtQ4K, OutT>(s, g, g, 1, xq8, K, N, T, split);
     }
     if (fmt == 2) {
         GemvSeg<FmtQ6K, OutT> g{{base, K / 256 * (uint32_t)kQ6KBytes}, y, nullptr};
-        return launch_q8<FmtQ6K, OutT>(s, g, g, 1, xq8, K, N, T);
+        return launch_q8<FmtQ6K, OutT>(s, g, g, 1, xq8, K, N, T, split);
     }
     GemvSeg<FmtQ8Aos, OutT> g{{base, K / 32 * (uint32_t)kQ8_0Bytes}, y, nullptr};
-    return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T);
+    return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T, split);
 }
 
 template <class F, class ActT, class OutT>
@@ -276,6 +277,12 @@ int mx_gemv_q8_0_q8(mx_stream_t s, const void* x, const void* W, uint16_t* y, ui
 }
 int mx_gemv_q4_K_q8_batched(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
     return gemv_aos_q8<half_t>(1, s, x, W, reinterpret_cast<half_t*>(y), K, N, T);
+}
+int mx_gemv_q4_K_q8s_batched(mx_stream_t s, const void* x_q8s, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    return gemv_aos_q8<half_t>(1, s, x_q8s, W, reinterpret_cast<half_t*>(y), K, N, T, true);
+}
+int mx_gemv_q6_K_q8s_batched(mx_stream_t s, const void* x_q8s, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    return gemv_aos_q8<half_t>(2, s, x_q8s, W, reinterpret_cast<half_t*>(y), K, N, T, true);
 }
 int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
     return gemv_aos_q8<half_t>(2, s, x, W, reinterpret_cast<half_t*>(y), K, N, T);

@@ -31,6 +31,7 @@ struct MoeArgs {
     float alpha, limit;              // swiglu_oai parameters
     uint32_t act_div;                // activation row of output row r is r / act_div
     uint32_t K, N, KT, n_experts;
+    uint32_t q8_split;               // activation rows are block_q8_1s (48 B) instead of block_q8_1x
 };
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t grp = lane / G, gl = lane % G;
     const uint32_t K = a.K, N = a.N, KT = a.KT;
-    const size_t q8_row_bytes = (size_t)(K / 32) * kQ81xBytes;
+    const size_t q8_row_bytes = (size_t)(K / 32) * (a.q8_split ? kQ81sBytes : kQ81xBytes);
     const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
     const uint32_t n_tiles = (K + KT - 1) / KT;
     for (uint32_t t0 = r_begin; t0 < r_end; t0 += TT) {
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
                 }
                 if (n_tiles > 1 || !staged) {
                     __syncthreads();
-                    act = stage_act<F::SUM_GRAN, TT>(lds, xrow, k0, kt, KT);
+                    act = stage_act<F::SUM_GRAN, TT>(lds, xrow, k0, kt, KT, a.q8_split != 0);
                     __syncthreads();
                     staged = true;
                 }
@@ -343,6 +344,24 @@ static int check_moe(const void* x, const void* out, uint32_t K, uint32_t N, uin
     return MX_OK;
 }
 
+// K-quant AoS expert banks, expert-grouped rows, int-dot: shared argument checks and launch
+template <class F, int NW, int EPI>
+static int moe_grouped_kquant(mx_stream_t s, const void* act_q8, bool split, const void* W0, const void* W1, uint64_t expert_stride_bytes,
+                              const uint32_t* expert_offsets, uint16_t* out, uint32_t E, uint32_t K, uint32_t N, uint32_t total_rows, uint32_t block_bytes,
+                              uint32_t w_align) {
+    if (int rc = check_moe(act_q8, out, K, N, E)) return rc;
+    MX_REQUIRE_PTR(W0); MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(K % 256 == 0 && expert_stride_bytes % w_align == 0);
+    MX_REQUIRE_ALIGN(W0, w_align); MX_REQUIRE_ALIGN(W1, w_align);
+    if (split) MX_REQUIRE_ALIGN(act_q8, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(act_q8); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out);
+    a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = split ? 1u : 0u;
+    const uint32_t row_bytes = K / 256 * block_bytes;
+    typename F::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
+    return launch_moe<F, NW, EPI>(s, b0, b1, a, E, grouped_tt(total_rows, E));
+}
+
 }  // namespace mxq
 
 using namespace mxq;
@@ -389,6 +408,27 @@ int mx_moe_decode_down_q4k(mx_stream_t s, const uint16_t* h, const void* down_W,
 int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_out,
                            uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
     return moe_decode_fact<FmtQ6K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes, kQ6KBytes, 2);
+}
+// ------------------------------------------------------------ K-quant AoS experts, grouped rows, int-dot
+int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
+                                       uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_grouped_kquant<FmtQ4K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows,
+                                                   kQ4KBytes, 16);
+}
+int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
+                                       uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_grouped_kquant<FmtQ6K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows,
+                                                   kQ6KBytes, 2);
+}
+int mx_moe_prefill_down_packed_q4k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W, const uint32_t* expert_offsets, uint16_t* out_packed,
+                                      uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_grouped_kquant<FmtQ4K, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H,
+                                                        total_rows, kQ4KBytes, 16);
+}
+int mx_moe_prefill_down_packed_q6k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W, const uint32_t* expert_offsets, uint16_t* out_packed,
+                                      uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    return moe_grouped_kquant<FmtQ6K, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H,
+                                                        total_rows, kQ6KBytes, 2);
 }
 // ------------------------------------------------------------ Q8_0 SoA experts, grouped rows, int-dot GEMV form
 static int moe_grouped_gate_up_silu_q8_gemv(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,

@@ -38,10 +38,15 @@ struct ActTile {
     uint32_t KT;
 };
 
-// Stage T q8_1x rows, elements [k0, k0+kt), into LDS.  `xrow(t)` -> pointer to
+// Stage T q8_1 rows, elements [k0, k0+kt), into LDS.  `xrow(t)` -> pointer to
 // the first block of activation row t.  All threads of the block call this.
+// split = false: block_q8_1x {d, s, qs[32]} (40 B); the per-16 sums of SUM_GRAN 16 are
+// recomputed from the quants.  split = true: block_q8_1s {d, s0, s1, pad, qs[32]} (48 B,
+// include/ie/quant_blocks.hpp:174-181); the stored half sums are used as they are
+// (src/ops/gemv_q8dot.cpp:483-597): per 16 they are the same numbers (s0 = d * float(sum of the
+// half)); per 32 the sum s0 + s1 carries one more fp32 rounding than d * float(sum32).
 template <int SUM_GRAN, int T, class RowFn>
-__device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc) {
+__device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc, bool split = false) {
     uint4* qs = reinterpret_cast<uint4*>(lds);
     uint8_t* hdr = lds + (size_t)T * KT_alloc;
     const uint32_t halves = (kt + 63) / 64 * 4;   // padded to whole 64-element units with zeros
@@ -49,20 +54,31 @@ __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t 
         const uint32_t t = i / halves, hb = i - t * halves;
         uint2 q0 = make_uint2(0, 0), q1 = q0;
         float2 ds = make_float2(0.f, 0.f);                          // {d, s = d * sum32}
+        float s_half = 0.f;                                         // split: stored d * sum16 of this half
         if (hb * 16 < kt) {
-            const uint8_t* blk = xrow(t) + (size_t)(k0 / 32 + (hb >> 1)) * kQ81xBytes;
-            const uint2* q = reinterpret_cast<const uint2*>(blk + 8 + (hb & 1u) * 16u);
+            const uint8_t* blk = xrow(t) + (size_t)(k0 / 32 + (hb >> 1)) * (split ? kQ81sBytes : kQ81xBytes);
+            const uint2* q = reinterpret_cast<const uint2*>(blk + (split ? 16 : 8) + (hb & 1u) * 16u);
             q0 = q[0];
             q1 = q[1];
-            ds = *reinterpret_cast<const float2*>(blk);
+            if (split) {
+                const float4 h = *reinterpret_cast<const float4*>(blk);
+                ds = make_float2(h.x, h.y + h.z);
+                s_half = (hb & 1u) ? h.z : h.y;
+            } else {
+                ds = *reinterpret_cast<const float2*>(blk);
+            }
         }
         qs[(size_t)t * (KT_alloc / 16) + hb] = make_uint4(q0.x, q0.y, q1.x, q1.y);
         if (SUM_GRAN == 16) {
-            int s = dot4(0x01010101u, q0.x, 0);
-            s = dot4(0x01010101u, q0.y, s);
-            s = dot4(0x01010101u, q1.x, s);
-            s = dot4(0x01010101u, q1.y, s);
-            reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 16) + hb] = make_float2(ds.x, ds.x * (float)s);
+            float sh = s_half;
+            if (!split) {
+                int s = dot4(0x01010101u, q0.x, 0);
+                s = dot4(0x01010101u, q0.y, s);
+                s = dot4(0x01010101u, q1.x, s);
+                s = dot4(0x01010101u, q1.y, s);
+                sh = ds.x * (float)s;
+            }
+            reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 16) + hb] = make_float2(ds.x, sh);
         } else if ((hb & 1u) == 0) {
             if (SUM_GRAN == 32)
                 reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = ds;

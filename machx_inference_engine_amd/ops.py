@@ -123,6 +123,11 @@ def gemv_q4_K_q8_batched(x_q8, W, K, N, T, y=None):
     return _gemv_q8("mx_gemv_q4_K_q8_batched", x_q8, (_u8(W),), K, N, T, y)
 
 
+def gemv_kquant_q8s_batched(fmt, x_q8s, W, K, N, T, y=None):
+    """fmt in ('q4_K', 'q6_K'); x_q8s: block_q8_1s rows from quantize_q8_1s."""
+    return _gemv_q8("mx_gemv_%s_q8s_batched" % fmt, x_q8s, (_u8(W),), K, N, T, y)
+
+
 def gemv_q6_K_q8_batched(x_q8, W, K, N, T, y=None):
     return _gemv_q8("mx_gemv_q6_K_q8_batched", x_q8, (_u8(W),), K, N, T, y)
 
@@ -240,6 +245,22 @@ def moe_decode_down_kquant(fmt, h, down_W, topk_idx, topk_w, H, E_ffn, K_top, ex
     y_out = _out(y_out, (T, H), torch.float16, h)
     _call("mx_moe_decode_down_%s" % fmt, _f16(h), _u8(down_W), _ptr(topk_idx), _f16(topk_w), _ptr(y_out), H, E_ffn, K_top, expert_stride_bytes, T)
     return y_out
+
+
+def moe_prefill_gate_up_silu_kquant_q8(fmt, xq8_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None):
+    """fmt in ('q4k', 'q6k'); xq8_packed: block_q8_1x rows."""
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8_packed)
+    _call("mx_moe_prefill_gate_up_silu_%s_q8" % fmt, _ptr(xq8_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
+          expert_stride_bytes, TK)
+    return h_packed
+
+
+def moe_prefill_down_packed_kquant_q8(fmt, hq8s_packed, down_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, out_packed=None):
+    """fmt in ('q4k', 'q6k'); hq8s_packed: block_q8_1s rows."""
+    out_packed = _out(out_packed, (TK, H), torch.float16, hq8s_packed)
+    _call("mx_moe_prefill_down_packed_%s_q8" % fmt, _ptr(hq8s_packed), _u8(down_W), _ptr(expert_offsets), _ptr(out_packed), E, H, E_ffn,
+          expert_stride_bytes, TK)
+    return out_packed
 
 
 def moe_gather_rows(x, indices, n_rows, hidden, y_packed=None):

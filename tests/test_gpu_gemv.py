@@ -170,3 +170,24 @@ def test_full_size_properties_config1(mx):
     assert np.allclose(y2, 2 * yf, rtol=1e-6, atol=1e-6 * rms)
     check(yf, O.gemv_f64(O.Q4_K, W, x, K, N)[0], "config1 float chain", max_rel=1e-4)
     check(yq, O.gemv_q8chain(O.Q4_K, W, O.quantize_q8_1(x), K, N)[0], "config1 q8 chain")
+
+
+@pytest.mark.parametrize("fmt,K,N,T", [("q4_K", 1024, 96, 5), ("q4_K", 4096, 256, 16), ("q6_K", 2048, 130, 3), ("q6_K", 768, 64, 8)])
+def test_gemv_kquant_q8s_batched(mx, fmt, K, N, T):
+    """block_q8_1s activation rows (stored half sums, src/ops/gemv_q8dot.cpp:483-597) at the gate against
+    the q8-chain oracle.  Q6_K folds per 16 elements, so s0 / s1 are exactly the numbers the
+    block_q8_1x form recomputes (bit-identical); Q4_K folds per 32 with s0 + s1, one more fp32
+    rounding than d * float(sum32)."""
+    F = {"q4_K": O.Q4_K, "q6_K": O.Q6_K}[fmt]
+    W = weights(F, 700 + N, N, K)
+    x = O.normal(701 + T, (T, K)).astype(np.float32)
+    xd = dev(x)
+    xq, xqs = mx.ops.quantize_q8_1(xd), mx.ops.quantize_q8_1s(xd)
+    a = mx.ops.gemv_kquant_q8s_batched(fmt, xqs, dev(W), K, N, T)
+    b = getattr(mx.ops, "gemv_%s_q8_batched" % fmt)(xq, dev(W), K, N, T)
+    if fmt == "q6_K":
+        assert torch.equal(a, b)
+    else:
+        assert (a == b).float().mean().item() > 0.99
+    ref = O.gemv_q8chain(F, W, host(xq), K, N)
+    check(host(a).astype(np.float32), ref, "%s q8s batched T=%d" % (fmt, T))

@@ -222,3 +222,43 @@ def test_moe_decode_kquant_fp16_activations(mx, T, E, Kt, H, EF):
                 e = int(ids[t, k])
                 y_ref[t] += float(w16[t, k]) * O.gemv_f64(F, Wd[e], h_h[t * Kt + k:t * Kt + k + 1], EF, H)[0]
         check(host(y).astype(np.float32), y_ref, "moe decode down %s" % fmt)
+
+
+@pytest.mark.parametrize("T,E,Kt,H,EF", [(40, 8, 2, 512, 256), (200, 32, 4, 256, 768)])
+def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
+    """moe_prefill_gate_up_silu_q4k_q8 / _q6k_q8 (block_q8_1x rows) and moe_prefill_down_packed_q4k_q8 /
+    _q6k_q8 (block_q8_1s rows) against the q8-chain oracle, expert by expert."""
+    ops = mx.ops
+    mk = lambda F, seed, N, K: np.stack([O.quantize(F, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
+    x = f16(O.normal(8600, (T, H)))
+    ids, w = route(8601, T, E, Kt)
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    TK = T * Kt
+    counts = np.diff(off.astype(np.int64))
+    xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
+    xq = ops.quantize_q8_1(xp)
+    xq_h = host(xq).reshape(TK, -1)
+    h_keep = None
+    for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
+        Wg, Wu = mk(F, 8700, EF, H), mk(F, 8800, EF, H)
+        hp = ops.moe_prefill_gate_up_silu_kquant_q8(fmt, xq, dev(Wg), dev(Wu), dev(off), TK, E, H, EF, Wg[0].size)
+        h_ref = np.zeros((TK, EF), np.float32)
+        for e in range(E):
+            if counts[e]:
+                rows = slice(off[e], off[e + 1])
+                g = O.gemv_q8chain(F, Wg[e], xq_h[rows], H, EF)
+                u = O.gemv_q8chain(F, Wu[e], xq_h[rows], H, EF)
+                h_ref[rows] = O.swiglu_np(g.astype(np.float32), u.astype(np.float32))
+        check(host(hp).astype(np.float32), h_ref, "grouped gate_up silu %s int-dot" % fmt)
+        h_keep = hp
+    hq = ops.quantize_q8_1s(h_keep)
+    hq_x = host(ops.quantize_q8_1(h_keep)).reshape(TK, -1)   # same quants and d in the 40-byte layout for the oracle
+    for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
+        Wd = mk(F, 8900, H, EF)
+        op = ops.moe_prefill_down_packed_kquant_q8(fmt, hq, dev(Wd), dev(off), TK, E, H, EF, Wd[0].size)
+        o_ref = np.zeros((TK, H), np.float64)
+        for e in range(E):
+            if counts[e]:
+                rows = slice(off[e], off[e + 1])
+                o_ref[rows] = O.gemv_q8chain(F, Wd[e], hq_x[rows], EF, H)
+        check(host(op).astype(np.float32), o_ref, "grouped down packed %s int-dot (q8_1s rows)" % fmt)
