@@ -139,6 +139,15 @@ int mx_gemv_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, u
 int mx_gemv_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N);
 int mx_gemv_mxfp4_soa_f16(mx_stream_t s, const uint16_t* A, const uint8_t* qs_plane, const uint8_t* e_plane,
                           uint16_t* y, uint32_t K, uint32_t N);
+/* Launch-count fusions of the W4A16 GEMV (same inner loop):
+ *   gemv_q4_K_dual (_dual_ssm, _dual_ffn)  src/ops/gemv_q4k.cpp:170-275,594-612: two matrices of the same
+ *     shape against one activation vector, y_a = W_a . A, y_b = W_b . A
+ *   gemv_q4_K_down_accum                    include/ie/ops.hpp:827-831, src/ops/gemv_q4k.cpp:398-472:
+ *     y[n] = half(float(y[n]) + float(sh_g[0]) * (W . A)[n])  */
+int mx_gemv_q4_K_dual(mx_stream_t s, const uint16_t* A, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b,
+                      uint32_t K, uint32_t N);
+int mx_gemv_q4_K_down_accum(mx_stream_t s, const uint16_t* A, const void* W, const uint16_t* sh_g, uint16_t* y, uint32_t K,
+                            uint32_t N);
 int mx_gemv_q4_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 int mx_gemv_q6_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);

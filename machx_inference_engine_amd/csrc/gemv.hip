@@ -71,9 +71,15 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
 // ---------------------------------------------------------------- float activations (T = 1)
 // Same unit walk; activations staged as fp32 plus per-16 sums; the fold is the
 // reference's acc += (d*sc) * sum(a*q) - (dmin*m) * sum(a)  (src/ops/gemv_q4k.cpp:119-146).
+// blockIdx.y selects one of two weight matrices that share the activation (gemv_q4_K_dual,
+// src/ops/gemv_q4k.cpp:170-275); accum_scale != NULL turns the store into the scaled
+// accumulate y = half(float(y) + float(accum_scale[0]) * acc) (gemv_q4_K_down_accum, :398-472).
 template <class F, int R, int G, class ActT, class OutT>
-__global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w, const ActT* A, OutT* y, uint32_t K, uint32_t N, uint32_t KT) {
+__global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w0, typename F::W w1, const ActT* A, OutT* y0, OutT* y1,
+                                                                  const half_t* accum_scale, uint32_t K, uint32_t N, uint32_t KT) {
     extern __shared__ __align__(16) uint8_t lds[];
+    const typename F::W& w = blockIdx.y ? w1 : w0;
+    OutT* y = blockIdx.y ? y1 : y0;
     float* xa = reinterpret_cast<float*>(lds);          // [KT]
     float* s16 = xa + KT;                                // [KT/16]
     constexpr int GROUPS = 64 / G;
@@ -115,7 +121,10 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float v = group_sum<G>(acc[r]);
-            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N) store_out(y + row0 + r, v);
+            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N) {
+                if (accum_scale) store_out(y + row0 + r, load_act(y + row0 + r) + (float)accum_scale[0] * v);
+                else store_out(y + row0 + r, v);
+            }
         }
     }
 }
@@ -231,21 +240,24 @@ static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, O
 }
 
 template <class F, class ActT, class OutT>
-static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, OutT* y, uint32_t K, uint32_t N) {
+static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, OutT* y, uint32_t K, uint32_t N, const typename F::W* w_b = nullptr,
+                       OutT* y_b = nullptr, const half_t* accum_scale = nullptr) {
+    const uint32_t nseg = w_b ? 2u : 1u;
+    const typename F::W w1 = w_b ? *w_b : w;
     uint32_t KT = 8192;
     if (KT > K) KT = (K + 255) / 256 * 256;
     const uint32_t lds = KT * 4 + KT / 16 * 4;
     const uint32_t G = pick_group((K + 63) / 64);
     const uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
-    const uint32_t cap = (uint32_t)cu_count() * 8;
-    dim3 grid(n_rg < cap ? n_rg : cap);
+    const uint32_t cap = (uint32_t)cu_count() * 8 / nseg;
+    dim3 grid(n_rg < cap ? n_rg : cap, nseg);
     if (G == 16)
-        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);
     else if (G == 32)
-        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 32, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 32, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);
     else
-        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 64, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, A, y, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 64, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);
     return launch_status();
 }
 
@@ -347,6 +359,22 @@ int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x, const uint8_t* gate_qs
 
 int mx_gemv_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
     return gemv_aos_fact(1, s, reinterpret_cast<const half_t*>(A), W, reinterpret_cast<half_t*>(y), K, N);
+}
+int mx_gemv_q4_K_dual(mx_stream_t s, const uint16_t* A, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y_a, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(W_a); MX_REQUIRE_PTR(W_b); MX_REQUIRE_PTR(y_b);
+    MX_REQUIRE_ALIGN(W_a, 16); MX_REQUIRE_ALIGN(W_b, 16);
+    const uint32_t rb = K / 256 * (uint32_t)kQ4KBytes;
+    const FmtQ4K::W wa{static_cast<const uint8_t*>(W_a), rb}, wb{static_cast<const uint8_t*>(W_b), rb};
+    return launch_fact<FmtQ4K>(s, wa, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y_a), K, N, &wb, reinterpret_cast<half_t*>(y_b));
+}
+int mx_gemv_q4_K_down_accum(mx_stream_t s, const uint16_t* A, const void* W, const uint16_t* sh_g, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(W); MX_REQUIRE_PTR(sh_g);
+    MX_REQUIRE_ALIGN(W, 16);
+    const FmtQ4K::W w{static_cast<const uint8_t*>(W), K / 256 * (uint32_t)kQ4KBytes};
+    return launch_fact<FmtQ4K, half_t, half_t>(s, w, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y), K, N, nullptr, nullptr,
+                                               reinterpret_cast<const half_t*>(sh_g));
 }
 int mx_gemv_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
     return gemv_aos_fact(2, s, reinterpret_cast<const half_t*>(A), W, reinterpret_cast<half_t*>(y), K, N);

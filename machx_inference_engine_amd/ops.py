@@ -313,6 +313,18 @@ def build_moe_packing(topk_ids, topk_w, E):
     return off, si, wp, t2p
 
 
+def gemv_q4_K_dual(A, W_a, W_b, K, N):
+    ya = torch.empty(N, dtype=torch.float16, device=A.device)
+    yb = torch.empty(N, dtype=torch.float16, device=A.device)
+    _call("mx_gemv_q4_K_dual", _f16(A), _u8(W_a), _u8(W_b), _ptr(ya), _ptr(yb), K, N)
+    return ya, yb
+
+
+def gemv_q4_K_down_accum(A, W, sh_g, y, K, N):
+    _call("mx_gemv_q4_K_down_accum", _f16(A), _u8(W), _f16(sh_g), _f16(y), K, N)
+    return y
+
+
 # ---------------------------------------------------------------- routing / packing on the device
 def moe_router(x, W_gate, n_experts, k):
     """x fp16 [T, H], W_gate fp32 [E, H] -> (topk_idx int32 [T, k] ascending, topk_w fp16 [T, k])."""

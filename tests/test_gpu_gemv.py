@@ -191,3 +191,20 @@ def test_gemv_kquant_q8s_batched(mx, fmt, K, N, T):
         assert (a == b).float().mean().item() > 0.99
     ref = O.gemv_q8chain(F, W, host(xq), K, N)
     check(host(a).astype(np.float32), ref, "%s q8s batched T=%d" % (fmt, T))
+
+
+@pytest.mark.parametrize("K,N", [(2048, 32), (4096, 1000)])
+def test_gemv_q4_K_dual_and_down_accum(mx, K, N):
+    """gemv_q4_K_dual == two single GEMVs, bit for bit (same kernel, same order);
+    gemv_q4_K_down_accum: y = half(float(y) + float(sh_g) * acc) (src/ops/gemv_q4k.cpp:398-472)."""
+    Wa, Wb = weights(O.Q4_K, 1100, N, K), weights(O.Q4_K, 1101, N, K)
+    x16 = acts(1102, 1, K)
+    xd = dev(x16[0]).half()
+    ya, yb = mx.ops.gemv_q4_K_dual(xd, dev(Wa), dev(Wb), K, N)
+    assert torch.equal(ya, mx.ops.gemv_q4_K(xd, dev(Wa), K, N)) and torch.equal(yb, mx.ops.gemv_q4_K(xd, dev(Wb), K, N))
+    check(host(yb).astype(np.float32), O.gemv_f64(O.Q4_K, Wb, x16, K, N)[0], "dual second output")
+    y0 = O.round_fp16(O.normal(1103, (N,), 0.0, 1.0))
+    g = O.round_fp16(np.array([0.37], np.float32))
+    y = mx.ops.gemv_q4_K_down_accum(xd, dev(Wa), dev(g).half(), dev(y0).half(), K, N)
+    ref = y0.astype(np.float64) + float(g[0]) * O.gemv_f64(O.Q4_K, Wa, x16, K, N)[0]
+    check(host(y).astype(np.float32), ref, "down_accum")
