@@ -167,9 +167,12 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
     const uint32_t KT = (K256 + n_tiles - 1) / n_tiles * 256;   // balanced tiles
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
+    // A CU streams at a fixed rate (its waves' loads in flight over the memory latency), so the
+    // launch is balanced per CU, not per workgroup: with a whole number of workgroups per CU
+    // the dispatcher gives every CU the same number of them, and the strided row-group loop
+    // hands each CU the same number of row groups to within one per workgroup.
     const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu / nseg;
-    const uint32_t per = (n_rg + cap - 1) / cap;                // row groups per workgroup
-    dim3 grid((n_rg + per - 1) / per, nseg);
+    dim3 grid(n_rg < cap ? n_rg : cap, nseg);
     const uint32_t lds = act_tile_bytes(T, KT, F::SUM_GRAN);
     hipLaunchKernelGGL((gemv_q8_kernel<F, T, R, G, U, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real, split ? 1u : 0u);
     return launch_status();
