@@ -142,9 +142,12 @@ static int cu_count() {
 constexpr uint32_t kLdsBudget = 48 * 1024;
 constexpr int kRows = 2;             // rows per lane group, float-activation kernels
 constexpr uint32_t kWgsPerCu = 4;    // persistent grid: workgroups per CU
-// rows per lane group / unroll of the unit walk: one row and two units in flight
-// for a single token, two rows sharing each activation read when batched
-template <int T> struct GemvShape { static constexpr int R = (T == 1) ? 1 : 2, U = (T == 1) ? 2 : 1; };
+// rows per lane group / unroll of the unit walk: one row and two units in flight for a single
+// token; batched, two rows share each activation read once the per-token work dominates
+// (T > 4, or T > 2 for the formats whose fold carries a min term), one row below that
+template <int T, int SUM_GRAN> struct GemvShape {
+    static constexpr int R = (T <= 2 || (T <= 4 && SUM_GRAN == 0)) ? 1 : 2, U = (T == 1) ? 2 : 1;
+};
 
 // lanes per row: the G in {16, 32, 64} that wastes the fewest lane slots, larger on ties
 static uint32_t pick_group(uint32_t units) {
@@ -159,7 +162,7 @@ static uint32_t pick_group(uint32_t units) {
 template <class F, int T, int G, class OutT>
 static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8,
                         uint32_t K, uint32_t N, uint32_t T_real, bool split) {
-    constexpr int R = GemvShape<T>::R, U = GemvShape<T>::U;
+    constexpr int R = GemvShape<T, F::SUM_GRAN>::R, U = GemvShape<T, F::SUM_GRAN>::U;
     constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
     const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);   // LDS bytes per 32 activation elements
     const uint32_t KT_max = (kLdsBudget / (per_elem_x32 * T)) * 32 / 256 * 256;
