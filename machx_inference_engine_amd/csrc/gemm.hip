@@ -448,10 +448,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
 
     // ---- which tile: XCD-aware order (workgroup i runs on XCD i % 8; each XCD walks a
     // contiguous range of tiles, 4 token tiles x consecutive column tiles at a time)
+    // Expert-grouped tiles are uneven (dead tiles past the real count, 1-4 live token sub-tiles),
+    // so they are dealt round-robin over the XCDs instead of in contiguous ranges.
     const uint32_t total = g.tiles_m * g.tiles_n;
     const uint32_t per_xcd = (total + 7) / 8;
-    const uint32_t linear = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-    if ((blockIdx.x >> 3) >= per_xcd || linear >= total) return;
+    const uint32_t linear = (MODE == GEMM_DENSE) ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    if ((MODE == GEMM_DENSE && (blockIdx.x >> 3) >= per_xcd) || linear >= total) return;
     uint32_t tm, tn;
     {
         constexpr uint32_t GM = 4;
