@@ -49,14 +49,17 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 // Two consecutive weights of a fragment from integer codes held as fp16 subnormals: the bits
 // 0x0000 | u (u < 1024) read as fp16 are exactly u * 2^-24, so half(fma(u * 2^-24, scale * 2^24, off))
 // is the dequantized weight with the integer -> float conversion folded into the operand
-// (v_fma_mixlo/mixhi_f16: fp16 source, fp32 scale/offset, fused fp32 multiply-add, one RNE to
-// fp16).  The power-of-two rescale of `scale` is exact, so the value is bit-identical to
-// converting the code to float first.
+// (v_fma_mix_f32: fp16 source, fp32 scale/offset, fused fp32 multiply-add), then one RNE pack to
+// fp16 (v_cvt_pk_f16_f32).  The power-of-two rescale of `scale` is exact, so the value is
+// bit-identical to converting the code to float first.  Left to itself the compiler fuses
+// convert + fma + convert into v_fma_mixlo/mixhi_f16, which measures about half the rate of the
+// other VALU ops next to MFMA work on this chip; spelling the pack as an instruction keeps the two
+// halves apart.
 __device__ __forceinline__ uint32_t mix_pair(_Float16 x0, _Float16 x1, float scale, float off) {
-    half2_t o;
-    o.x = (_Float16)__builtin_fmaf((float)x0, scale, off);
-    o.y = (_Float16)__builtin_fmaf((float)x1, scale, off);
-    return __builtin_bit_cast(uint32_t, o);
+    const float f0 = __builtin_fmaf((float)x0, scale, off), f1 = __builtin_fmaf((float)x1, scale, off);
+    uint32_t r;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(f0), "v"(f1));
+    return r;
 }
 __device__ __forceinline__ half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 
