@@ -256,7 +256,7 @@ static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, Out
     const uint32_t G = pick_group((K + 63) / 64);
     const uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
-    const uint32_t cap = (uint32_t)cu_count() * 8 / nseg;
+    const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu / nseg;   // persistent and CU-balanced, as the int-dot launch
     dim3 grid(n_rg < cap ? n_rg : cap, nseg);
     if (G == 16)
         hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);

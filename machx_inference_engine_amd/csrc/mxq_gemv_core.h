@@ -186,17 +186,49 @@ __device__ __forceinline__ float code_to_f(uint32_t w, int j) {
     return (float)(int)(int8_t)(w >> (8 * j));
 }
 
-// kt activations from A (zero up to the next multiple of 64) -> xa[], sums of 16 -> s16[]
+// kt activations from A (zero up to the next multiple of 64) -> xa[], sums of 16 -> s16[].
+// One thread per 16 elements, fetched with 128-bit loads where the row allows it.
+__device__ __forceinline__ void load16(const half_t* p, float (&v)[16]) {
+    if ((reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+        const uint4 a = reinterpret_cast<const uint4*>(p)[0], b = reinterpret_cast<const uint4*>(p)[1];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            v[2 * j] = h2f(w[j] & 0xFFFFu);
+            v[2 * j + 1] = h2f(w[j] >> 16);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = (float)p[j];
+    }
+}
+__device__ __forceinline__ void load16(const float* p, float (&v)[16]) {
+    if ((reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 f = reinterpret_cast<const float4*>(p)[j];
+            v[4 * j] = f.x; v[4 * j + 1] = f.y; v[4 * j + 2] = f.z; v[4 * j + 3] = f.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = p[j];
+    }
+}
 template <class ActT>
 __device__ __forceinline__ void stage_fact(float* xa, float* s16, const ActT* A, uint32_t kt) {
     for (uint32_t i = threadIdx.x; i < (kt + 63) / 64 * 4; i += blockDim.x) {
+        float v[16];
+        if (i * 16 < kt) {
+            load16(A + i * 16, v);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) v[j] = 0.f;
+        }
         float s = 0.f;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const float v = (i * 16 < kt) ? load_act(A + i * 16 + j) : 0.f;
-            xa[i * 16 + j] = v;
-            s += v;
-        }
+        for (int j = 0; j < 16; ++j) s += v[j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) reinterpret_cast<float4*>(xa + i * 16)[j] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
         s16[i] = s;
     }
 }
