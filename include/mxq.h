@@ -56,23 +56,26 @@ int mx_quantize_q8_1s(mx_stream_t s, const uint16_t* x_f16, void* out_q8s, uint6
 int mx_quantize_q8_1s_f32(mx_stream_t s, const float* x, void* out_q8s, uint64_t n);
 
 /* ---------------------------------------------------------------- block dequant
- * dequant_q8_0/q4_K/q6_K  include/ie/dequant.hpp, src/ops/dequant_kernels.cpp:55-269
+ * dequant_q8_0/q4_K/q5_K/q6_K  include/ie/dequant.hpp, src/ops/dequant_kernels.cpp:55-269
  * dequant_mxfp4           src/ops/dequant_kernels.cpp:325-359
  * Bit-exact with ie::ref::dequant_* (include/ie/dequant_ref.hpp:32-96); fp16
  * output is the single RNE rounding of that fp32 value.  n_elements must be a
  * whole number of blocks.  `_f32` variants write the unrounded fp32 value.  */
 int mx_dequant_q8_0(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
 int mx_dequant_q4_K(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
+int mx_dequant_q5_K(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
 int mx_dequant_q6_K(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
 int mx_dequant_mxfp4(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
 int mx_dequant_q8_0_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
 int mx_dequant_q4_K_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
+int mx_dequant_q5_K_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
 int mx_dequant_q6_K_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
 int mx_dequant_mxfp4_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
-/* dequant_*_to_Bt  src/ops/dequant_kernels.cpp:282-320,392-431,611-632,364-390:
+/* dequant_*_to_Bt  src/ops/dequant_kernels.cpp:282-320,392-431,567-609,611-632,364-390:
  * whole matrix -> fp16 Bt[k*N + n].  */
 int mx_dequant_q8_0_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_q4_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q5_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_q6_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_mxfp4_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 

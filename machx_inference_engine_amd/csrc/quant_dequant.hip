@@ -75,7 +75,7 @@ static int quantize_launch(mx_stream_t s, const ActT* x, void* out, uint64_t n) 
 // (include/ie/dequant_ref.hpp:32-96): the fp32 result is bit-identical for every
 // association because each partial product is exact (11-bit d times <= 12-bit
 // integer); only Q4_K's final subtraction rounds, once, fused or not.
-enum { FMT_Q8_0 = 0, FMT_Q4_K = 1, FMT_Q6_K = 2, FMT_MXFP4 = 3 };
+enum { FMT_Q8_0 = 0, FMT_Q4_K = 1, FMT_Q6_K = 2, FMT_MXFP4 = 3, FMT_Q5_K = 4 };
 
 template <int FMT>
 struct BlockInfo;
@@ -87,6 +87,8 @@ template <>
 struct BlockInfo<FMT_Q6_K> { static constexpr uint32_t elems = 256, bytes = kQ6KBytes; };
 template <>
 struct BlockInfo<FMT_MXFP4> { static constexpr uint32_t elems = 32, bytes = kMxfp4Bytes; };
+template <>
+struct BlockInfo<FMT_Q5_K> { static constexpr uint32_t elems = 256, bytes = 176; };
 
 __device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
 
@@ -112,6 +114,20 @@ __device__ __forceinline__ void dequant8(const uint8_t* b, uint32_t e0, float (&
         for (int i = 0; i < 8; ++i) {
             const uint32_t byte = b[16 + 32 * g + l + i];
             y[i] = d1 * (float)(hi ? byte >> 4 : byte & 15u) - m1;
+        }
+    } else if (FMT == FMT_Q5_K) {
+        // {d, dmin, scales[12], qh[32], qs[128]} (include/ie/quant_blocks.hpp:79-85); Q4_K plus bit 2g+hi of qh[l]
+        const uint32_t g = e0 >> 6, hi = (e0 >> 5) & 1u, l = e0 & 31u;
+        const uint32_t* sc32 = reinterpret_cast<const uint32_t*>(b + 4);
+        uint32_t sc, mn;
+        q4k_scale_pair(sc32[0], sc32[1], sc32[2], (int)g, sc, mn);
+        const float d1 = h2f(ld16(b)) * (float)((sc >> (8 * hi)) & 0xFFu);
+        const float m1 = h2f(ld16(b + 2)) * (float)((mn >> (8 * hi)) & 0xFFu);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t byte = b[48 + 32 * g + l + i];
+            const uint32_t q = (hi ? byte >> 4 : byte & 15u) + (((b[16 + l + i] >> (2 * g + hi)) & 1u) << 4);
+            y[i] = d1 * (float)q - m1;
         }
     } else if (FMT == FMT_Q6_K) {
         const uint32_t h = e0 >> 7, sub = (e0 >> 5) & 3u, l = e0 & 31u;
@@ -173,7 +189,7 @@ static int dequant_flat(mx_stream_t s, const void* packed, OutT* out, uint64_t n
     MX_REQUIRE_PTR(packed);
     MX_REQUIRE_PTR(out);
     MX_REQUIRE_SHAPE(n > 0 && n % BlockInfo<FMT>::elems == 0);
-    MX_REQUIRE_ALIGN(packed, FMT == FMT_Q4_K ? 4 : (FMT == FMT_MXFP4 ? 1 : 2));
+    MX_REQUIRE_ALIGN(packed, (FMT == FMT_Q4_K || FMT == FMT_Q5_K) ? 4 : (FMT == FMT_MXFP4 ? 1 : 2));
     const uint64_t groups = n / 8, blocks = (groups + 255) / 256;
     MX_REQUIRE_SHAPE(blocks <= 0x7FFFFFFFull);
     hipLaunchKernelGGL((dequant_flat_kernel<FMT, OutT>), dim3((uint32_t)blocks), dim3(256), 0, as_stream(s), static_cast<const uint8_t*>(packed), out, groups);
@@ -185,7 +201,7 @@ static int dequant_bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, ui
     MX_REQUIRE_PTR(W);
     MX_REQUIRE_PTR(Bt);
     MX_REQUIRE_SHAPE(K > 0 && N > 0 && K % BlockInfo<FMT>::elems == 0 && K / 8 <= 65535);
-    MX_REQUIRE_ALIGN(W, FMT == FMT_Q4_K ? 4 : (FMT == FMT_MXFP4 ? 1 : 2));
+    MX_REQUIRE_ALIGN(W, (FMT == FMT_Q4_K || FMT == FMT_Q5_K) ? 4 : (FMT == FMT_MXFP4 ? 1 : 2));
     hipLaunchKernelGGL((dequant_bt_kernel<FMT>), dim3((N + 255) / 256, K / 8), dim3(256), 0, as_stream(s), static_cast<const uint8_t*>(W), reinterpret_cast<half_t*>(Bt), K, N);
     return launch_status();
 }
@@ -223,6 +239,7 @@ int mx_quantize_q8_1s_f32(mx_stream_t s, const float* x, void* out, uint64_t n) 
     }
 MX_DEQ(q8_0, FMT_Q8_0)
 MX_DEQ(q4_K, FMT_Q4_K)
+MX_DEQ(q5_K, FMT_Q5_K)
 MX_DEQ(q6_K, FMT_Q6_K)
 MX_DEQ(mxfp4, FMT_MXFP4)
 #undef MX_DEQ

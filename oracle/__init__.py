@@ -13,10 +13,10 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-Q8_0, Q4_K, Q6_K, MXFP4 = 0, 1, 2, 3
-FMT_NAMES = {Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", MXFP4: "mxfp4"}
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32}
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210, MXFP4: 17}
+Q8_0, Q4_K, Q6_K, MXFP4, Q5_K = 0, 1, 2, 3, 4   # Q5_K: dequant only
+FMT_NAMES = {Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", MXFP4: "mxfp4", Q5_K: "q5_K"}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, Q5_K: 256}
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210, MXFP4: 17, Q5_K: 176}
 Q8_1X_BYTES, Q8_1S_BYTES = 40, 48
 
 

@@ -11,7 +11,7 @@
  *   orc_fp16_to_fp32 / orc_fp32_to_fp16     pinned: exhaustive 2^16 sweep vs numpy
  *                                            float16 + vs oracle/_ref
  *   orc_get_scale_min_k4                     pinned: oracle/_ref + golden fixture
- *   orc_dequant (Q8_0, Q4_K, Q6_K)           pinned: oracle/_ref (ie::ref::dequant_*),
+ *   orc_dequant (Q8_0, Q4_K, Q5_K, Q6_K)     pinned: oracle/_ref (ie::ref::dequant_*),
  *                                            golden fixtures, closed forms
  *   orc_dequant (MXFP4)                      pinned: closed forms (e=127 -> E2M1 table,
  *                                            e in {0,1} denormals, 2^(e-128)), the
@@ -42,7 +42,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_Q8_0 = 0, ORC_Q4_K = 1, ORC_Q6_K = 2, ORC_MXFP4 = 3 };
+enum { ORC_Q8_0 = 0, ORC_Q4_K = 1, ORC_Q6_K = 2, ORC_MXFP4 = 3, ORC_Q5_K = 4 /* dequant only */ };
 
 /* ---------------------------------------------------------------- layouts
  * include/ie/quant_blocks.hpp:26-30 (Q8_0), :55-60 (MXFP4), :67-73 (Q4_K),
@@ -51,6 +51,7 @@ enum { ORC_Q8_0 = 0, ORC_Q4_K = 1, ORC_Q6_K = 2, ORC_MXFP4 = 3 };
 #define Q8_0_BYTES 34
 #define Q4_K_BYTES 144
 #define Q6_K_BYTES 210
+#define Q5_K_BYTES 176
 #define MXFP4_BYTES 17
 #define Q8_1X_BYTES 40
 #define Q8_1S_BYTES 48
@@ -170,6 +171,25 @@ static void deq_q4_K(const uint8_t* b, float* y) {
     }
 }
 
+/* include/ie/dequant_ref.hpp:56-75, layout include/ie/quant_blocks.hpp:79-85 {d, dmin, scales[12],
+ * qh[32], qs[128]}.  As Q4_K with a fifth bit: element e = 64g + 32hi + l takes bit (2g + hi) of
+ * qh[l]; (d*sc)*q - (dmin*m) with q in 0..31. */
+static void deq_q5_K(const uint8_t* b, float* y) {
+    const float d = orc_fp16_to_fp32(rd16(b)), dmin = orc_fp16_to_fp32(rd16(b + 2));
+    const uint8_t* scales = b + 4;
+    const uint8_t* qh = b + 16;
+    const uint8_t* qs = b + 48;
+    for (int e = 0; e < 256; ++e) {
+        const int g = e >> 6, hi = (e >> 5) & 1, l = e & 31;
+        uint8_t sc, mn;
+        orc_get_scale_min_k4(2 * g + hi, scales, &sc, &mn);
+        const float d1 = d * (float)sc, m1 = dmin * (float)mn;
+        const uint8_t byte = qs[32 * g + l];
+        const int q = (hi ? (byte >> 4) : (byte & 15)) + (((qh[l] >> (2 * g + hi)) & 1) ? 16 : 0);
+        y[e] = d1 * (float)q - m1;
+    }
+}
+
 /* include/ie/dequant_ref.hpp:78-96.  Element e = 128h + 32sub + l. */
 static void deq_q6_K(const uint8_t* b, float* y) {
     const uint8_t* ql = b;
@@ -208,6 +228,7 @@ ORC_API int orc_block_bytes(int fmt) {
         case ORC_Q4_K: return Q4_K_BYTES;
         case ORC_Q6_K: return Q6_K_BYTES;
         case ORC_MXFP4: return MXFP4_BYTES;
+        case ORC_Q5_K: return Q5_K_BYTES;
     }
     return 0;
 }
@@ -217,6 +238,7 @@ static void deq_block(int fmt, const uint8_t* b, float* y) {
         case ORC_Q4_K: deq_q4_K(b, y); break;
         case ORC_Q6_K: deq_q6_K(b, y); break;
         case ORC_MXFP4: deq_mxfp4(b, y); break;
+        case ORC_Q5_K: deq_q5_K(b, y); break;
     }
 }
 

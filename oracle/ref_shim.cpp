@@ -29,12 +29,13 @@ void ref_get_scale_min_k4(int j, const uint8_t* q, uint8_t* sc, uint8_t* m) {
     ie::ref::get_scale_min_k4(j, q, *sc, *m);
 }
 
-// fmt: 0 Q8_0, 1 Q4_K, 2 Q6_K  (MXFP4 has no host routine in the reference headers)
+// fmt: 0 Q8_0, 1 Q4_K, 2 Q6_K, 4 Q5_K  (MXFP4 has no host routine in the reference headers)
 int ref_dequant(int fmt, const void* packed, size_t n, float* out) {
     switch (fmt) {
         case 0: ie::ref::dequant_q8_0_buffer(packed, n, out); return 0;
         case 1: ie::ref::dequant_q4_K_buffer(packed, n, out); return 0;
         case 2: ie::ref::dequant_q6_K_buffer(packed, n, out); return 0;
+        case 4: ie::ref::dequant_q5_K_buffer(packed, n, out); return 0;
     }
     return 1;
 }

@@ -22,7 +22,7 @@ def sane_blocks(fmt, seed, nb):
     """Random block bytes with the fp16 scale fields forced finite (exponent < 31)."""
     bb = O.BLOCK_BYTES[fmt]
     raw = O.rand_bytes(seed, nb * bb).reshape(nb, bb).copy()
-    for off in {O.Q8_0: [1], O.Q4_K: [1, 3], O.Q6_K: [209]}[fmt]:
+    for off in {O.Q8_0: [1], O.Q4_K: [1, 3], O.Q6_K: [209], O.Q5_K: [1, 3]}[fmt]:
         raw[:, off] &= 0xBB  # clear one exponent bit: never Inf/NaN, keeps sign and subnormals
     return raw
 
@@ -32,7 +32,7 @@ def main():
     if r is None:
         raise SystemExit("oracle/_ref/libmxref.so not built (reference tree not mounted?)")
     out = {}
-    for fmt in (O.Q8_0, O.Q4_K, O.Q6_K):
+    for fmt in (O.Q8_0, O.Q4_K, O.Q6_K, O.Q5_K):
         nb = 96
         raw = sane_blocks(fmt, 0xC0FFEE + fmt, nb)
         raw[0] = 0  # all-zero block

@@ -49,6 +49,31 @@ def test_dequant_to_Bt_is_transpose(mx, fmt):
     assert np.array_equal(bt, O.dequant_to_Bt(fmt, W, K, N))
 
 
+def test_dequant_q5_K_bit_exact_and_Bt(mx):
+    """Q5_K (dequant only: src/ops/dequant_kernels.cpp:149-210,567-609).  Blocks: random bytes with
+    finite scales, and Q4_K-encoded rows given a random fifth-bit plane (realistic scale fields)."""
+    K, N = 512, 40
+    raw = O.rand_bytes(0xC0FFEE + 5, 600 * 176).reshape(600, 176).copy()
+    raw[:, 1] &= 0xBB
+    raw[:, 3] &= 0xBB
+    q4 = O.quantize(O.Q4_K, O.normal(55, (N, K), 0.0, 0.02)).reshape(-1, 144)
+    q5 = np.zeros((q4.shape[0], 176), np.uint8)
+    q5[:, :16] = q4[:, :16]
+    q5[:, 16:48] = O.rand_bytes(56, q4.shape[0] * 32).reshape(-1, 32)
+    q5[:, 48:] = q4[:, 16:]
+    blocks = np.concatenate([raw, q5, np.zeros((1, 176), np.uint8)])
+    n = blocks.shape[0] * 256
+    ref = O.dequant(O.Q5_K, blocks)
+    got32 = host(mx.ops.dequant("q5_K", dev(blocks), n, dtype=torch.float32))
+    assert np.array_equal(got32.view(np.uint32), ref.view(np.uint32))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(host(mx.ops.dequant("q5_K", dev(blocks), n)).view(np.uint16), O.fp32_to_fp16(ref))
+    W = q5.reshape(N, -1)
+    bt = host(mx.ops.dequant_to_Bt("q5_K", dev(W), K, N)).view(np.uint16)
+    assert np.array_equal(bt, O.fp32_to_fp16(O.dequant(O.Q5_K, W)).reshape(N, K).T)
+    assert np.array_equal(bt, O.dequant_to_Bt(O.Q5_K, W, K, N))
+
+
 @pytest.mark.parametrize("dtype", (torch.float16, torch.float32))
 def test_quantize_q8_1_bit_exact(mx, dtype):
     x = O.normal(0x0801, 32 * 1000, 0.0, 1.0)

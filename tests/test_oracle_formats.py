@@ -8,6 +8,7 @@ import pytest
 import oracle as O
 
 FMTS3 = (O.Q8_0, O.Q4_K, O.Q6_K)
+FMTS_REF = FMTS3 + (O.Q5_K,)   # formats the reference's host headers can dequantize
 
 
 def bits(a):
@@ -36,13 +37,13 @@ def test_fp32_to_fp16_vs_numpy_ties_and_golden(golden):
 
 
 # ---------------------------------------------------------------- dequant
-@pytest.mark.parametrize("fmt", FMTS3)
+@pytest.mark.parametrize("fmt", FMTS_REF)
 def test_dequant_matches_reference_golden(golden, fmt):
     name = O.FMT_NAMES[fmt]
     assert np.array_equal(bits(O.dequant(fmt, golden["deq_in_" + name])), bits(golden["deq_out_" + name]))
 
 
-@pytest.mark.parametrize("fmt", FMTS3)
+@pytest.mark.parametrize("fmt", FMTS_REF)
 def test_dequant_matches_ref_build_random(fmt):
     r = O.load_ref()
     if r is None:
@@ -85,6 +86,21 @@ def test_dequant_closed_forms():
     y = O.dequant(O.Q4_K, b)
     assert np.array_equal(y[160:192], 1.0 * nib[160:192] - 0.75)
     assert np.array_equal(y[:160], 0.5 * nib[:160].astype(np.float32))
+    # Q5_K: same scales, d = 0.5: y = 0.5 * q5, the fifth bit of element 64g + 32hi + l in bit 2g + hi of qh[l]
+    b5 = np.zeros(176, np.uint8)
+    b5[0:2] = np.array([0x3800], np.uint16).view(np.uint8)
+    b5[2:4] = np.array([0x3400], np.uint16).view(np.uint8)
+    b5[4:8] = 1
+    b5[12:16] = 1
+    q5 = (np.arange(256) * 11 + 5) % 32
+    for e in range(256):
+        g, hi, l = e // 64, (e // 32) % 2, e % 32
+        b5[48 + 32 * g + l] |= (q5[e] & 15) << (4 * hi)
+        b5[16 + l] |= (q5[e] >> 4) << (2 * g + hi)
+    assert np.array_equal(O.dequant(O.Q5_K, b5), 0.5 * q5.astype(np.float32))
+    b5[4 + 2 + 4] = 3        # min of sub-block 2 = 3 -> y = 0.5 * q - 0.75 there only
+    y = O.dequant(O.Q5_K, b5)
+    assert np.array_equal(y[64:96], 0.5 * q5[64:96] - 0.75) and np.array_equal(y[:64], 0.5 * q5[:64].astype(np.float32))
     # Q6_K: d = 1, scales = 1 -> y = q - 32 with q the 6-bit code of element e
     b = np.zeros(210, np.uint8)
     b[192:208] = 1
