@@ -33,12 +33,11 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kBM = 128;            // tokens per workgroup tile
+constexpr int kBM = 128;            // tokens per workgroup tile (NI = 4 token tiles of 32); NI = 2 serves dense launches with too few tiles
 constexpr int kBK = 128;            // K chunk
 constexpr int kWaveN = 64;          // weight rows per wave (2 MFMA tiles)
 constexpr int kGemmThreads = 256;
-constexpr uint32_t kABuf = kBM * kBK * 2u;   // one A chunk in LDS: 128 rows x 256 B, unpadded, 16-byte columns XOR-swizzled by row
-constexpr uint32_t kGemmLds = 2u * kABuf;
+// One A chunk in LDS: BM rows x 256 B, unpadded, 16-byte columns XOR-swizzled by row.
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     const float2_t f = {a, b};
@@ -373,18 +372,18 @@ __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t byte_of
 // so the address is the lane's step-0 address XOR-ed with step_col(S) << 4.
 // `mi` = number of live 32-token tiles of this workgroup tile (4 unless PARTIAL: expert-grouped
 // tiles are often mostly empty, and their dead token tiles skip both the LDS reads and the MFMAs).
-template <int S, class QF, bool PARTIAL>
+template <int S, class QF, bool PARTIAL, int NI>
 __device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
-                                         float16_t (&acc)[4][2], uint32_t mi) {
-    Frag af[4], bf[2];
+                                         float16_t (&acc)[NI][2], uint32_t mi) {
+    Frag af[NI], bf[2];
     const uint32_t a_s = a_frag0 ^ (QF::step_col(S) << 4);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
         if (!PARTIAL || (uint32_t)i < mi) af[i].q = *reinterpret_cast<const uint4*>(lds + a_s + i * 8192);
     QF::template frag<S>(raw[0], dec[0], bf[0]);
     QF::template frag<S>(raw[1], dec[1], bf[1]);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
         if (!PARTIAL || (uint32_t)i < mi) {
             acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[0].v, acc[i][0], 0, 0, 0);
             acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[1].v, acc[i][1], 0, 0, 0);
@@ -420,10 +419,10 @@ __device__ __forceinline__ void mma_pipe(const typename QF::Raw (&raw)[2], const
     }
 }
 
-template <class QF, bool PARTIAL>
+template <class QF, bool PARTIAL, int NI>
 __device__ __forceinline__ void mma_chunk(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
-                                          float16_t (&acc)[4][2], uint32_t mi) {
-    if constexpr (!PARTIAL) {
+                                          float16_t (&acc)[NI][2], uint32_t mi) {
+    if constexpr (!PARTIAL && NI == 4) {
         Frag af[4], bf[2][2];
 #pragma unroll
         for (int i = 0; i < 4; ++i) af[i].q = *reinterpret_cast<const uint4*>(lds + a_frag0 + i * 8192);
@@ -432,20 +431,23 @@ __device__ __forceinline__ void mma_chunk(const typename QF::Raw (&raw)[2], cons
         __builtin_amdgcn_sched_barrier(0);   // prologue stays ahead of the pipelined steps
         mma_pipe<0, QF>(raw, dec, lds, a_frag0, acc, af, bf);
     } else {
-        mma_step<0, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<1, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<2, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<3, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<4, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<5, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<6, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
-        mma_step<7, QF, PARTIAL>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<0, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<1, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<2, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<3, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<4, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<5, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<6, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
+        mma_step<7, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
     }
 }
 
-template <class QF, int MODE>
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
+// NI = 32-token tiles per workgroup tile: 4 (128 tokens, two workgroups per CU), or 2 (64 tokens,
+// three per CU) for dense launches whose 128-token tiles would leave CUs without work.
+template <class QF, int MODE, int NI>
+__global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
+    constexpr uint32_t BM = 32u * NI, ABUF = BM * kBK * 2u;   // tokens per tile, bytes of one A chunk in LDS
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
     constexpr uint32_t BN = GATE_UP ? 4 * 32 : 4 * kWaveN;   // output columns per workgroup
 
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
             for (uint32_t e0 = 0; e0 < g.E && !found; e0 += 64) {
                 const uint32_t ee = e0 + ln;
                 const uint32_t lo = ee < g.E ? g.expert_offsets[ee] : 0u, hi = ee < g.E ? g.expert_offsets[ee + 1] : 0u;
-                const uint32_t nt = (hi - lo + kBM - 1) / kBM;
+                const uint32_t nt = (hi - lo + BM - 1) / BM;
                 uint32_t incl = nt;
 #pragma unroll
                 for (int d = 1; d < 64; d <<= 1) {
@@ -487,7 +489,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
                 const bool hit = tm >= excl && tm < excl + nt;
                 if (hit) {
                     s_tile[0] = ee;
-                    s_tile[1] = lo + (tm - excl) * kBM;
+                    s_tile[1] = lo + (tm - excl) * BM;
                     s_tile[2] = hi;
                 }
                 found = __ballot(hit) != 0ull;
@@ -501,7 +503,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         row_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[1]);
         row_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[2]);
     } else {
-        row_lo = tm * kBM;
+        row_lo = tm * BM;
     }
     const typename QF::W w0 = QF::expert(bank0, e), w1 = QF::expert(GATE_UP ? bank1 : bank0, e);
 
@@ -517,28 +519,29 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
 
     const uint32_t n_chunks = g.K / kBK;
     constexpr bool PARTIAL = MODE != GEMM_DENSE;
-    const uint32_t live_rows = (row_hi - row_lo) >= (uint32_t)kBM ? (uint32_t)kBM : row_hi - row_lo;
+    const uint32_t live_rows = (row_hi - row_lo) >= BM ? BM : row_hi - row_lo;
     const uint32_t mi = (live_rows + 31u) / 32u;
 
     // A staging: wave w brings rows 32w .. 32w+31 of the chunk, 4 rows (1 KB) per load; lane L
     // fills LDS slot (row 4j + L/16, column L%16) of that 1 KB with global column
     // (L%16) ^ (row & 15).  Rows past the end of the tile re-read its last row (never used).
-    uint32_t a_off[8];
+    constexpr int NL = 2 * NI;   // 1 KB loads per wave per chunk
+    uint32_t a_off[NL];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t R = 32u * wave + 4u * j + (lane >> 4);
+    for (int j = 0; j < NL; ++j) {
+        const uint32_t R = (BM / 4u) * wave + 4u * j + (lane >> 4);
         const uint32_t Rc = R < live_rows ? R : live_rows - 1u;
         a_off[j] = Rc * (g.K * 2u) + (((lane & 15u) ^ (R & 15u)) << 4);
     }
     const uint8_t* a_glb = reinterpret_cast<const uint8_t*>(g.A + (size_t)row_lo * g.K);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds_raw;
-    const uint32_t a_dst = lds_base + wave * 8192u;   // this wave's 32 rows inside an A buffer
+    const uint32_t a_dst = lds_base + wave * (BM / 4u) * 256u;   // this wave's quarter of the rows inside an A buffer
     // step-0 fragment address of this lane inside an A buffer
     const uint32_t frag0 = r * 256u + (((QF::H_COL * h) ^ (r & 15u)) << 4);
 
-    float16_t acc[4][2];
+    float16_t acc[NI][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -550,7 +553,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
     // first: memory returns in order, and they come from L2 while the weights come from HBM.
     typename QF::Raw raw[2];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) load_to_lds16(a_glb, a_off[j], a_dst + 1024u * j);
+    for (int j = 0; j < NL; ++j) load_to_lds16(a_glb, a_off[j], a_dst + 1024u * j);
     raw[0] = QF::load(w0, wrow[0], 0, h);
     raw[1] = QF::load(w1, wrow[1], 0, h);
     __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
@@ -558,9 +561,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
 
     for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
         const uint8_t* a_next = a_glb + (size_t)(c + 1) * (kBK * 2u);
-        const uint32_t dst = a_dst + ((c + 1) & 1u) * kABuf;
+        const uint32_t dst = a_dst + ((c + 1) & 1u) * ABUF;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
+        for (int j = 0; j < NL; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
         typename QF::Raw nxt[2];
         nxt[0] = QF::load(w0, wrow[0], c + 1, h);
         nxt[1] = QF::load(w1, wrow[1], c + 1, h);
@@ -568,7 +571,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         typename QF::Dec dec[2];
         dec[0] = QF::prepare(raw[0], c, h);
         dec[1] = QF::prepare(raw[1], c, h);
-        mma_chunk<QF, PARTIAL>(raw, dec, lds_raw, (c & 1u) * kABuf + frag0, acc, mi);
+        mma_chunk<QF, PARTIAL, NI>(raw, dec, lds_raw, (c & 1u) * ABUF + frag0, acc, mi);
         raw[0] = nxt[0];
         raw[1] = nxt[1];
         __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): A rows of chunk c+1 are in LDS
@@ -579,12 +582,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
         typename QF::Dec dec[2];
         dec[0] = QF::prepare(raw[0], c, h);
         dec[1] = QF::prepare(raw[1], c, h);
-        mma_chunk<QF, PARTIAL>(raw, dec, lds_raw, (c & 1u) * kABuf + frag0, acc, mi);
+        mma_chunk<QF, PARTIAL, NI>(raw, dec, lds_raw, (c & 1u) * ABUF + frag0, acc, mi);
     }
 
     // ---- epilogue.  MFMA C layout: lane holds column n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4.
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t row = row_lo + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
@@ -606,26 +609,47 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(typename QF::Bank
 }
 
 // ---------------------------------------------------------------- host side
-template <class QF, int MODE>
-static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
-    constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU) ? 128 : 256;
+template <class QF, int MODE, int NI>
+static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
+    constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU) ? 128 : 256, BM = 32u * NI, lds = 2u * BM * kBK * 2u;
     g.tiles_n = (g.N + BN - 1) / BN;
-    g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + kBM - 1) / kBM : (rows_bound + kBM - 1) / kBM + g.E;
+    g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + BM - 1) / BM : (rows_bound + BM - 1) / BM + g.E;
     const uint64_t total = (uint64_t)g.tiles_m * g.tiles_n;
     const uint64_t grid = (total + 7) / 8 * 8;
     if (grid > 0x7FFFFFFFull) return MX_ERR_SHAPE;
-    static bool attr_set = false;   // LDS above the 64 KB default needs the opt-in, once per kernel
+    static bool attr_set = false;   // LDS at the 64 KB default limit: opt in once per kernel
     if (!attr_set) {
-        const hipError_t er = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<QF, MODE>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds);
+        const hipError_t er = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<QF, MODE, NI>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (er != hipSuccess) {
             g_last_hip_error = (int)er;
             return MX_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<QF, MODE>), dim3((uint32_t)grid), dim3(kGemmThreads), kGemmLds, as_stream(s), b0, b1, g);
+    hipLaunchKernelGGL((gemm_kernel<QF, MODE, NI>), dim3((uint32_t)grid), dim3(kGemmThreads), lds, as_stream(s), b0, b1, g);
     return launch_status();
+}
+
+static int gemm_cu_count() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    }
+    return n;
+}
+
+// Dense launches whose 128-token tiles cover at most half of the CUs take 64-token tiles instead
+// (twice the workgroups; measured: 64 tiles -> +20 %, 224 tiles -> -9 %); everything else runs
+// 128-token tiles.
+template <class QF, int MODE>
+static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
+    if constexpr (MODE == GEMM_DENSE) {
+        const uint64_t tiles128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 255) / 256);
+        if (g.M > 64 && 2 * tiles128 <= (uint64_t)gemm_cu_count()) return launch_gemm_ni<QF, MODE, 2>(s, b0, b1, g, rows_bound);
+    }
+    return launch_gemm_ni<QF, MODE, 4>(s, b0, b1, g, rows_bound);
 }
 
 static int check_gemm(const void* A, const void* W, const void* y, uint32_t M, uint32_t K, uint32_t N, uint32_t k_align, uint32_t w_align = 16) {
