@@ -151,6 +151,16 @@ int mx_gemv_q4_K_dual(mx_stream_t s, const uint16_t* A, const void* W_a, const v
                       uint32_t K, uint32_t N);
 int mx_gemv_q4_K_down_accum(mx_stream_t s, const uint16_t* A, const void* W, const uint16_t* sh_g, uint16_t* y, uint32_t K,
                             uint32_t N);
+/*   gemv_q4_K_shexp_gate_up                 include/ie/ops.hpp:807-813, src/ops/gemv_q4k.cpp:288-395:
+ *     y_h[n] = half(silu(W_gate . A)[n] * (W_up . A)[n]) and, from one extra workgroup,
+ *     sh_g_out[0] = half(sigmoid(sum_k A[k] * W_shg[k]))
+ *   gemv_q4_K_dual_ssm_gbeta                include/ie/ops.hpp:819-826, src/ops/gemv_q4k.cpp:480-590:
+ *     a = float(half(W_alpha . A)), b = float(half(W_beta . A));
+ *     g_out[n] = A_log[n] * softplus(a[n] + dt_bias[n]), beta_out[n] = sigmoid(b[n])   (any N)  */
+int mx_gemv_q4_K_shexp_gate_up(mx_stream_t s, const uint16_t* A, const void* W_gate, const void* W_up, const float* W_shg,
+                               uint16_t* y_h, uint16_t* sh_g_out, uint32_t K, uint32_t N);
+int mx_gemv_q4_K_dual_ssm_gbeta(mx_stream_t s, const uint16_t* A, const void* W_alpha, const void* W_beta, const float* A_log,
+                                const float* dt_bias, float* g_out, float* beta_out, uint32_t K, uint32_t N);
 int mx_gemv_q4_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 int mx_gemv_q6_K_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
 int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uint32_t K, uint32_t N);
@@ -281,6 +291,11 @@ int mx_moe_prefill_reduce(mx_stream_t s, const uint16_t* out_packed, const uint3
                           uint16_t* y, uint32_t T, uint32_t K_top, uint32_t H);
 int mx_moe_gather_rows(mx_stream_t s, const uint16_t* x, const int32_t* indices, uint16_t* y_packed, uint32_t n_rows,
                        uint32_t hidden);
+/* moe_scatter_add  include/ie/ops.hpp:1053-1064, src/ops/moe.cpp:284-313
+ *   y[indices[i], :] = half(float(y[indices[i], :]) + float(x_packed[i, :]) * float(weights[i]));
+ *   plain read-modify-write as in the reference, so the rows one call names must be distinct. */
+int mx_moe_scatter_add(mx_stream_t s, const uint16_t* x_packed, const int32_t* indices, const uint16_t* weights, uint16_t* y,
+                       uint32_t n_tok, uint32_t hidden);
 /* MXFP4-expert (gpt-oss) kernels.  The reference runs this layer as a host loop
  * over experts of gemv_mxfp4_soa_q8 / add_bias / swiglu_oai launches
  * (src/model/gptoss.cpp:366-420); these entry points are that loop moved onto the

@@ -74,23 +74,57 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
 // blockIdx.y selects one of two weight matrices that share the activation (gemv_q4_K_dual,
 // src/ops/gemv_q4k.cpp:170-275); accum_scale != NULL turns the store into the scaled
 // accumulate y = half(float(y) + float(accum_scale[0]) * acc) (gemv_q4_K_down_accum, :398-472).
-template <class F, int R, int G, class ActT, class OutT>
+// Epilogues of the float-activation kernel.  FACT_STORE: plain / dual (grid.y picks the matrix) /
+// scaled accumulate.  The pair modes walk the same row of two matrices in one lane group:
+// FACT_SILU_PAIR writes y0[n] = half(silu(g) * u) and one extra workgroup writes the shared-expert
+// gate scalar sigmoid(W_shg . A) (gemv_q4_K_shexp_gate_up, src/ops/gemv_q4k.cpp:288-395);
+// FACT_GBETA rounds both sums through fp16 and writes g = A_log[n] * softplus(a + dt_bias[n]),
+// beta = sigmoid(b) (gemv_q4_K_dual_ssm_gbeta, src/ops/gemv_q4k.cpp:480-590).
+enum { FACT_STORE = 0, FACT_SILU_PAIR = 1, FACT_GBETA = 2 };
+struct FactTail {
+    const float* p0;   // SILU_PAIR: W_shg [K];   GBETA: A_log [N]
+    const float* p1;   //                         GBETA: dt_bias [N]
+    void* o0;          // SILU_PAIR: sh_g_out (fp16 scalar);  GBETA: g_out (fp32 [N])
+    void* o1;          //                                     GBETA: beta_out (fp32 [N])
+};
+
+template <class F, int R, int G, class ActT, class OutT, int EPI>
 __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w0, typename F::W w1, const ActT* A, OutT* y0, OutT* y1,
-                                                                  const half_t* accum_scale, uint32_t K, uint32_t N, uint32_t KT) {
+                                                                  const half_t* accum_scale, FactTail tail, uint32_t K, uint32_t N, uint32_t KT) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const typename F::W& w = blockIdx.y ? w1 : w0;
-    OutT* y = blockIdx.y ? y1 : y0;
+    constexpr bool PAIR = EPI != FACT_STORE;
+    static_assert(!PAIR || R == 2, "pair modes keep one row of each matrix per lane group");
+    const typename F::W& w = (!PAIR && blockIdx.y) ? w1 : w0;
+    OutT* y = (!PAIR && blockIdx.y) ? y1 : y0;
     float* xa = reinterpret_cast<float*>(lds);          // [KT]
     float* s16 = xa + KT;                                // [KT/16]
     constexpr int GROUPS = 64 / G;
-    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * (PAIR ? 1 : R);
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t grp = lane / G, gl = lane % G;
     const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
     const uint32_t n_tiles = (K + KT - 1) / KT;
+    uint32_t n_wg = gridDim.x;
+    if constexpr (EPI == FACT_SILU_PAIR) {
+        // last workgroup: the gate scalar, a plain fp32 dot over the whole workgroup
+        n_wg -= 1;
+        if (blockIdx.x == n_wg) {
+            float part = 0.f;
+            for (uint32_t i = threadIdx.x; i < K; i += blockDim.x) part += load_act(A + i) * tail.p0[i];
+            part = group_sum<64>(part);
+            if (lane == (uint32_t)group_sum_lane<64>(lane)) xa[wave] = part;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                float dot = 0.f;
+                for (int i = 0; i < kGemvWaves; ++i) dot += xa[i];
+                static_cast<half_t*>(tail.o0)[0] = (half_t)(1.0f / (1.0f + __expf(-dot)));
+            }
+            return;
+        }
+    }
     bool staged = false;
-    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
-        const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += n_wg) {
+        const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * (PAIR ? 1 : R);
         float acc[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -106,7 +140,10 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
             const bool half_tail = (kt & 63u) != 0;
             typename F::Cursor cu[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) cu[r] = F::cursor(w, (row0 + r < N) ? row0 + r : N - 1, k0 / 64 + gl);
+            for (int r = 0; r < R; ++r) {
+                const uint32_t row = PAIR ? row0 : row0 + r;
+                cu[r] = F::cursor((PAIR && r) ? w1 : w, row < N ? row : N - 1, k0 / 64 + gl);
+            }
             for (uint32_t it = 0; it * G + gl < n_units; ++it) {
                 const uint32_t ul = it * G + gl, e0 = F::elem_off(ul);
                 typename F::Raw raw[R];
@@ -118,12 +155,26 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
                 }
             }
         }
+        float v[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const float v = group_sum<G>(acc[r]);
-            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N) {
-                if (accum_scale) store_out(y + row0 + r, load_act(y + row0 + r) + (float)accum_scale[0] * v);
-                else store_out(y + row0 + r, v);
+        for (int r = 0; r < R; ++r) v[r] = group_sum<G>(acc[r]);
+        const bool writer = lane == (uint32_t)group_sum_lane<G>(lane);
+        if constexpr (EPI == FACT_STORE) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (writer && row0 + r < N) {
+                    if (accum_scale) store_out(y + row0 + r, load_act(y + row0 + r) + (float)accum_scale[0] * v[r]);
+                    else store_out(y + row0 + r, v[r]);
+                }
+            }
+        } else if constexpr (EPI == FACT_SILU_PAIR) {
+            if (writer && row0 < N) store_out(y + row0, v[0] / (1.0f + __expf(-v[0])) * v[1]);
+        } else {
+            if (writer && row0 < N) {
+                const float a_h = (float)(half_t)v[0] + tail.p1[row0];
+                const float sp = fmaxf(a_h, 0.f) + log1pf(__expf(-fabsf(a_h)));
+                static_cast<float*>(tail.o0)[row0] = tail.p0[row0] * sp;
+                static_cast<float*>(tail.o1)[row0] = 1.0f / (1.0f + __expf(-(float)(half_t)v[1]));
             }
         }
     }
@@ -245,25 +296,26 @@ static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, O
     return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T, split);
 }
 
-template <class F, class ActT, class OutT>
+template <class F, class ActT, class OutT, int EPI = FACT_STORE>
 static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, OutT* y, uint32_t K, uint32_t N, const typename F::W* w_b = nullptr,
-                       OutT* y_b = nullptr, const half_t* accum_scale = nullptr) {
-    const uint32_t nseg = w_b ? 2u : 1u;
+                       OutT* y_b = nullptr, const half_t* accum_scale = nullptr, FactTail tail = FactTail{}) {
+    constexpr bool PAIR = EPI != FACT_STORE;
+    const uint32_t nseg = (w_b && !PAIR) ? 2u : 1u;
     const typename F::W w1 = w_b ? *w_b : w;
     uint32_t KT = 8192;
     if (KT > K) KT = (K + 255) / 256 * 256;
     const uint32_t lds = KT * 4 + KT / 16 * 4;
     const uint32_t G = pick_group((K + 63) / 64);
-    const uint32_t rows_per_wg = kGemvWaves * (64 / G) * kRows;
+    const uint32_t rows_per_wg = kGemvWaves * (64 / G) * (PAIR ? 1 : kRows);
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
     const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu / nseg;   // persistent and CU-balanced, as the int-dot launch
-    dim3 grid(n_rg < cap ? n_rg : cap, nseg);
+    dim3 grid((n_rg < cap ? n_rg : cap) + (EPI == FACT_SILU_PAIR ? 1 : 0), nseg);
     if (G == 16)
-        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT, EPI>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, tail, K, N, KT);
     else if (G == 32)
-        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 32, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 32, ActT, OutT, EPI>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, tail, K, N, KT);
     else
-        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 64, ActT, OutT>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, K, N, KT);
+        hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 64, ActT, OutT, EPI>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, tail, K, N, KT);
     return launch_status();
 }
 
@@ -381,6 +433,26 @@ int mx_gemv_q4_K_down_accum(mx_stream_t s, const uint16_t* A, const void* W, con
     const FmtQ4K::W w{static_cast<const uint8_t*>(W), K / 256 * (uint32_t)kQ4KBytes};
     return launch_fact<FmtQ4K, half_t, half_t>(s, w, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y), K, N, nullptr, nullptr,
                                                reinterpret_cast<const half_t*>(sh_g));
+}
+int mx_gemv_q4_K_shexp_gate_up(mx_stream_t s, const uint16_t* A, const void* W_gate, const void* W_up, const float* W_shg, uint16_t* y_h,
+                               uint16_t* sh_g_out, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y_h, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(W_gate); MX_REQUIRE_PTR(W_up); MX_REQUIRE_PTR(W_shg); MX_REQUIRE_PTR(sh_g_out);
+    MX_REQUIRE_ALIGN(W_gate, 16); MX_REQUIRE_ALIGN(W_up, 16);
+    const uint32_t rb = K / 256 * (uint32_t)kQ4KBytes;
+    const FmtQ4K::W wg{static_cast<const uint8_t*>(W_gate), rb}, wu{static_cast<const uint8_t*>(W_up), rb};
+    return launch_fact<FmtQ4K, half_t, half_t, FACT_SILU_PAIR>(s, wg, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y_h), K, N, &wu,
+                                                               nullptr, nullptr, FactTail{W_shg, nullptr, sh_g_out, nullptr});
+}
+int mx_gemv_q4_K_dual_ssm_gbeta(mx_stream_t s, const uint16_t* A, const void* W_alpha, const void* W_beta, const float* A_log,
+                                const float* dt_bias, float* g_out, float* beta_out, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, g_out, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(W_alpha); MX_REQUIRE_PTR(W_beta); MX_REQUIRE_PTR(A_log); MX_REQUIRE_PTR(dt_bias); MX_REQUIRE_PTR(beta_out);
+    MX_REQUIRE_ALIGN(W_alpha, 16); MX_REQUIRE_ALIGN(W_beta, 16);
+    const uint32_t rb = K / 256 * (uint32_t)kQ4KBytes;
+    const FmtQ4K::W wa{static_cast<const uint8_t*>(W_alpha), rb}, wb{static_cast<const uint8_t*>(W_beta), rb};
+    return launch_fact<FmtQ4K, half_t, half_t, FACT_GBETA>(s, wa, reinterpret_cast<const half_t*>(A), static_cast<half_t*>(nullptr), K, N, &wb,
+                                                           nullptr, nullptr, FactTail{A_log, dt_bias, g_out, beta_out});
 }
 int mx_gemv_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
     return gemv_aos_fact(2, s, reinterpret_cast<const half_t*>(A), W, reinterpret_cast<half_t*>(y), K, N);

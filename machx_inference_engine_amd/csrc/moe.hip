@@ -217,6 +217,28 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const half_t* x, const
     }
 }
 
+// moe_scatter_add (src/ops/moe.cpp:284-313): y[indices[i]] = half(float(y[indices[i]]) + float(x_packed[i]) * w[i]).
+// Plain read-modify-write as in the reference: the rows named by one call must be distinct.
+__global__ __launch_bounds__(256) void scatter_add_kernel(const half_t* x, const int32_t* idx, const half_t* w, half_t* y, uint32_t n_rows,
+                                                          uint32_t hidden) {
+    const uint32_t row = blockIdx.y;
+    const uint32_t c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (row >= n_rows || c >= hidden) return;
+    const float wr = (float)w[row];
+    const half_t* src = x + (size_t)row * hidden + c;
+    half_t* dst = y + (size_t)idx[row] * hidden + c;
+    if (c + 8 <= hidden && (hidden & 7u) == 0) {
+        union { uint4 v; half_t h[8]; } a, b;
+        a.v = *reinterpret_cast<const uint4*>(src);
+        b.v = *reinterpret_cast<const uint4*>(dst);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b.h[i] = (half_t)((float)b.h[i] + (float)a.h[i] * wr);
+        *reinterpret_cast<uint4*>(dst) = b.v;
+    } else {
+        for (uint32_t i = 0; i < 8 && c + i < hidden; ++i) dst[i] = (half_t)((float)dst[i] + (float)src[i] * wr);
+    }
+}
+
 // moe_reduce_q8 (src/ops/moe_q8.cpp:149-158): y[t] = sum_k y_packed[t*K+k]
 // moe_prefill_reduce_sum (:368-384): y[t] = sum_k out_packed[tk_to_packed[t*K+k]]
 // moe_prefill_reduce (src/ops/moe_fused.cpp:1927-1954): y[t] += sum_k w[row] * out_packed[row]
@@ -535,6 +557,16 @@ int mx_moe_gather_rows(mx_stream_t s, const uint16_t* x, const int32_t* indices,
     MX_REQUIRE_ALIGN(x, 16); MX_REQUIRE_ALIGN(y_packed, 16);
     hipLaunchKernelGGL(gather_rows_kernel, dim3((hidden + 2047) / 2048, n_rows), dim3(256), 0, as_stream(s), reinterpret_cast<const half_t*>(x),
                        indices, reinterpret_cast<half_t*>(y_packed), n_rows, hidden);
+    return launch_status();
+}
+int mx_moe_scatter_add(mx_stream_t s, const uint16_t* x_packed, const int32_t* indices, const uint16_t* weights, uint16_t* y, uint32_t n_tok,
+                       uint32_t hidden) {
+    MX_REQUIRE_PTR(x_packed); MX_REQUIRE_PTR(indices); MX_REQUIRE_PTR(weights); MX_REQUIRE_PTR(y);
+    MX_REQUIRE_SHAPE(n_tok > 0 && hidden > 0 && n_tok <= 65535);
+    MX_REQUIRE_ALIGN(x_packed, 16); MX_REQUIRE_ALIGN(y, 16);
+    hipLaunchKernelGGL(scatter_add_kernel, dim3((hidden + 2047) / 2048, n_tok), dim3(256), 0, as_stream(s),
+                       reinterpret_cast<const half_t*>(x_packed), indices, reinterpret_cast<const half_t*>(weights), reinterpret_cast<half_t*>(y),
+                       n_tok, hidden);
     return launch_status();
 }
 static int reduce_common(const void* packed, const void* y, uint32_t T, uint32_t K, uint32_t H) {

@@ -269,6 +269,12 @@ def moe_gather_rows(x, indices, n_rows, hidden, y_packed=None):
     return y_packed
 
 
+def moe_scatter_add(x_packed, indices, weights, y, n_tok, hidden):
+    """y[indices[i]] += weights[i] * x_packed[i] in place (rows named by one call must be distinct)."""
+    _call("mx_moe_scatter_add", _f16(x_packed), _ptr(indices), _f16(weights), _f16(y), n_tok, hidden)
+    return y
+
+
 def moe_gate_up_oai_mxfp4(x_q8, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, topk_idx, T, K, H, E_ffn, n_experts,
                           alpha=1.702, limit=7.0, h_out=None):
     h_out = _out(h_out, (T * K, E_ffn), torch.float16, x_q8)
@@ -323,6 +329,24 @@ def gemv_q4_K_dual(A, W_a, W_b, K, N):
 def gemv_q4_K_down_accum(A, W, sh_g, y, K, N):
     _call("mx_gemv_q4_K_down_accum", _f16(A), _u8(W), _f16(sh_g), _f16(y), K, N)
     return y
+
+
+def gemv_q4_K_shexp_gate_up(A, W_gate, W_up, W_shg, K, N):
+    """-> (y_h fp16 [N] = silu(W_gate.A) * (W_up.A), sh_g fp16 [1] = sigmoid(W_shg . A))."""
+    assert W_shg.dtype == torch.float32
+    y_h = torch.empty(N, dtype=torch.float16, device=A.device)
+    sh_g = torch.empty(1, dtype=torch.float16, device=A.device)
+    _call("mx_gemv_q4_K_shexp_gate_up", _f16(A), _u8(W_gate), _u8(W_up), _ptr(W_shg), _ptr(y_h), _ptr(sh_g), K, N)
+    return y_h, sh_g
+
+
+def gemv_q4_K_dual_ssm_gbeta(A, W_alpha, W_beta, A_log, dt_bias, K, N):
+    """-> (g fp32 [N] = A_log * softplus(half(W_alpha.A) + dt_bias), beta fp32 [N] = sigmoid(half(W_beta.A)))."""
+    assert A_log.dtype == torch.float32 and dt_bias.dtype == torch.float32
+    g = torch.empty(N, dtype=torch.float32, device=A.device)
+    beta = torch.empty(N, dtype=torch.float32, device=A.device)
+    _call("mx_gemv_q4_K_dual_ssm_gbeta", _f16(A), _u8(W_alpha), _u8(W_beta), _ptr(A_log), _ptr(dt_bias), _ptr(g), _ptr(beta), K, N)
+    return g, beta
 
 
 # ---------------------------------------------------------------- routing / packing on the device

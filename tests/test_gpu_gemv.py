@@ -208,3 +208,40 @@ def test_gemv_q4_K_dual_and_down_accum(mx, K, N):
     y = mx.ops.gemv_q4_K_down_accum(xd, dev(Wa), dev(g).half(), dev(y0).half(), K, N)
     ref = y0.astype(np.float64) + float(g[0]) * O.gemv_f64(O.Q4_K, Wa, x16, K, N)[0]
     check(host(y).astype(np.float32), ref, "down_accum")
+
+
+@pytest.mark.parametrize("K,N", [(2048, 512), (4096, 33)])
+def test_gemv_q4_K_shexp_gate_up(mx, K, N):
+    """y_h = half(silu(W_gate.A) * (W_up.A)) with fp32 sums, plus the gate scalar
+    sigmoid(W_shg . A) from the extra workgroup (src/ops/gemv_q4k.cpp:288-395)."""
+    Wg, Wu = weights(O.Q4_K, 1200, N, K), weights(O.Q4_K, 1201, N, K)
+    x16 = acts(1202, 1, K)
+    wshg = O.normal(1203, (K,), 0.0, 0.03)
+    y_h, sh_g = mx.ops.gemv_q4_K_shexp_gate_up(dev(x16[0]).half(), dev(Wg), dev(Wu), dev(wshg), K, N)
+    g = O.gemv_f64(O.Q4_K, Wg, x16, K, N)[0]
+    u = O.gemv_f64(O.Q4_K, Wu, x16, K, N)[0]
+    check(host(y_h).astype(np.float32), g / (1.0 + np.exp(-g)) * u, "shexp silu(g)*u")
+    dot = float(np.dot(x16[0].astype(np.float64), wshg.astype(np.float64)))
+    ref_g = 1.0 / (1.0 + np.exp(-dot))
+    assert abs(float(host(sh_g)[0]) - ref_g) <= 1e-3 * ref_g + 2.0 ** -11
+
+
+@pytest.mark.parametrize("K,N", [(2048, 32), (2048, 48)])
+def test_gemv_q4_K_dual_ssm_gbeta(mx, K, N):
+    """alpha/beta sums round through fp16, then g = A_log * softplus(a + dt_bias), beta = sigmoid(b)
+    (src/ops/gemv_q4k.cpp:480-590).  The fp16 rounding point is checked by feeding the kernel's own
+    dual GEMV outputs (bit-identical sums) through the closed form."""
+    Wa, Wb = weights(O.Q4_K, 1210, N, K), weights(O.Q4_K, 1211, N, K)
+    x16 = acts(1212, 1, K)
+    A_log = -np.exp(O.normal(1213, (N,), 0.0, 0.5)).astype(np.float32)
+    dt_bias = O.normal(1214, (N,), 0.0, 1.0)
+    xd = dev(x16[0]).half()
+    g, beta = mx.ops.gemv_q4_K_dual_ssm_gbeta(xd, dev(Wa), dev(Wb), dev(A_log), dev(dt_bias), K, N)
+    ya, yb = mx.ops.gemv_q4_K_dual(xd, dev(Wa), dev(Wb), K, N)
+    a = host(ya).astype(np.float64) + dt_bias.astype(np.float64)
+    ref_g = A_log.astype(np.float64) * (np.maximum(a, 0.0) + np.log1p(np.exp(-np.abs(a))))
+    ref_b = 1.0 / (1.0 + np.exp(-host(yb).astype(np.float64)))
+    assert np.max(np.abs(host(g) - ref_g)) <= 1e-5 * np.max(np.abs(ref_g))
+    assert np.max(np.abs(host(beta) - ref_b)) <= 1e-5
+    # and the sums themselves against the float-chain oracle
+    check(host(ya).astype(np.float32), O.gemv_f64(O.Q4_K, Wa, x16, K, N)[0], "alpha sums")

@@ -262,3 +262,18 @@ def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
                 rows = slice(off[e], off[e + 1])
                 o_ref[rows] = O.gemv_q8chain(F, Wd[e], hq_x[rows], EF, H)
         check(host(op).astype(np.float32), o_ref, "grouped down packed %s int-dot (q8_1s rows)" % fmt)
+
+
+@pytest.mark.parametrize("n_tok,hidden", [(7, 2048), (5, 100), (1, 8)])
+def test_moe_scatter_add_bit_exact(mx, n_tok, hidden):
+    """moe_scatter_add (src/ops/moe.cpp:284-313): y[idx[i]] = half(float(y[idx[i]]) + float(x[i]) * w[i]).
+    fp16 x fp16 products are exact in fp32, so the result is fixed bit for bit."""
+    T = n_tok + 3
+    xp = O.round_fp16(O.normal(1300 + hidden, (n_tok, hidden), 0.0, 1.0))
+    y0 = O.round_fp16(O.normal(1301 + hidden, (T, hidden), 0.0, 1.0))
+    w = O.round_fp16(np.abs(O.normal(1302, (n_tok,), 0.0, 0.5)))
+    idx = np.random.default_rng(1303).permutation(T)[:n_tok].astype(np.int32)
+    y = mx.ops.moe_scatter_add(dev(xp).half(), dev(idx), dev(w).half(), dev(y0).half(), n_tok, hidden)
+    ref = y0.copy()
+    ref[idx] = (y0[idx].astype(np.float32) + xp.astype(np.float32) * w[:, None].astype(np.float32)).astype(np.float16).astype(np.float32)
+    assert np.array_equal(host(y).astype(np.float32), ref)
