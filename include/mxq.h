@@ -78,6 +78,21 @@ int mx_dequant_q4_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K
 int mx_dequant_q5_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_q6_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_mxfp4_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+/* Transposed dequant of the repacked layouts; bit-identical to the AoS form of the same weights:
+ *   dequant_q4_moe_soa_to_Bt   include/ie/dequant.hpp:72-80   one expert region as streams qs | scales | {d,dmin}
+ *   dequant_q6_K_soa_to_Bt     include/ie/dequant.hpp:64-71   one expert region as streams ql | qh | scales | d
+ *   dequant_q4_soa_to_Bt       include/ie/ops.hpp:453-458, src/ops/gemv_q4_soa.cpp:319-348   natural-order planes
+ *   dequant_q6_soa_to_Bt       include/ie/ops.hpp:421-426, src/ops/gemv_q6_soa.cpp:415-444   natural-order planes
+ *   dequant_mxfp4_soa_to_Bt    include/ie/dequant.hpp:60-63, src/ops/gemv_mxfp4.cpp:316-341  qs / e planes
+ * Any N (the reference's N % 64 == 0 is not required).  */
+int mx_dequant_q4_moe_soa_to_Bt(mx_stream_t s, const void* soa_region, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q6_K_soa_to_Bt(mx_stream_t s, const void* soa_region, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q4_soa_to_Bt(mx_stream_t s, const uint8_t* q4_q, const int8_t* q4_sc, const int8_t* q4_mn, const uint16_t* q4_d,
+                            const uint16_t* q4_dmin, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q6_soa_to_Bt(mx_stream_t s, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc,
+                            const uint16_t* q6_d, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_mxfp4_soa_to_Bt(mx_stream_t s, const uint8_t* qs_plane, const uint8_t* e_plane, uint16_t* Bt, uint32_t K,
+                               uint32_t N);
 
 /* ---------------------------------------------------------------- decode GEMV, int-dot on q8 activations
  * y[n] = sum_k deq(W)[n,k] * (d8 * q8)[k], fp32 accumulate, fp16 out.
@@ -124,6 +139,18 @@ int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint
 int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W,
                                 uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* Int-dot GEMV over the repacked K-quant layouts (written by the mx_repack_* host functions below):
+ *   gemv_q4_K_reorder_q8     include/ie/ops.hpp:322-326, src/ops/gemv_q8dot.cpp:152-256   three-region streams
+ *   gemv_q4_soa_q8           include/ie/ops.hpp:444-451, src/ops/gemv_q4_soa.cpp:160-312  natural-order planes
+ *   gemv_q6_soa_q8(_batched) include/ie/ops.hpp:402-419, src/ops/gemv_q6_soa.cpp:137-407  natural-order bit planes
+ * Same products and fold as the AoS kernels; planes 16-byte aligned.  */
+int mx_gemv_q4_K_reorder_q8(mx_stream_t s, const void* x_q8, const void* W_reorder, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q4_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q4_q, const int8_t* q4_sc, const int8_t* q4_mn,
+                      const uint16_t* q4_d, const uint16_t* q4_dmin, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc,
+                      const uint16_t* q6_d, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi,
+                              const int8_t* q6_sc, const uint16_t* q6_d, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_mxfp4_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* qs_plane, const uint8_t* e_plane,
                                  uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 /* fp32-output twins of the T = 1 int-dot kernels (no reference counterpart; for
@@ -230,25 +257,27 @@ int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const ui
                    uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
                    uint32_t K, uint32_t E_ffn, uint32_t H);
 int mx_moe_reduce_q8(mx_stream_t s, const uint16_t* y_packed, uint16_t* y, uint32_t T, uint32_t K, uint32_t H);
-/* K-quant (AoS, expert-major) expert banks with fp16 activations, decode — the reference's fused
+/* K-quant expert-major expert banks with fp16 activations, decode — the reference's fused
  * Q4_K / Q6_K expert kernels; fp32 fold acc += (d*sc)*sum(a*q) - (dmin*m)*sum(a):
  *   moe_decode_gate_up_silu_q4k  include/ie/ops.hpp:1034-1041, src/ops/moe_fused.cpp:82-211
  *     h_out[t*K_top + k, n] = half(silu(gate_e . x_t) * (up_e . x_t)),  e = topk_idx[t*K_top + k]
  *   moe_decode_down_q4k / _q6k   include/ie/ops.hpp:1078-1095, src/ops/moe_fused.cpp:224-330,352-522
  *     y_out[t, n] = half(sum_k topk_w[t*K_top + k] * (down_e . h[t*K_top + k])); written, not accumulated
  * The reference signatures are single-token; T (last argument) generalises them to T tokens per
- * launch, T = 1 being the reference call.  H % 256 == 0, E_ffn % 256 == 0; the `soa` flag of the
- * reference (per-expert SoA views) is not taken: AoS banks only.  */
+ * launch, T = 1 being the reference call.  H % 256 == 0, E_ffn % 256 == 0.  soa = 0: every expert
+ * region is an array of GGUF blocks; soa != 0: every region holds the same blocks as per-field
+ * streams (q4k_wview / q6k_wview<true>, include/ie/quant_soa.hpp:33-125), written by
+ * mx_repack_moe_q4k_soa_host / mx_repack_moe_q6k_soa_host.  */
 int mx_moe_decode_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x, const void* gate_W, const void* up_W,
                                    const int32_t* topk_idx, uint16_t* h_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
-                                   uint64_t expert_stride_bytes, uint32_t T);
+                                   uint64_t expert_stride_bytes, int soa, uint32_t T);
 int mx_moe_decode_down_q4k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx,
                            const uint16_t* topk_w, uint16_t* y_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
-                           uint64_t expert_stride_bytes, uint32_t T);
+                           uint64_t expert_stride_bytes, int soa, uint32_t T);
 int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx,
                            const uint16_t* topk_w, uint16_t* y_out, uint32_t H, uint32_t E_ffn, uint32_t K_top,
-                           uint64_t expert_stride_bytes, uint32_t T);
-/* Int-dot grouped kernels for K-quant (AoS) expert banks, expert-sorted rows partitioned by
+                           uint64_t expert_stride_bytes, int soa, uint32_t T);
+/* Int-dot grouped kernels for K-quant expert banks (soa as above), expert-sorted rows partitioned by
  * expert_offsets[E+1] (total_rows = expert_offsets[E], known to the host from the packing):
  *   moe_prefill_gate_up_silu_q4k_q8       include/ie/ops.hpp:912-919, src/ops/moe_fused.cpp:546-725   block_q8_1x rows
  *   moe_prefill_gate_up_silu_q6k_q8       src/ops/moe_qwen3.cpp:52-551 (include/ie/moe_qwen3.hpp)      block_q8_1x rows
@@ -256,19 +285,19 @@ int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W,
  *                                         include/ie/ops.hpp:993-1006, src/ops/moe_fused.cpp:1603-1924  block_q8_1s rows
  *     out_packed[row, n] = half(down_e . h_row), unweighted (moe_prefill_reduce applies the weights);
  *     any E_ffn % 256 == 0 (the reference's register-resident variant needs E_ffn == 512).
- * The `soa` flag of the reference is not taken: AoS banks only.  */
+  */
 int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W,
                                        const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
-                                       uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+                                       uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W,
                                        const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
-                                       uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+                                       uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 int mx_moe_prefill_down_packed_q4k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W,
                                       const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t H,
-                                      uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+                                      uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 int mx_moe_prefill_down_packed_q6k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W,
                                       const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t H,
-                                      uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+                                      uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 /* Expert-grouped form: activation rows are expert-sorted and partitioned by
  * expert_offsets[E+1]; each expert's weights are streamed once per tile of rows;
  * experts without rows cost nothing (src/ops/moe_q8.cpp:211).
@@ -359,6 +388,25 @@ int mx_build_moe_packing(const int32_t* topk_ids, const float* topk_w, uint32_t 
  * Q8_0  AoS -> SoA planes  src/model/qwen35moe_split.cpp:134-144  */
 int mx_repack_mxfp4_to_soa(const void* blocks, uint64_t n_blocks, uint8_t* qs_plane, uint8_t* e_plane);
 int mx_repack_q8_0_to_soa(const void* blocks, uint64_t n_blocks, int8_t* qs_plane, uint16_t* d_plane);
+/* K-quant repacks (pure bit moves; every weight keeps its value):
+ *   repack_q4_K_to_reorder    include/ie/ops.hpp:316-321, src/ops/gemv_q8dot.cpp:134-147
+ *     all nb = N*K/256 blocks of a matrix -> qs[128] x nb | scales[12] x nb | {d,dmin}[4] x nb (N*K/256*144 bytes)
+ *   repack_moe_q4k_soa_host   include/ie/quant_soa.hpp:127-141   the same split inside each expert region
+ *   repack_moe_q6k_soa_host   include/ie/quant_soa.hpp:143-157   ql[128] x nb | qh[64] x nb | scales[16] x nb | d[2] x nb
+ *     (src and dst are whole banks of n_experts * nblocks_per_expert blocks and must not alias)
+ *   repack_q4_K_to_soa        include/ie/ops.hpp:431-440, src/ops/gemv_q4_soa.cpp:115-151
+ *     natural element order per row: q4_q N*K/2 bytes (element k = nibble k&1 of byte k/2), q4_sc / q4_mn N*K/32
+ *     unpacked 6-bit scales / mins, q4_d / q4_dmin N*K/256 fp16 bits
+ *   repack_q6_K_to_soa        include/ie/ops.hpp:393-399, src/ops/gemv_q6_soa.cpp:71-126
+ *     q6_lo N*K/2 (low nibbles), q6_hi N*K/4 (element k = bits 2*(k&3) of byte k/4), q6_sc N*K/16 int8,
+ *     q6_d N*K/256 fp16 bits; unlike the reference's, the planes need not be zeroed first  */
+int mx_repack_q4_K_to_reorder(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* out);
+int mx_repack_moe_q4k_soa_host(const void* src, void* dst, uint32_t n_experts, uint64_t nblocks_per_expert);
+int mx_repack_moe_q6k_soa_host(const void* src, void* dst, uint32_t n_experts, uint64_t nblocks_per_expert);
+int mx_repack_q4_K_to_soa(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* q4_q, int8_t* q4_sc, int8_t* q4_mn,
+                          uint16_t* q4_d, uint16_t* q4_dmin);
+int mx_repack_q6_K_to_soa(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* q6_lo, uint8_t* q6_hi, int8_t* q6_sc,
+                          uint16_t* q6_d);
 
 #ifdef __cplusplus
 }

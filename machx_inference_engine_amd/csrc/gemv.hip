@@ -385,6 +385,39 @@ int mx_gemv_q8_0_soa_q8(mx_stream_t s, const void* x, const int8_t* qs_W, const 
     return mx_gemv_q8_0_soa_q8_batched(s, x, qs_W, d_W, y, K, N, 1);
 }
 
+// Repacked K-quant layouts (same dots and fold as the AoS kernels; only the loads differ).
+int mx_gemv_q4_K_reorder_q8(mx_stream_t s, const void* x_q8, const void* W_reorder, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(x_q8, y, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(W_reorder);
+    MX_REQUIRE_ALIGN(x_q8, 8);
+    MX_REQUIRE_ALIGN(W_reorder, 16);
+    GemvSeg<FmtQ4KStr, half_t> g{FmtQ4KStr::view(static_cast<const uint8_t*>(W_reorder), (uint64_t)N * (K / 256), K / 256), reinterpret_cast<half_t*>(y),
+                                 nullptr};
+    return launch_q8<FmtQ4KStr, half_t>(s, g, g, 1, x_q8, K, N, 1);
+}
+int mx_gemv_q4_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q4_q, const int8_t* q4_sc, const int8_t* q4_mn, const uint16_t* q4_d,
+                      const uint16_t* q4_dmin, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(x_q8, y, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(q4_q); MX_REQUIRE_PTR(q4_sc); MX_REQUIRE_PTR(q4_mn); MX_REQUIRE_PTR(q4_d); MX_REQUIRE_PTR(q4_dmin);
+    MX_REQUIRE_ALIGN(x_q8, 8);
+    MX_REQUIRE_ALIGN(q4_q, 16); MX_REQUIRE_ALIGN(q4_sc, 2); MX_REQUIRE_ALIGN(q4_mn, 2);
+    GemvSeg<FmtQ4KNat, half_t> g{{q4_q, q4_sc, q4_mn, q4_d, q4_dmin, K}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtQ4KNat, half_t>(s, g, g, 1, x_q8, K, N, 1);
+}
+int mx_gemv_q6_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc,
+                              const uint16_t* q6_d, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    if (int rc = check_common(x_q8, y, K, N, T, 256)) return rc;
+    MX_REQUIRE_PTR(q6_lo); MX_REQUIRE_PTR(q6_hi); MX_REQUIRE_PTR(q6_sc); MX_REQUIRE_PTR(q6_d);
+    MX_REQUIRE_ALIGN(x_q8, 8);
+    MX_REQUIRE_ALIGN(q6_lo, 16); MX_REQUIRE_ALIGN(q6_hi, 16); MX_REQUIRE_ALIGN(q6_sc, 4);
+    GemvSeg<FmtQ6KNat, half_t> g{{q6_lo, q6_hi, q6_sc, q6_d, K}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtQ6KNat, half_t>(s, g, g, 1, x_q8, K, N, T);
+}
+int mx_gemv_q6_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc, const uint16_t* q6_d,
+                      uint16_t* y, uint32_t K, uint32_t N) {
+    return mx_gemv_q6_soa_q8_batched(s, x_q8, q6_lo, q6_hi, q6_sc, q6_d, y, K, N, 1);
+}
+
 int mx_gemv_mxfp4_soa_q8_batched(mx_stream_t s, const void* x, const uint8_t* qs, const uint8_t* e, uint16_t* y, uint32_t K, uint32_t N,
                                  uint32_t T) {
     if (int rc = check_common(x, y, K, N, T, 32)) return rc;

@@ -344,8 +344,8 @@ static int launch_moe_fact(mx_stream_t s, const typename F::Bank& b0, const type
 
 template <class F, int MODE>
 static int moe_decode_fact(mx_stream_t s, const uint16_t* act, const void* W0, const void* W1, const int32_t* topk_idx, const uint16_t* topk_w,
-                           uint16_t* out, uint32_t K, uint32_t N, uint32_t K_top, uint32_t T, uint64_t expert_stride_bytes, uint32_t block_bytes,
-                           uint32_t w_align) {
+                           uint16_t* out, uint32_t K, uint32_t N, uint32_t K_top, uint32_t T, uint64_t expert_stride_bytes) {
+    constexpr uint32_t w_align = F::W_ALIGN;
     MX_REQUIRE_PTR(act); MX_REQUIRE_PTR(W0); MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(out);
     if (MODE == FACT_DOWN) MX_REQUIRE_PTR(topk_w);
     MX_REQUIRE_SHAPE(K > 0 && N > 0 && K % 256 == 0 && K_top > 0 && T > 0 && expert_stride_bytes % w_align == 0);
@@ -353,8 +353,7 @@ static int moe_decode_fact(mx_stream_t s, const uint16_t* act, const void* W0, c
     MoeFactArgs a{};
     a.act = reinterpret_cast<const half_t*>(act); a.topk_idx = topk_idx; a.topk_w = reinterpret_cast<const half_t*>(topk_w);
     a.out = reinterpret_cast<half_t*>(out); a.K = K; a.N = N; a.K_top = K_top;
-    const uint32_t row_bytes = K / 256 * block_bytes;
-    typename F::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
+    const typename F::Bank b0 = F::bank(W0, expert_stride_bytes, K, N), b1 = F::bank(W1, expert_stride_bytes, K, N);
     return launch_moe_fact<F, MODE>(s, b0, b1, a, MODE == FACT_DOWN ? T : T * K_top);
 }
 
@@ -369,8 +368,8 @@ static int check_moe(const void* x, const void* out, uint32_t K, uint32_t N, uin
 // K-quant AoS expert banks, expert-grouped rows, int-dot: shared argument checks and launch
 template <class F, int NW, int EPI>
 static int moe_grouped_kquant(mx_stream_t s, const void* act_q8, bool split, const void* W0, const void* W1, uint64_t expert_stride_bytes,
-                              const uint32_t* expert_offsets, uint16_t* out, uint32_t E, uint32_t K, uint32_t N, uint32_t total_rows, uint32_t block_bytes,
-                              uint32_t w_align) {
+                              const uint32_t* expert_offsets, uint16_t* out, uint32_t E, uint32_t K, uint32_t N, uint32_t total_rows) {
+    constexpr uint32_t w_align = F::W_ALIGN;
     if (int rc = check_moe(act_q8, out, K, N, E)) return rc;
     MX_REQUIRE_PTR(W0); MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(expert_offsets);
     MX_REQUIRE_SHAPE(K % 256 == 0 && expert_stride_bytes % w_align == 0);
@@ -379,8 +378,7 @@ static int moe_grouped_kquant(mx_stream_t s, const void* act_q8, bool split, con
     MoeArgs a{};
     a.xq8 = static_cast<const uint8_t*>(act_q8); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out);
     a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = split ? 1u : 0u;
-    const uint32_t row_bytes = K / 256 * block_bytes;
-    typename F::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
+    const typename F::Bank b0 = F::bank(W0, expert_stride_bytes, K, N), b1 = F::bank(W1, expert_stride_bytes, K, N);
     return launch_moe<F, NW, EPI>(s, b0, b1, a, E, grouped_tt(total_rows, E));
 }
 
@@ -418,39 +416,49 @@ int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const ui
     FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
     return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, T * K, 1);
 }
-// ------------------------------------------------------------ K-quant AoS experts, fp16 activations, decode
+// ------------------------------------------------------------ K-quant experts, fp16 activations, decode
+// soa != 0: every expert region holds its blocks as per-field streams (include/ie/quant_soa.hpp:33-51)
 int mx_moe_decode_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x, const void* gate_W, const void* up_W, const int32_t* topk_idx, uint16_t* h_out,
-                                   uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
-    return moe_decode_fact<FmtQ4K, FACT_GATE_UP>(s, x, gate_W, up_W, topk_idx, nullptr, h_out, H, E_ffn, K_top, T, expert_stride_bytes, kQ4KBytes, 16);
+                                   uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, int soa, uint32_t T) {
+    if (soa) return moe_decode_fact<FmtQ4KStr, FACT_GATE_UP>(s, x, gate_W, up_W, topk_idx, nullptr, h_out, H, E_ffn, K_top, T, expert_stride_bytes);
+    return moe_decode_fact<FmtQ4K, FACT_GATE_UP>(s, x, gate_W, up_W, topk_idx, nullptr, h_out, H, E_ffn, K_top, T, expert_stride_bytes);
 }
 int mx_moe_decode_down_q4k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_out,
-                           uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
-    return moe_decode_fact<FmtQ4K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes, kQ4KBytes, 16);
+                           uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, int soa, uint32_t T) {
+    if (soa) return moe_decode_fact<FmtQ4KStr, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes);
+    return moe_decode_fact<FmtQ4K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes);
 }
 int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_out,
-                           uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, uint32_t T) {
-    return moe_decode_fact<FmtQ6K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes, kQ6KBytes, 2);
+                           uint32_t H, uint32_t E_ffn, uint32_t K_top, uint64_t expert_stride_bytes, int soa, uint32_t T) {
+    if (soa) return moe_decode_fact<FmtQ6KStr, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes);
+    return moe_decode_fact<FmtQ6K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes);
 }
-// ------------------------------------------------------------ K-quant AoS experts, grouped rows, int-dot
+// ------------------------------------------------------------ K-quant experts, grouped rows, int-dot
 int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
-                                       uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
-    return moe_grouped_kquant<FmtQ4K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows,
-                                                   kQ4KBytes, 16);
+                                       uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa,
+                                       uint32_t total_rows) {
+    if (soa)
+        return moe_grouped_kquant<FmtQ4KStr, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+    return moe_grouped_kquant<FmtQ4K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
 }
 int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
-                                       uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
-    return moe_grouped_kquant<FmtQ6K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows,
-                                                   kQ6KBytes, 2);
+                                       uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa,
+                                       uint32_t total_rows) {
+    if (soa)
+        return moe_grouped_kquant<FmtQ6KStr, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+    return moe_grouped_kquant<FmtQ6K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
 }
 int mx_moe_prefill_down_packed_q4k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W, const uint32_t* expert_offsets, uint16_t* out_packed,
-                                      uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
-    return moe_grouped_kquant<FmtQ4K, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H,
-                                                        total_rows, kQ4KBytes, 16);
+                                      uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
+    if (soa)
+        return moe_grouped_kquant<FmtQ4KStr, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H, total_rows);
+    return moe_grouped_kquant<FmtQ4K, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H, total_rows);
 }
 int mx_moe_prefill_down_packed_q6k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W, const uint32_t* expert_offsets, uint16_t* out_packed,
-                                      uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
-    return moe_grouped_kquant<FmtQ6K, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H,
-                                                        total_rows, kQ6KBytes, 2);
+                                      uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
+    if (soa)
+        return moe_grouped_kquant<FmtQ6KStr, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H, total_rows);
+    return moe_grouped_kquant<FmtQ6K, 1, EPI_DOWN_BIAS>(s, hq8s_packed, true, down_W, down_W, expert_stride_bytes, expert_offsets, out_packed, E, E_ffn, H, total_rows);
 }
 // ------------------------------------------------------------ Q8_0 SoA experts, grouped rows, int-dot GEMV form
 static int moe_grouped_gate_up_silu_q8_gemv(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,

@@ -73,6 +73,8 @@ struct FmtQ4K {
         uint32_t row_bytes;
     };
     __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
+    static Bank bank(const void* base, uint64_t stride, uint32_t K, uint32_t) { return {static_cast<const uint8_t*>(base), stride, K / 256 * (uint32_t)kQ4KBytes}; }
+    static constexpr uint32_t W_ALIGN = 16;
     static constexpr int SUM_GRAN = 32;
     static constexpr bool PAIRED = true;
     static constexpr uint32_t GROUP_OFF = 16;
@@ -138,6 +140,8 @@ struct FmtQ6K {
         uint32_t row_bytes;
     };
     __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
+    static Bank bank(const void* base, uint64_t stride, uint32_t K, uint32_t) { return {static_cast<const uint8_t*>(base), stride, K / 256 * (uint32_t)kQ6KBytes}; }
+    static constexpr uint32_t W_ALIGN = 2;
     static constexpr int SUM_GRAN = 16;
     static constexpr bool PAIRED = false;
     static constexpr uint32_t GROUP_OFF = 32;
@@ -179,6 +183,258 @@ struct FmtQ6K {
         o.c[3] = d * (float)(int)(int8_t)(r.sc.y >> (16u + j8));
 #pragma unroll
         for (int g = 0; g < 4; ++g) o.m[g] = 32.f * o.c[g];
+    }
+};
+
+// ---------------------------------------------------------------- Q4_K, per-region streams
+// The blocks of one matrix (or of one expert region) split into three streams of the same
+// bytes:  qs[128] x nb | scales[12] x nb | {d,dmin}[4] x nb,  nb = N * K/256
+// (repack_q4_K_to_reorder, src/ops/gemv_q8dot.cpp:134-147; per expert region
+// repack_moe_q4k_soa_host, include/ie/quant_soa.hpp:33-41,127-141).  Same units, same decode as
+// the AoS form; only the load addresses differ.
+struct FmtQ4KStr {
+    struct W {
+        const uint8_t* qs;
+        const uint8_t* sc;
+        const uint8_t* dm;
+        uint32_t bpr;         // blocks per row
+    };
+    struct Cursor {
+        const uint8_t* qs;    // the unit's 32 bytes of the lane's first block
+        const uint8_t* sc;
+        const uint8_t* dm;
+        uint32_t g;
+    };
+    typedef FmtQ4K::Raw Raw;
+    // expert e: region at base + e * expert_stride_bytes holding nb blocks as three streams
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint64_t nb;
+        uint32_t bpr;
+    };
+    __host__ __device__ static __forceinline__ W view(const uint8_t* p, uint64_t nb, uint32_t bpr) { return {p, p + nb * 128u, p + nb * 140u, bpr}; }
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return view(b.base + (size_t)e * b.expert_stride_bytes, b.nb, b.bpr); }
+    static Bank bank(const void* base, uint64_t stride, uint32_t K, uint32_t N) {
+        return {static_cast<const uint8_t*>(base), stride, (uint64_t)N * (K / 256), K / 256};
+    }
+    static constexpr int SUM_GRAN = 32;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr bool CODES_UNSIGNED = true;
+    static constexpr uint32_t W_ALIGN = 16;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        const size_t ib = (size_t)n * w.bpr + (u >> 2);
+        return {w.qs + ib * 128u + (u & 3u) * 32u, w.sc + ib * 12u, w.dm + ib * 4u, u & 3u};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const size_t step = (size_t)i * (G / 4);
+        const uint4* q = reinterpret_cast<const uint4*>(cu.qs + step * 128u);
+        const uint32_t* sc = reinterpret_cast<const uint32_t*>(cu.sc + step * 12u);
+        Raw r;
+        r.hdr = make_uint4(*reinterpret_cast<const uint32_t*>(cu.dm + step * 4u), sc[0], sc[1], sc[2]);
+        r.q0 = q[0];
+        r.q1 = q[1];
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) { FmtQ4K::decode(r, FmtQ4K::Cursor{nullptr, cu.g}, o); }
+};
+
+// ---------------------------------------------------------------- Q6_K, per-region streams
+// ql[128] x nb | qh[64] x nb | scales[16] x nb | d[2] x nb  (repack_moe_q6k_soa_host,
+// include/ie/quant_soa.hpp:43-51,143-157).  Units and decode as FmtQ6K.
+struct FmtQ6KStr {
+    struct W {
+        const uint8_t* ql;
+        const uint8_t* qh;
+        const uint8_t* sc;
+        const uint8_t* d;
+        uint32_t bpr;
+    };
+    struct Cursor {
+        const uint8_t* ql;    // + 64h + 16j of the lane's first block
+        const uint8_t* qh;    // + 32h + 16j
+        const uint8_t* sc;    // + 8h
+        const uint8_t* d;
+        uint32_t hj;
+    };
+    typedef FmtQ6K::Raw Raw;
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint64_t nb;
+        uint32_t bpr;
+    };
+    __host__ __device__ static __forceinline__ W view(const uint8_t* p, uint64_t nb, uint32_t bpr) {
+        return {p, p + nb * 128u, p + nb * 192u, p + nb * 208u, bpr};
+    }
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return view(b.base + (size_t)e * b.expert_stride_bytes, b.nb, b.bpr); }
+    static Bank bank(const void* base, uint64_t stride, uint32_t K, uint32_t N) {
+        return {static_cast<const uint8_t*>(base), stride, (uint64_t)N * (K / 256), K / 256};
+    }
+    static constexpr int SUM_GRAN = 16;
+    static constexpr bool PAIRED = false;
+    static constexpr uint32_t GROUP_OFF = 32;
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr bool CODES_UNSIGNED = true;
+    static constexpr uint32_t W_ALIGN = 2;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return FmtQ6K::elem_off(u); }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        const size_t ib = (size_t)n * w.bpr + (u >> 2);
+        const uint32_t h = (u >> 1) & 1u, j = u & 1u;
+        return {w.ql + ib * 128u + 64u * h + 16u * j, w.qh + ib * 64u + 32u * h + 16u * j, w.sc + ib * 16u + 8u * h, w.d + ib * 2u, u & 3u};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const size_t step = (size_t)i * (G / 4);
+        Raw o;
+        o.qla = load_u4_a2(cu.ql + step * 128u);
+        o.qlb = load_u4_a2(cu.ql + step * 128u + 32u);
+        o.qh = load_u4_a2(cu.qh + step * 64u);
+        o.sc = load_u2_a2(cu.sc + step * 16u);
+        o.d = *reinterpret_cast<const uint16_t*>(cu.d + step * 2u);
+        return o;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) { FmtQ6K::decode(r, FmtQ6K::Cursor{nullptr, cu.hj}, o); }
+};
+
+// ---------------------------------------------------------------- natural-order planes
+// Eight natural-order nibbles of one dword -> two dwords of byte codes in element order.
+__device__ __forceinline__ void nibbles_to_codes(uint32_t x, uint32_t& a, uint32_t& b) {
+    const uint32_t ev = x & 0x0F0F0F0Fu, od = (x >> 4) & 0x0F0F0F0Fu;   // elements 0,2,4,6 / 1,3,5,7
+    a = __builtin_amdgcn_perm(od, ev, 0x05010400u);                      // elements 0,1,2,3
+    b = __builtin_amdgcn_perm(od, ev, 0x07030602u);                      // elements 4,5,6,7
+}
+
+// Q4_K repacked per row into natural element order (repack_q4_K_to_soa, src/ops/gemv_q4_soa.cpp:18-28,
+// 115-151): q[n*(K/2) + k/2] nibble (k&1), per-32 unpacked 6-bit scale / min as int8, per-256 fp16
+// d / dmin.  Unit u = elements [64u, 64u+64): 32 bytes of nibbles, two (scale, min) pairs.
+struct FmtQ4KNat {
+    struct W {
+        const uint8_t* q;
+        const int8_t* sc;
+        const int8_t* mn;
+        const uint16_t* d;
+        const uint16_t* dmin;
+        uint32_t K;
+    };
+    struct Cursor {
+        const uint8_t* q;
+        const uint8_t* sc;
+        const uint8_t* mn;
+        const uint8_t* d;
+        const uint8_t* dmin;
+    };
+    struct Raw {
+        uint4 q0, q1;
+        uint32_t sc2, mn2, d, dmin;
+    };
+    static constexpr int SUM_GRAN = 32;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr bool CODES_UNSIGNED = true;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        const size_t sb = (size_t)n * (w.K >> 5) + 2u * u, bb = (size_t)n * (w.K >> 8) + (u >> 2);
+        return {w.q + (size_t)n * (w.K >> 1) + (size_t)u * 32u, reinterpret_cast<const uint8_t*>(w.sc + sb), reinterpret_cast<const uint8_t*>(w.mn + sb),
+                reinterpret_cast<const uint8_t*>(w.d + bb), reinterpret_cast<const uint8_t*>(w.dmin + bb)};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const uint4* q = reinterpret_cast<const uint4*>(cu.q + (size_t)i * (G * 32));
+        Raw r;
+        r.q0 = q[0];
+        r.q1 = q[1];
+        r.sc2 = *reinterpret_cast<const uint16_t*>(cu.sc + (size_t)i * (G * 2));
+        r.mn2 = *reinterpret_cast<const uint16_t*>(cu.mn + (size_t)i * (G * 2));
+        r.d = *reinterpret_cast<const uint16_t*>(cu.d + (size_t)i * (G / 4 * 2));
+        r.dmin = *reinterpret_cast<const uint16_t*>(cu.dmin + (size_t)i * (G / 4 * 2));
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
+        const uint32_t w[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            nibbles_to_codes(w[2 * g], o.q[g][0], o.q[g][1]);
+            nibbles_to_codes(w[2 * g + 1], o.q[g][2], o.q[g][3]);
+        }
+        const float d = h2f(r.d), dmin = h2f(r.dmin);
+        o.c[0] = o.c[1] = d * (float)(r.sc2 & 0xFFu);
+        o.c[2] = o.c[3] = d * (float)(r.sc2 >> 8);
+        o.m[0] = o.m[1] = dmin * (float)(r.mn2 & 0xFFu);
+        o.m[2] = o.m[3] = dmin * (float)(r.mn2 >> 8);
+    }
+};
+
+// Q6_K repacked per row into natural element order (repack_q6_K_to_soa, src/ops/gemv_q6_soa.cpp:62-126):
+// lo[n*(K/2) + k/2] nibble (k&1), hi[n*(K/4) + k/4] 2-bit field (k&3), per-16 int8 scale, per-256 fp16
+// d.  Unit u = elements [64u, 64u+64): 32 bytes lo, 16 bytes hi, four scales.  Codes stay unsigned
+// (0..63); the -32 goes into the min term as for the AoS form.
+struct FmtQ6KNat {
+    struct W {
+        const uint8_t* lo;
+        const uint8_t* hi;
+        const int8_t* sc;
+        const uint16_t* d;
+        uint32_t K;
+    };
+    struct Cursor {
+        const uint8_t* lo;
+        const uint8_t* hi;
+        const uint8_t* sc;
+        const uint8_t* d;
+    };
+    struct Raw {
+        uint4 l0, l1, h;
+        uint32_t sc4, d;
+    };
+    static constexpr int SUM_GRAN = 16;
+    static constexpr bool PAIRED = false;
+    static constexpr uint32_t GROUP_OFF = 16;
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr bool CODES_UNSIGNED = true;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {w.lo + (size_t)n * (w.K >> 1) + (size_t)u * 32u, w.hi + (size_t)n * (w.K >> 2) + (size_t)u * 16u,
+                reinterpret_cast<const uint8_t*>(w.sc + (size_t)n * (w.K >> 4) + 4u * u),
+                reinterpret_cast<const uint8_t*>(w.d + (size_t)n * (w.K >> 8) + (u >> 2))};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const uint4* l = reinterpret_cast<const uint4*>(cu.lo + (size_t)i * (G * 32));
+        Raw r;
+        r.l0 = l[0];
+        r.l1 = l[1];
+        r.h = *reinterpret_cast<const uint4*>(cu.hi + (size_t)i * (G * 16));
+        r.sc4 = *reinterpret_cast<const uint32_t*>(cu.sc + (size_t)i * (G * 4));
+        r.d = *reinterpret_cast<const uint16_t*>(cu.d + (size_t)i * (G / 4 * 2));
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
+        const uint32_t w[8] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w, r.l1.x, r.l1.y, r.l1.z, r.l1.w};
+        const uint32_t hw[4] = {r.h.x, r.h.y, r.h.z, r.h.w};
+        const float d = h2f(r.d);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            uint32_t lo[4];
+            nibbles_to_codes(w[2 * g], lo[0], lo[1]);
+            nibbles_to_codes(w[2 * g + 1], lo[2], lo[3]);
+            // 16 two-bit fields f0..f15 of one dword -> bits 4..5 of 16 byte codes: a 4x4 byte transpose
+            const uint32_t t0 = hw[g] & 0x03030303u, t1 = (hw[g] >> 2) & 0x03030303u;      // f0,f4,f8,f12 / f1,f5,f9,f13
+            const uint32_t t2 = (hw[g] >> 4) & 0x03030303u, t3 = (hw[g] >> 6) & 0x03030303u;
+            const uint32_t p01a = __builtin_amdgcn_perm(t1, t0, 0x05010400u), p01b = __builtin_amdgcn_perm(t1, t0, 0x07030602u);
+            const uint32_t p23a = __builtin_amdgcn_perm(t3, t2, 0x05010400u), p23b = __builtin_amdgcn_perm(t3, t2, 0x07030602u);
+            o.q[g][0] = lo[0] | (__builtin_amdgcn_perm(p23a, p01a, 0x05040100u) << 4);       // f0..f3
+            o.q[g][1] = lo[1] | (__builtin_amdgcn_perm(p23a, p01a, 0x07060302u) << 4);       // f4..f7
+            o.q[g][2] = lo[2] | (__builtin_amdgcn_perm(p23b, p01b, 0x05040100u) << 4);       // f8..f11
+            o.q[g][3] = lo[3] | (__builtin_amdgcn_perm(p23b, p01b, 0x07060302u) << 4);       // f12..f15
+            o.c[g] = d * (float)(int)(int8_t)(r.sc4 >> (8 * g));
+            o.m[g] = 32.f * o.c[g];
+        }
     }
 };
 

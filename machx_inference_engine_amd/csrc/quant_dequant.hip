@@ -92,6 +92,36 @@ struct BlockInfo<FMT_Q5_K> { static constexpr uint32_t elems = 256, bytes = 176;
 
 __device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
 
+// Field-pointer forms of the Q4_K / Q6_K decoders: the same arithmetic whether the fields of a
+// block sit together (AoS) or in per-field streams.
+__device__ __forceinline__ void dequant8_q4k(const uint8_t* dm, const uint8_t* scales, const uint8_t* qs, uint32_t e0, float (&y)[8]) {
+#pragma clang fp contract(off)
+    const uint32_t g = e0 >> 6, hi = (e0 >> 5) & 1u, l = e0 & 31u;
+    const uint32_t* sc32 = reinterpret_cast<const uint32_t*>(scales);
+    uint32_t sc, mn;
+    q4k_scale_pair(sc32[0], sc32[1], sc32[2], (int)g, sc, mn);
+    const float d1 = h2f(ld16(dm)) * (float)((sc >> (8 * hi)) & 0xFFu);
+    const float m1 = h2f(ld16(dm + 2)) * (float)((mn >> (8 * hi)) & 0xFFu);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t byte = qs[32 * g + l + i];
+        y[i] = d1 * (float)(hi ? byte >> 4 : byte & 15u) - m1;
+    }
+}
+__device__ __forceinline__ void dequant8_q6k(const uint8_t* ql, const uint8_t* qh, const uint8_t* scales, const uint8_t* dp, uint32_t e0, float (&y)[8]) {
+#pragma clang fp contract(off)
+    const uint32_t h = e0 >> 7, sub = (e0 >> 5) & 3u, l = e0 & 31u;
+    const float d = h2f(ld16(dp));
+    const float ds = d * (float)(int)(int8_t)scales[8 * h + 2 * sub + (l >> 4)];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t lb = ql[64 * h + 32 * (sub & 1u) + l + i];
+        const uint32_t nib = (sub & 2u) ? lb >> 4 : lb & 15u;
+        const uint32_t hi2 = (qh[32 * h + l + i] >> (2 * sub)) & 3u;
+        y[i] = ds * (float)((int)(nib | (hi2 << 4)) - 32);
+    }
+}
+
 // Dequantize the 8 consecutive elements [e0, e0+8) of block `b` (e0 % 8 == 0).
 template <int FMT>
 __device__ __forceinline__ void dequant8(const uint8_t* b, uint32_t e0, float (&y)[8]) {
@@ -104,17 +134,7 @@ __device__ __forceinline__ void dequant8(const uint8_t* b, uint32_t e0, float (&
 #pragma unroll
         for (int i = 0; i < 8; ++i) y[i] = d * (float)(int)(int8_t)b[2 + e0 + i];
     } else if (FMT == FMT_Q4_K) {
-        const uint32_t g = e0 >> 6, hi = (e0 >> 5) & 1u, l = e0 & 31u;
-        const uint32_t* sc32 = reinterpret_cast<const uint32_t*>(b + 4);
-        uint32_t sc, mn;
-        q4k_scale_pair(sc32[0], sc32[1], sc32[2], (int)g, sc, mn);
-        const float d1 = h2f(ld16(b)) * (float)((sc >> (8 * hi)) & 0xFFu);
-        const float m1 = h2f(ld16(b + 2)) * (float)((mn >> (8 * hi)) & 0xFFu);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t byte = b[16 + 32 * g + l + i];
-            y[i] = d1 * (float)(hi ? byte >> 4 : byte & 15u) - m1;
-        }
+        dequant8_q4k(b, b + 4, b + 16, e0, y);
     } else if (FMT == FMT_Q5_K) {
         // {d, dmin, scales[12], qh[32], qs[128]} (include/ie/quant_blocks.hpp:79-85); Q4_K plus bit 2g+hi of qh[l]
         const uint32_t g = e0 >> 6, hi = (e0 >> 5) & 1u, l = e0 & 31u;
@@ -130,16 +150,7 @@ __device__ __forceinline__ void dequant8(const uint8_t* b, uint32_t e0, float (&
             y[i] = d1 * (float)q - m1;
         }
     } else if (FMT == FMT_Q6_K) {
-        const uint32_t h = e0 >> 7, sub = (e0 >> 5) & 3u, l = e0 & 31u;
-        const float d = h2f(ld16(b + 208));
-        const float ds = d * (float)(int)(int8_t)b[192 + 8 * h + 2 * sub + (l >> 4)];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t lb = b[64 * h + 32 * (sub & 1u) + l + i];
-            const uint32_t nib = (sub & 2u) ? lb >> 4 : lb & 15u;
-            const uint32_t hi2 = (b[128 + 32 * h + l + i] >> (2 * sub)) & 3u;
-            y[i] = ds * (float)((int)(nib | (hi2 << 4)) - 32);
-        }
+        dequant8_q6k(b, b + 128, b + 192, b + 208, e0, y);
     } else {
         const float d = e8m0_half(b[0]);
         const uint32_t hi = e0 >> 4, j0 = e0 & 15u;
@@ -206,6 +217,83 @@ static int dequant_bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, ui
     return launch_status();
 }
 
+// ---------------------------------------------------------------- repacked layouts -> Bt
+// Views give the 8 elements [8*kg, 8*kg+8) of row n.  Values are bit-identical to the AoS
+// decoders above: the repacks move bits, they never change a value's representation.
+struct Q4KStrView {     // qs[128] x nb | scales[12] x nb | {d,dmin}[4] x nb   (include/ie/quant_soa.hpp:33-41)
+    const uint8_t* base; uint64_t nb; uint32_t bpr;
+    __device__ __forceinline__ void get(uint32_t n, uint32_t kg, float (&y)[8]) const {
+        const uint64_t ib = (uint64_t)n * bpr + (kg >> 5);
+        dequant8_q4k(base + nb * 140u + ib * 4u, base + nb * 128u + ib * 12u, base + ib * 128u, (kg & 31u) * 8u, y);
+    }
+};
+struct Q6KStrView {     // ql[128] x nb | qh[64] x nb | scales[16] x nb | d[2] x nb   (include/ie/quant_soa.hpp:43-51)
+    const uint8_t* base; uint64_t nb; uint32_t bpr;
+    __device__ __forceinline__ void get(uint32_t n, uint32_t kg, float (&y)[8]) const {
+        const uint64_t ib = (uint64_t)n * bpr + (kg >> 5);
+        dequant8_q6k(base + ib * 128u, base + nb * 128u + ib * 64u, base + nb * 192u + ib * 16u, base + nb * 208u + ib * 2u, (kg & 31u) * 8u, y);
+    }
+};
+struct Q4KNatView {     // natural-order nibble plane + unpacked per-32 scale/min + per-256 d/dmin (src/ops/gemv_q4_soa.cpp:18-28)
+    const uint8_t* q; const int8_t* sc; const int8_t* mn; const uint16_t* d; const uint16_t* dmin; uint32_t K;
+    __device__ __forceinline__ void get(uint32_t n, uint32_t kg, float (&y)[8]) const {
+#pragma clang fp contract(off)
+        const uint32_t k = kg * 8u;
+        const uint32_t w = *reinterpret_cast<const uint32_t*>(q + (size_t)n * (K >> 1) + (k >> 1));
+        const size_t sb = (size_t)n * (K >> 5) + (k >> 5), bb = (size_t)n * (K >> 8) + (k >> 8);
+        const float d1 = h2f(d[bb]) * (float)(int)sc[sb];
+        const float m1 = h2f(dmin[bb]) * (float)(int)mn[sb];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = d1 * (float)((w >> (4 * i)) & 15u) - m1;
+    }
+};
+struct Q6KNatView {     // natural-order 4-bit and 2-bit planes + per-16 int8 scale + per-256 d (src/ops/gemv_q6_soa.cpp:62-126)
+    const uint8_t* lo; const uint8_t* hi; const int8_t* sc; const uint16_t* d; uint32_t K;
+    __device__ __forceinline__ void get(uint32_t n, uint32_t kg, float (&y)[8]) const {
+#pragma clang fp contract(off)
+        const uint32_t k = kg * 8u;
+        const uint32_t wl = *reinterpret_cast<const uint32_t*>(lo + (size_t)n * (K >> 1) + (k >> 1));
+        const uint32_t wh = *reinterpret_cast<const uint16_t*>(hi + (size_t)n * (K >> 2) + (k >> 2));
+        const float ds = h2f(d[(size_t)n * (K >> 8) + (k >> 8)]) * (float)(int)sc[(size_t)n * (K >> 4) + (k >> 4)];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = ds * (float)((int)(((wl >> (4 * i)) & 15u) | (((wh >> (2 * i)) & 3u) << 4)) - 32);
+    }
+};
+struct Mxfp4SoaView {   // qs_plane[n*(K/2) + 16b + j], e_plane[n*(K/32) + b]   (src/ops/gemv_mxfp4.cpp:13-16,316-341)
+    const uint8_t* qs; const uint8_t* e; uint32_t K;
+    __device__ __forceinline__ void get(uint32_t n, uint32_t kg, float (&y)[8]) const {
+        const uint32_t b = kg >> 2, e0 = (kg & 3u) * 8u;
+        const float d = e8m0_half(e[(size_t)n * (K >> 5) + b]);
+        const uint8_t* p = qs + (size_t)n * (K >> 1) + 16u * b + (e0 & 15u);
+        const uint32_t hi = e0 >> 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t c = hi ? p[i] >> 4 : p[i] & 15u;
+            const int mag = (int)((0x0C08060403020100ull >> (8 * (c & 7u))) & 0xFFu);
+            y[i] = (float)((c & 8u) ? -mag : mag) * d;
+        }
+    }
+};
+
+template <class V>
+__global__ __launch_bounds__(256) void dequant_bt_view_kernel(V v, half_t* Bt, uint32_t N) {
+    const uint32_t n = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t kg = blockIdx.y;
+    if (n >= N) return;
+    float y[8];
+    v.get(n, kg, y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) Bt[(size_t)(kg * 8u + i) * N + n] = f32_to_f16_rne(y[i]);
+}
+
+template <class V>
+static int dequant_bt_view(mx_stream_t s, const V& v, uint16_t* Bt, uint32_t K, uint32_t N, uint32_t k_align) {
+    MX_REQUIRE_PTR(Bt);
+    MX_REQUIRE_SHAPE(K > 0 && N > 0 && K % k_align == 0 && K / 8 <= 65535);
+    hipLaunchKernelGGL((dequant_bt_view_kernel<V>), dim3((N + 255) / 256, K / 8), dim3(256), 0, as_stream(s), v, reinterpret_cast<half_t*>(Bt), N);
+    return launch_status();
+}
+
 }  // namespace mxq
 
 using namespace mxq;
@@ -243,5 +331,33 @@ MX_DEQ(q5_K, FMT_Q5_K)
 MX_DEQ(q6_K, FMT_Q6_K)
 MX_DEQ(mxfp4, FMT_MXFP4)
 #undef MX_DEQ
+
+// Transposed dequant of the repacked layouts.
+int mx_dequant_q4_moe_soa_to_Bt(mx_stream_t s, const void* soa_region, uint16_t* Bt, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(soa_region);
+    MX_REQUIRE_ALIGN(soa_region, 4);
+    return dequant_bt_view(s, Q4KStrView{static_cast<const uint8_t*>(soa_region), (uint64_t)N * (K / 256), K / 256}, Bt, K, N, 256);
+}
+int mx_dequant_q6_K_soa_to_Bt(mx_stream_t s, const void* soa_region, uint16_t* Bt, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(soa_region);
+    MX_REQUIRE_ALIGN(soa_region, 2);
+    return dequant_bt_view(s, Q6KStrView{static_cast<const uint8_t*>(soa_region), (uint64_t)N * (K / 256), K / 256}, Bt, K, N, 256);
+}
+int mx_dequant_q4_soa_to_Bt(mx_stream_t s, const uint8_t* q4_q, const int8_t* q4_sc, const int8_t* q4_mn, const uint16_t* q4_d,
+                            const uint16_t* q4_dmin, uint16_t* Bt, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(q4_q); MX_REQUIRE_PTR(q4_sc); MX_REQUIRE_PTR(q4_mn); MX_REQUIRE_PTR(q4_d); MX_REQUIRE_PTR(q4_dmin);
+    MX_REQUIRE_ALIGN(q4_q, 4);
+    return dequant_bt_view(s, Q4KNatView{q4_q, q4_sc, q4_mn, q4_d, q4_dmin, K}, Bt, K, N, 256);
+}
+int mx_dequant_q6_soa_to_Bt(mx_stream_t s, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc, const uint16_t* q6_d, uint16_t* Bt,
+                            uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(q6_lo); MX_REQUIRE_PTR(q6_hi); MX_REQUIRE_PTR(q6_sc); MX_REQUIRE_PTR(q6_d);
+    MX_REQUIRE_ALIGN(q6_lo, 4); MX_REQUIRE_ALIGN(q6_hi, 2);
+    return dequant_bt_view(s, Q6KNatView{q6_lo, q6_hi, q6_sc, q6_d, K}, Bt, K, N, 256);
+}
+int mx_dequant_mxfp4_soa_to_Bt(mx_stream_t s, const uint8_t* qs_plane, const uint8_t* e_plane, uint16_t* Bt, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(qs_plane); MX_REQUIRE_PTR(e_plane);
+    return dequant_bt_view(s, Mxfp4SoaView{qs_plane, e_plane, K}, Bt, K, N, 32);
+}
 
 }  // extern "C"

@@ -6,6 +6,7 @@ the queue becomes torch's current stream, and a violated precondition raises
 MxError instead of silently doing nothing.  Outputs are allocated here when the
 caller does not pass them (the reference's callers own all buffers).
 """
+import numpy as np
 import torch
 
 from . import lib
@@ -86,6 +87,13 @@ def dequant(fmt, packed, n_elements, out=None, dtype=torch.float16):
 def dequant_to_Bt(fmt, W, K, N, Bt=None):
     Bt = _out(Bt, (K, N), torch.float16, W)
     _call("mx_dequant_%s_to_Bt" % fmt, _u8(W), _ptr(Bt), K, N)
+    return Bt
+
+
+def dequant_soa_to_Bt(name, planes, K, N, Bt=None):
+    """name in ('q4_moe_soa', 'q6_K_soa', 'q4_soa', 'q6_soa', 'mxfp4_soa'); planes = device tensors in C-ABI order."""
+    Bt = _out(Bt, (K, N), torch.float16, planes[0])
+    _call("mx_dequant_%s_to_Bt" % name, *[_ptr(t) for t in planes], _ptr(Bt), K, N)
     return Bt
 
 
@@ -234,32 +242,36 @@ def moe_prefill_reduce(out_packed, tk_to_packed, weights_packed, y, T, K_top, H)
     return y
 
 
-def moe_decode_gate_up_silu_q4k(x, gate_W, up_W, topk_idx, H, E_ffn, K_top, expert_stride_bytes, T=1, h_out=None):
+def moe_decode_gate_up_silu_q4k(x, gate_W, up_W, topk_idx, H, E_ffn, K_top, expert_stride_bytes, T=1, h_out=None, soa=False):
     h_out = _out(h_out, (T * K_top, E_ffn), torch.float16, x)
-    _call("mx_moe_decode_gate_up_silu_q4k", _f16(x), _u8(gate_W), _u8(up_W), _ptr(topk_idx), _ptr(h_out), H, E_ffn, K_top, expert_stride_bytes, T)
+    _call("mx_moe_decode_gate_up_silu_q4k", _f16(x), _u8(gate_W), _u8(up_W), _ptr(topk_idx), _ptr(h_out), H, E_ffn, K_top, expert_stride_bytes,
+          int(soa), T)
     return h_out
 
 
-def moe_decode_down_kquant(fmt, h, down_W, topk_idx, topk_w, H, E_ffn, K_top, expert_stride_bytes, T=1, y_out=None):
+def moe_decode_down_kquant(fmt, h, down_W, topk_idx, topk_w, H, E_ffn, K_top, expert_stride_bytes, T=1, y_out=None, soa=False):
     """fmt in ('q4k', 'q6k')."""
     y_out = _out(y_out, (T, H), torch.float16, h)
-    _call("mx_moe_decode_down_%s" % fmt, _f16(h), _u8(down_W), _ptr(topk_idx), _f16(topk_w), _ptr(y_out), H, E_ffn, K_top, expert_stride_bytes, T)
+    _call("mx_moe_decode_down_%s" % fmt, _f16(h), _u8(down_W), _ptr(topk_idx), _f16(topk_w), _ptr(y_out), H, E_ffn, K_top, expert_stride_bytes,
+          int(soa), T)
     return y_out
 
 
-def moe_prefill_gate_up_silu_kquant_q8(fmt, xq8_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None):
+def moe_prefill_gate_up_silu_kquant_q8(fmt, xq8_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None,
+                                       soa=False):
     """fmt in ('q4k', 'q6k'); xq8_packed: block_q8_1x rows."""
     h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8_packed)
     _call("mx_moe_prefill_gate_up_silu_%s_q8" % fmt, _ptr(xq8_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
-          expert_stride_bytes, TK)
+          expert_stride_bytes, int(soa), TK)
     return h_packed
 
 
-def moe_prefill_down_packed_kquant_q8(fmt, hq8s_packed, down_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, out_packed=None):
+def moe_prefill_down_packed_kquant_q8(fmt, hq8s_packed, down_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, out_packed=None,
+                                      soa=False):
     """fmt in ('q4k', 'q6k'); hq8s_packed: block_q8_1s rows."""
     out_packed = _out(out_packed, (TK, H), torch.float16, hq8s_packed)
     _call("mx_moe_prefill_down_packed_%s_q8" % fmt, _ptr(hq8s_packed), _u8(down_W), _ptr(expert_offsets), _ptr(out_packed), E, H, E_ffn,
-          expert_stride_bytes, TK)
+          expert_stride_bytes, int(soa), TK)
     return out_packed
 
 
@@ -307,7 +319,6 @@ def moe_grouped_down_mxfp4(hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias
 
 def build_moe_packing(topk_ids, topk_w, E):
     """Host counting sort (numpy in, numpy out): expert_offsets[E+1], sorted_idx, weights_packed, tk_to_packed."""
-    import numpy as np
     ids = np.ascontiguousarray(topk_ids, np.int32)
     w = np.ascontiguousarray(topk_w, np.float32)
     T, K = ids.shape
@@ -329,6 +340,64 @@ def gemv_q4_K_dual(A, W_a, W_b, K, N):
 def gemv_q4_K_down_accum(A, W, sh_g, y, K, N):
     _call("mx_gemv_q4_K_down_accum", _f16(A), _u8(W), _f16(sh_g), _f16(y), K, N)
     return y
+
+
+def gemv_q4_K_reorder_q8(x_q8, W_reorder, K, N, y=None):
+    return _gemv_q8("mx_gemv_q4_K_reorder_q8", x_q8, (_u8(W_reorder),), K, N, 1, y)
+
+
+def gemv_q4_soa_q8(x_q8, planes, K, N, y=None):
+    """planes = (q4_q, q4_sc, q4_mn, q4_d, q4_dmin) from repack_q4_K_to_soa."""
+    return _gemv_q8("mx_gemv_q4_soa_q8", x_q8, tuple(_ptr(t) for t in planes), K, N, 1, y)
+
+
+def gemv_q6_soa_q8(x_q8, planes, K, N, T=1, y=None):
+    """planes = (q6_lo, q6_hi, q6_sc, q6_d) from repack_q6_K_to_soa."""
+    return _gemv_q8("mx_gemv_q6_soa_q8" + ("_batched" if T > 1 else ""), x_q8, tuple(_ptr(t) for t in planes), K, N, T, y)
+
+
+# ---------------------------------------------------------------- host repackers (numpy in, numpy out)
+def _np_u8(a):
+    a = np.ascontiguousarray(a).view(np.uint8).ravel()
+    return a
+
+
+def repack_q4_K_to_reorder(W, K, N):
+    W = _np_u8(W)
+    out = np.empty(N * (K // 256) * 144, np.uint8)
+    _host("mx_repack_q4_K_to_reorder", W.ctypes.data, K, N, out.ctypes.data)
+    return out
+
+
+def repack_moe_kquant_soa(fmt, bank, n_experts, nblocks_per_expert):
+    """fmt in ('q4k', 'q6k'): AoS expert-major bank -> the same regions as per-field streams."""
+    bank = _np_u8(bank)
+    out = np.empty_like(bank)
+    _host("mx_repack_moe_%s_soa_host" % fmt, bank.ctypes.data, out.ctypes.data, n_experts, nblocks_per_expert)
+    return out
+
+
+def repack_q4_K_to_soa(W, K, N):
+    W = _np_u8(W)
+    q = np.empty(N * K // 2, np.uint8)
+    sc, mn = np.empty(N * K // 32, np.int8), np.empty(N * K // 32, np.int8)
+    d, dmin = np.empty(N * K // 256, np.uint16), np.empty(N * K // 256, np.uint16)
+    _host("mx_repack_q4_K_to_soa", W.ctypes.data, K, N, q.ctypes.data, sc.ctypes.data, mn.ctypes.data, d.ctypes.data, dmin.ctypes.data)
+    return q, sc, mn, d, dmin
+
+
+def repack_q6_K_to_soa(W, K, N):
+    W = _np_u8(W)
+    lo, hi = np.empty(N * K // 2, np.uint8), np.empty(N * K // 4, np.uint8)
+    sc, d = np.empty(N * K // 16, np.int8), np.empty(N * K // 256, np.uint16)
+    _host("mx_repack_q6_K_to_soa", W.ctypes.data, K, N, lo.ctypes.data, hi.ctypes.data, sc.ctypes.data, d.ctypes.data)
+    return lo, hi, sc, d
+
+
+def _host(name, *args):
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise MxError(name, rc)
 
 
 def gemv_q4_K_shexp_gate_up(A, W_gate, W_up, W_shg, K, N):

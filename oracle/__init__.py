@@ -267,6 +267,80 @@ def repack_q8_0_to_soa(blocks):
     return qs, d
 
 
+# ---------------------------------------------------------------- K-quant repacks (numpy restatements)
+def repack_kquant_streams(fmt, bank, n_experts, nblocks_per_expert):
+    """Per expert region: the nb blocks' fields gathered into per-field streams, region size unchanged.
+    Q4_K: qs[128] x nb | scales[12] x nb | {d,dmin}[4] x nb; Q6_K: ql[128] x nb | qh[64] x nb |
+    scales[16] x nb | d[2] x nb  (include/ie/quant_soa.hpp:33-51,127-157; with one region and
+    nb = N*K/256 the Q4_K form is repack_q4_K_to_reorder, src/ops/gemv_q8dot.cpp:134-147).
+    Pinned against the reference's own repack_moe_q{4,6}k_soa_host where oracle/_ref is built."""
+    bs = BLOCK_BYTES[fmt]
+    b = _c(bank, np.uint8).reshape(n_experts, nblocks_per_expert, bs)
+    fields = [(16, 144), (4, 16), (0, 4)] if fmt == Q4_K else [(0, 128), (128, 192), (192, 208), (208, 210)]
+    return np.concatenate([b[:, :, lo:hi].reshape(n_experts, -1) for lo, hi in fields], axis=1).ravel()
+
+
+def q4_K_codes(W):
+    """AoS Q4_K blocks -> (q [nb,256] uint8 natural order, sc [nb,8], mn [nb,8], d [nb] u16, dmin [nb] u16);
+    element 64g + 32h + l is nibble h of qs[32g + l] (include/ie/dequant_ref.hpp:38-53)."""
+    b = _c(W, np.uint8).reshape(-1, 144)
+    qs = b[:, 16:].reshape(-1, 4, 32)
+    q = np.stack([qs & 15, qs >> 4], axis=2).reshape(-1, 256)
+    s = b[:, 4:16]
+    sc = np.concatenate([s[:, 0:4] & 63, (s[:, 8:12] & 15) | ((s[:, 0:4] >> 6) << 4)], axis=1)    # get_scale_min_k4, all j at once
+    mn = np.concatenate([s[:, 4:8] & 63, (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)], axis=1)
+    return q, sc, mn, b[:, 0:2].copy().view(np.uint16).ravel(), b[:, 2:4].copy().view(np.uint16).ravel()
+
+
+def q6_K_codes(W):
+    """AoS Q6_K blocks -> (q6u [nb,256] uint8 in 0..63, natural order, sc [nb,16] int8, d [nb] u16);
+    element 128h + 32s + l: low nibble = nibble (s>>1) of ql[64h + 32(s&1) + l], high bits
+    (qh[32h + l] >> 2s) & 3 (include/ie/dequant_ref.hpp:78-96)."""
+    b = _c(W, np.uint8).reshape(-1, 210)
+    ql = b[:, :128].reshape(-1, 2, 2, 32)          # [nb, h, s&1, l]
+    qh = b[:, 128:192].reshape(-1, 2, 1, 32)
+    q = np.empty((b.shape[0], 2, 4, 32), np.uint8)
+    for s_ in range(4):
+        lo = (ql[:, :, s_ & 1] >> 4) if s_ & 2 else (ql[:, :, s_ & 1] & 15)
+        q[:, :, s_] = lo | (((qh[:, :, 0] >> (2 * s_)) & 3) << 4)
+    return q.reshape(-1, 256), b[:, 192:208].copy().view(np.int8), b[:, 208:210].copy().view(np.uint16).ravel()
+
+
+def repack_q4_K_to_soa(W):
+    """-> (q4_q, q4_sc, q4_mn, q4_d, q4_dmin): natural-order nibble plane (element k = nibble k&1 of byte
+    k/2), unpacked per-32 scale / min, per-256 d / dmin (src/ops/gemv_q4_soa.cpp:18-28,115-151)."""
+    q, sc, mn, d, dmin = q4_K_codes(W)
+    return (q[:, 0::2] | (q[:, 1::2] << 4)).ravel(), sc.astype(np.int8).ravel(), mn.astype(np.int8).ravel(), d, dmin
+
+
+def repack_q6_K_to_soa(W):
+    """-> (q6_lo, q6_hi, q6_sc, q6_d): low nibbles two per byte, high bit pairs four per byte (element k =
+    bits 2*(k&3) of byte k/4), per-16 int8 scales, per-256 d (src/ops/gemv_q6_soa.cpp:62-126)."""
+    q, sc, d = q6_K_codes(W)
+    lo, hi = q & 15, q >> 4
+    return ((lo[:, 0::2] | (lo[:, 1::2] << 4)).ravel(), (hi[:, 0::4] | (hi[:, 1::4] << 2) | (hi[:, 2::4] << 4) | (hi[:, 3::4] << 6)).ravel(),
+            sc.ravel(), d)
+
+
+def dequant_q4_soa(planes):
+    """value = (d * s_raw) * q4 - dmin * m_raw in fp32, element order natural (src/ops/gemv_q4_soa.cpp:30-35)."""
+    q, sc, mn, d, dmin = planes
+    codes = np.stack([q & 15, q >> 4], axis=1).reshape(-1, 256).astype(np.float32)
+    d1 = (fp16_to_fp32(d)[:, None] * sc.reshape(-1, 8).astype(np.float32)).astype(np.float32)
+    m1 = (fp16_to_fp32(dmin)[:, None] * mn.reshape(-1, 8).astype(np.float32)).astype(np.float32)
+    return ((np.repeat(d1, 32, axis=1) * codes).astype(np.float32) - np.repeat(m1, 32, axis=1)).astype(np.float32).ravel()
+
+
+def dequant_q6_soa(planes):
+    """value = (d * sc) * (q6u - 32) in fp32 (src/ops/gemv_q6_soa.cpp:415-444)."""
+    lo, hi, sc, d = planes
+    l4 = np.stack([lo & 15, lo >> 4], axis=1).reshape(-1, 256)
+    h2 = np.stack([(hi >> (2 * i)) & 3 for i in range(4)], axis=1).reshape(-1, 256)
+    q = (l4 | (h2 << 4)).astype(np.int32) - 32
+    ds = (fp16_to_fp32(d)[:, None] * sc.reshape(-1, 16).astype(np.float32)).astype(np.float32)
+    return (np.repeat(ds, 16, axis=1) * q.astype(np.float32)).astype(np.float32).ravel()
+
+
 # ---------------------------------------------------------------- the reference, where built
 def load_ref():
     """oracle/_ref/libmxref.so (the reference's own host code) or None when it was not built."""

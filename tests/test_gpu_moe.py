@@ -204,6 +204,10 @@ def test_moe_decode_kquant_fp16_activations(mx, T, E, Kt, H, EF):
     w16 = f16(w)
     idd = dev(ids.astype(np.int32).reshape(-1))
     h = ops.moe_decode_gate_up_silu_q4k(dev(x).half(), dev(Wg), dev(Wu), idd, H, EF, Kt, Wg[0].size, T)
+    # per-expert SoA regions (include/ie/quant_soa.hpp:33-51): same bits, same arithmetic, same result
+    soa = lambda fmt, W: dev(ops.repack_moe_kquant_soa(fmt, W, E, W[0].size // O.BLOCK_BYTES[O.Q4_K if fmt == "q4k" else O.Q6_K]))
+    h_soa = ops.moe_decode_gate_up_silu_q4k(dev(x).half(), soa("q4k", Wg), soa("q4k", Wu), idd, H, EF, Kt, Wg[0].size, T, soa=True)
+    assert torch.equal(h, h_soa)
     h_h = host(h).astype(np.float32)
     h_ref = np.zeros((T * Kt, EF), np.float32)
     for t in range(T):
@@ -216,6 +220,7 @@ def test_moe_decode_kquant_fp16_activations(mx, T, E, Kt, H, EF):
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wd = mk(F, 8500, H, EF)
         y = ops.moe_decode_down_kquant(fmt, h, dev(Wd), idd, dev(w16.reshape(-1)).half(), H, EF, Kt, Wd[0].size, T)
+        assert torch.equal(y, ops.moe_decode_down_kquant(fmt, h, soa(fmt, Wd), idd, dev(w16.reshape(-1)).half(), H, EF, Kt, Wd[0].size, T, soa=True))
         y_ref = np.zeros((T, H), np.float64)
         for t in range(T):
             for k in range(Kt):
@@ -242,6 +247,8 @@ def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wg, Wu = mk(F, 8700, EF, H), mk(F, 8800, EF, H)
         hp = ops.moe_prefill_gate_up_silu_kquant_q8(fmt, xq, dev(Wg), dev(Wu), dev(off), TK, E, H, EF, Wg[0].size)
+        soa = lambda W: dev(ops.repack_moe_kquant_soa(fmt, W, E, W[0].size // O.BLOCK_BYTES[F]))
+        assert torch.equal(hp, ops.moe_prefill_gate_up_silu_kquant_q8(fmt, xq, soa(Wg), soa(Wu), dev(off), TK, E, H, EF, Wg[0].size, soa=True))
         h_ref = np.zeros((TK, EF), np.float32)
         for e in range(E):
             if counts[e]:
@@ -256,6 +263,8 @@ def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wd = mk(F, 8900, H, EF)
         op = ops.moe_prefill_down_packed_kquant_q8(fmt, hq, dev(Wd), dev(off), TK, E, H, EF, Wd[0].size)
+        Wd_soa = dev(ops.repack_moe_kquant_soa(fmt, Wd, E, Wd[0].size // O.BLOCK_BYTES[F]))
+        assert torch.equal(op, ops.moe_prefill_down_packed_kquant_q8(fmt, hq, Wd_soa, dev(off), TK, E, H, EF, Wd[0].size, soa=True))
         o_ref = np.zeros((TK, H), np.float64)
         for e in range(E):
             if counts[e]:
