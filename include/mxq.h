@@ -209,6 +209,15 @@ int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const
  * K % 256 == 0 (Q6_K), K % 128 == 0 (Q8_0); W is the GGUF block stream, 2-byte aligned.  */
 int mx_gemm_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+/* Plain dense GEMM for the dequant-to-Bt route (formats without a fused quant-GEMM: Q5_K, MXFP4):
+ *   gemm_fp16          include/ie/ops.hpp:275-286, src/ops/gemm_fp16.cpp:46-178    C fp32 [M,N]
+ *   gemm_fp16_onednn   include/ie/ops.hpp:460-465, src/ops/gemm_onednn.cpp:75-111  y fp16 [M,N]
+ * A fp16 [M,K] row-major, B fp16 [K,N] row-major (the Bt the mx_dequant_*_to_Bt functions write),
+ * fp32 accumulation.  Argument order (M, N, K) as in the reference.  Both run rocBLAS' gemm_ex (the
+ * reference's second one is a library matmul too); the library is loaded on first use and
+ * MX_ERR_UNSUPPORTED is returned where it is not installed.  */
+int mx_gemm_fp16(mx_stream_t s, const uint16_t* A, const uint16_t* B, float* C, uint32_t M, uint32_t N, uint32_t K);
+int mx_gemm_fp16_onednn(mx_stream_t s, const uint16_t* A, const uint16_t* B, uint16_t* y, uint32_t M, uint32_t N, uint32_t K);
 /* Expert-grouped GEMM over expert-sorted fp16 rows (Q8_0 SoA expert banks): the matrix-core
  * form of moe_prefill_gate_up_silu_q8 / moe_prefill_down_q8 (include/ie/moe_q8.hpp:51-72) for
  * fp16 activations — same arguments except that the activation rows are fp16 instead of

@@ -90,6 +90,13 @@ def dequant_to_Bt(fmt, W, K, N, Bt=None):
     return Bt
 
 
+def gemm_fp16(A, B, M, N, K, out_dtype=torch.float32, C=None):
+    """C[M,N] = A[M,K] . B[K,N] (fp16 operands, fp32 accumulate); fp32 out = gemm_fp16, fp16 out = gemm_fp16_onednn."""
+    C = _out(C, (M, N), out_dtype, A)
+    _call("mx_gemm_fp16" if out_dtype == torch.float32 else "mx_gemm_fp16_onednn", _f16(A), _f16(B), _ptr(C), M, N, K)
+    return C
+
+
 def dequant_soa_to_Bt(name, planes, K, N, Bt=None):
     """name in ('q4_moe_soa', 'q6_K_soa', 'q4_soa', 'q6_soa', 'mxfp4_soa'); planes = device tensors in C-ABI order."""
     Bt = _out(Bt, (K, N), torch.float16, planes[0])

@@ -197,3 +197,31 @@ def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
         y = ops.moe_prefill_reduce(op, dev(t2p.astype(np.uint32)), dev(wp).half(), torch.zeros((T, H), dtype=torch.float16, device="cuda"), T, Kt, H)
         y_ref = (host(op).astype(np.float32) * f16(wp)[:, None])[t2p].reshape(T, Kt, H).sum(axis=1)
         check(host(y).astype(np.float32), y_ref, "prefill_reduce over %s rows" % fmt, max_rel=2e-3)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8, 32), (33, 130, 288), (256, 512, 2048)])
+def test_gemm_fp16_plain(mx, M, N, K):
+    """gemm_fp16 (fp32 C) and gemm_fp16_onednn (fp16 y): A[M,K] . B[K,N], fp32 accumulation
+    (include/ie/ops.hpp:275-286,460-465), against fp64 on the same fp16 operands."""
+    A = O.round_fp16(O.normal(3000 + M, (M, K), 0.0, 1.0))
+    B = O.round_fp16(O.normal(3001 + N, (K, N), 0.0, 0.05))
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    C = mx.ops.gemm_fp16(dev(A).half(), dev(B).half(), M, N, K)
+    check(host(C).ravel(), ref.ravel(), "gemm_fp16 fp32 out", abs_floor=0.0, max_rel=2e-4)
+    y = mx.ops.gemm_fp16(dev(A).half(), dev(B).half(), M, N, K, out_dtype=torch.float16)
+    check(host(y).astype(np.float32).ravel(), ref.ravel(), "gemm_fp16_onednn fp16 out")
+
+
+def test_q5_K_prefill_route(mx):
+    """The reference's Q5_K prefill: dequant_q5_K_to_Bt + gemm_fp16_onednn (include/ie/dequant.hpp:81-86)."""
+    M, N, K = 48, 96, 512
+    W = O.quantize(O.Q4_K, O.normal(3100, (N, K), 0.0, 0.02))
+    # Q5_K blocks from Q4_K ones: same header and nibbles, seeded high bits (the oracle has no Q5_K quantizer)
+    b4 = W.reshape(-1, 144)
+    b5 = np.concatenate([b4[:, :16], O.rand_bytes(3101, b4.shape[0] * 32).reshape(-1, 32), b4[:, 16:]], axis=1)
+    A = O.round_fp16(O.normal(3102, (M, K), 0.0, 1.0))
+    Bt = mx.ops.dequant_to_Bt("q5_K", dev(b5), K, N)
+    wd = O.round_fp16(O.dequant(O.Q5_K, b5)).reshape(N, K)
+    assert np.array_equal(host(Bt).astype(np.float32), wd.T)
+    y = mx.ops.gemm_fp16(dev(A).half(), Bt, M, N, K, out_dtype=torch.float16)
+    check(host(y).astype(np.float32).ravel(), (A.astype(np.float64) @ wd.T.astype(np.float64)).ravel(), "q5_K dequant + gemm_fp16")
