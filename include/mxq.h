@@ -249,6 +249,20 @@ int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* do
 int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
                          const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
                          uint64_t expert_stride_bytes, uint32_t total_rows);
+/* Accumulate form of the down projection (the reference's first prefill path), same matrix-core kernel
+ * with an atomic fp32 epilogue:
+ *   moe_prefill_down_q4k / _q6k       include/ie/ops.hpp:930-954, src/ops/moe_fused.cpp:937-1085
+ *     y_fp32[sorted_token_idx[row], n] += float(sorted_token_w[row]) * (down_e . h_row)[n]; the caller zeroes
+ *     y_fp32; the order of the additions (and so the last bits) is not fixed, as in the reference
+ *   moe_prefill_merge_fp32_to_fp16    include/ie/ops.hpp:956-962, src/ops/moe_fused.cpp:1956-1972
+ *     y_fp16[i] = half(float(y_fp16[i]) + y_fp32[i])  */
+int mx_moe_prefill_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
+                            const int32_t* sorted_token_idx, const uint16_t* sorted_token_w, float* y_fp32, uint32_t E,
+                            uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_prefill_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
+                            const int32_t* sorted_token_idx, const uint16_t* sorted_token_w, float* y_fp32, uint32_t E,
+                            uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows);
+int mx_moe_prefill_merge_fp32_to_fp16(mx_stream_t s, const float* y_fp32, uint16_t* y_fp16, uint64_t n);
 
 /* ---------------------------------------------------------------- MoE, expert-indexed GEMV
  * Q8_0-expert decode kernels (device-resident routing: the expert of token slot

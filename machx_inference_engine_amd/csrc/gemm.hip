@@ -346,6 +346,8 @@ struct GemmArgs {
     half_t* Y;                        // [M, N]
     const uint32_t* expert_offsets;   // grouped: [E+1]
     const half_t* route_w;            // GEMM_MOE_DOWN: [TK] fp16 row weights, or NULL for unweighted rows
+    const int32_t* row_token;         // GEMM_MOE_DOWN, accumulate form: token of each sorted row
+    float* y_acc;                     //   and the fp32 [T, N] buffer w * acc is atomically added into (Y unused)
     uint32_t M, K, N, E;
     uint32_t tiles_m, tiles_n;        // dense tile grid; grouped: tiles_m is an upper bound
 };
@@ -602,7 +604,10 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
                     if (n >= g.N) continue;
                     float o = acc[i][j][v];
                     if (MODE == GEMM_MOE_DOWN && g.route_w) o *= (float)g.route_w[row];
-                    g.Y[(size_t)row * g.N + n] = (half_t)o;
+                    if (MODE == GEMM_MOE_DOWN && g.y_acc)
+                        __hip_atomic_fetch_add(g.y_acc + (size_t)g.row_token[row] * g.N + n, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else
+                        g.Y[(size_t)row * g.N + n] = (half_t)o;
                 }
             }
         }
@@ -666,14 +671,15 @@ static int check_gemm(const void* A, const void* W, const void* y, uint32_t M, u
 template <class QF, int MODE>
 static int moe_gemm_aos(mx_stream_t s, const uint16_t* rows, const void* W0, const void* W1, uint64_t expert_stride_bytes, const uint32_t* expert_offsets,
                         const uint16_t* sorted_w, uint16_t* out, uint32_t E, uint32_t K, uint32_t N, uint32_t total_rows, uint32_t block_bytes,
-                        uint32_t w_align) {
-    if (int rc = check_gemm(rows, W0, out, total_rows, K, N, 256, w_align)) return rc;
+                        uint32_t w_align, const int32_t* row_token = nullptr, float* y_acc = nullptr) {
+    if (int rc = check_gemm(rows, W0, y_acc ? static_cast<const void*>(y_acc) : out, total_rows, K, N, 256, w_align)) return rc;
     MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(expert_offsets);
     MX_REQUIRE_SHAPE(E > 0 && expert_stride_bytes % w_align == 0);
     MX_REQUIRE_ALIGN(W1, w_align);
     GemmArgs g{};
     g.A = reinterpret_cast<const half_t*>(rows); g.Y = reinterpret_cast<half_t*>(out); g.expert_offsets = expert_offsets;
     g.route_w = reinterpret_cast<const half_t*>(sorted_w); g.M = total_rows; g.K = K; g.N = N; g.E = E;
+    g.row_token = row_token; g.y_acc = y_acc;
     const uint32_t row_bytes = K / 256 * block_bytes;
     typename QF::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
     return launch_gemm<QF, MODE>(s, b0, b1, g, total_rows);
@@ -763,6 +769,23 @@ int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* do
                          uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
     return moe_gemm_aos<GemmQ6K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
                                                 total_rows, kQ6KBytes, 2);
+}
+
+// Accumulate form of the down projection (moe_prefill_down_q4k / _q6k, include/ie/ops.hpp:930-954):
+// y_fp32[sorted_token_idx[row], n] += sorted_token_w[row] * (down_e . h_row)[n], fp32 atomics.
+int mx_moe_prefill_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const int32_t* sorted_token_idx,
+                            const uint16_t* sorted_token_w, float* y_fp32, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes,
+                            uint32_t total_rows) {
+    MX_REQUIRE_PTR(sorted_token_idx); MX_REQUIRE_PTR(sorted_token_w); MX_REQUIRE_PTR(y_fp32);
+    return moe_gemm_aos<GemmQ4K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_token_w, nullptr, E, E_ffn, H,
+                                                total_rows, kQ4KBytes, 16, sorted_token_idx, y_fp32);
+}
+int mx_moe_prefill_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const int32_t* sorted_token_idx,
+                            const uint16_t* sorted_token_w, float* y_fp32, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes,
+                            uint32_t total_rows) {
+    MX_REQUIRE_PTR(sorted_token_idx); MX_REQUIRE_PTR(sorted_token_w); MX_REQUIRE_PTR(y_fp32);
+    return moe_gemm_aos<GemmQ6K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_token_w, nullptr, E, E_ffn, H,
+                                                total_rows, kQ6KBytes, 2, sorted_token_idx, y_fp32);
 }
 
 }  // extern "C"

@@ -239,6 +239,12 @@ __global__ __launch_bounds__(256) void scatter_add_kernel(const half_t* x, const
     }
 }
 
+// moe_prefill_merge_fp32_to_fp16 (src/ops/moe_fused.cpp:1956-1972): y16[i] = half(float(y16[i]) + y32[i])
+__global__ __launch_bounds__(256) void merge_f32_kernel(const float* y32, half_t* y16, uint64_t n) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y16[i] = (half_t)((float)y16[i] + y32[i]);
+}
+
 // moe_reduce_q8 (src/ops/moe_q8.cpp:149-158): y[t] = sum_k y_packed[t*K+k]
 // moe_prefill_reduce_sum (:368-384): y[t] = sum_k out_packed[tk_to_packed[t*K+k]]
 // moe_prefill_reduce (src/ops/moe_fused.cpp:1927-1954): y[t] += sum_k w[row] * out_packed[row]
@@ -575,6 +581,12 @@ int mx_moe_scatter_add(mx_stream_t s, const uint16_t* x_packed, const int32_t* i
     hipLaunchKernelGGL(scatter_add_kernel, dim3((hidden + 2047) / 2048, n_tok), dim3(256), 0, as_stream(s),
                        reinterpret_cast<const half_t*>(x_packed), indices, reinterpret_cast<const half_t*>(weights), reinterpret_cast<half_t*>(y),
                        n_tok, hidden);
+    return launch_status();
+}
+int mx_moe_prefill_merge_fp32_to_fp16(mx_stream_t s, const float* y_fp32, uint16_t* y_fp16, uint64_t n) {
+    MX_REQUIRE_PTR(y_fp32); MX_REQUIRE_PTR(y_fp16);
+    MX_REQUIRE_SHAPE(n > 0 && (n + 255) / 256 <= 0x7FFFFFFFull);
+    hipLaunchKernelGGL(merge_f32_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, as_stream(s), y_fp32, reinterpret_cast<half_t*>(y_fp16), n);
     return launch_status();
 }
 static int reduce_common(const void* packed, const void* y, uint32_t T, uint32_t K, uint32_t H) {

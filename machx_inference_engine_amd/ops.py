@@ -288,6 +288,20 @@ def moe_gather_rows(x, indices, n_rows, hidden, y_packed=None):
     return y_packed
 
 
+def moe_prefill_down_kquant_accum(fmt, h_packed, down_W, expert_offsets, sorted_token_idx, sorted_token_w, y_fp32, TK, E, H, E_ffn,
+                                  expert_stride_bytes):
+    """fmt in ('q4k', 'q6k'): y_fp32[token] += w * (down . h) with fp32 atomics (the caller zeroes y_fp32)."""
+    assert y_fp32.dtype == torch.float32
+    _call("mx_moe_prefill_down_%s" % fmt, _f16(h_packed), _u8(down_W), _ptr(expert_offsets), _ptr(sorted_token_idx), _f16(sorted_token_w),
+          _ptr(y_fp32), E, H, E_ffn, expert_stride_bytes, TK)
+    return y_fp32
+
+
+def moe_prefill_merge_fp32_to_fp16(y_fp32, y_fp16):
+    _call("mx_moe_prefill_merge_fp32_to_fp16", _ptr(y_fp32), _f16(y_fp16), y_fp16.numel())
+    return y_fp16
+
+
 def moe_scatter_add(x_packed, indices, weights, y, n_tok, hidden):
     """y[indices[i]] += weights[i] * x_packed[i] in place (rows named by one call must be distinct)."""
     _call("mx_moe_scatter_add", _f16(x_packed), _ptr(indices), _f16(weights), _f16(y), n_tok, hidden)

@@ -197,6 +197,15 @@ def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
         y = ops.moe_prefill_reduce(op, dev(t2p.astype(np.uint32)), dev(wp).half(), torch.zeros((T, H), dtype=torch.float16, device="cuda"), T, Kt, H)
         y_ref = (host(op).astype(np.float32) * f16(wp)[:, None])[t2p].reshape(T, Kt, H).sum(axis=1)
         check(host(y).astype(np.float32), y_ref, "prefill_reduce over %s rows" % fmt, max_rel=2e-3)
+        # accumulate form: fp32 atomics into y_fp32[token], then the fp32 -> fp16 merge (include/ie/ops.hpp:930-962)
+        y32 = torch.zeros((T, H), dtype=torch.float32, device="cuda")
+        ops.moe_prefill_down_kquant_accum(fmt, hp, dev(Wd), dev(off), dev(si.astype(np.int32)), dev(wp).half(), y32, TK, E, H, EF, Wd[0].size)
+        a_ref = np.zeros((T, H), np.float64)
+        np.add.at(a_ref, si, o_ref * f16(wp)[:, None])
+        check(host(y32), a_ref, "moe down %s accumulate form (fp32 atomics)" % fmt, abs_floor=0.0)
+        y0 = f16(O.normal(7200, (T, H)))
+        ym = ops.moe_prefill_merge_fp32_to_fp16(y32, dev(y0).half())
+        assert np.array_equal(host(ym), (y0 + host(y32)).astype(np.float16))
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 32), (33, 130, 288), (256, 512, 2048)])
