@@ -401,6 +401,14 @@ int mx_rms_norm_f32w_q8(mx_stream_t s, const uint16_t* x, const float* w, uint16
                         uint32_t hidden, float eps);
 int mx_gated_rms_norm_q8(mx_stream_t s, const float* x, const uint16_t* z, const uint16_t* weight, uint16_t* y,
                          void* q8_out, uint32_t n_rows, uint32_t hidden, float eps);
+/* Gated activations with the same fused emitter (no counterpart in the reference, which runs swiglu /
+ * swiglu_oai and then quantize_q8_1): y = half(silu(gate) * up) (swiglu, src/ops/elementwise.cpp:449-467)
+ * or the clamped gpt-oss form (swiglu_oai, :469-492; alpha 1.702, limit 7.0 there), and q8_out = the
+ * block_q8_1x stream of the rounded y, bit-identical to mx_quantize_q8_1(y).  y may be NULL when only
+ * the stream is wanted; n % 32 == 0.  */
+int mx_swiglu_q8(mx_stream_t s, const uint16_t* gate, const uint16_t* up, uint16_t* y, void* q8_out, uint64_t n);
+int mx_swiglu_oai_q8(mx_stream_t s, const uint16_t* gate, const uint16_t* up, uint16_t* y, void* q8_out, uint64_t n, float alpha,
+                     float limit);
 
 /* build_moe_packing  src/model/qwen3moe_pack.cpp:5-31 (host pointers): stable counting sort by expert.  */
 int mx_build_moe_packing(const int32_t* topk_ids, const float* topk_w, uint32_t T, uint32_t K, uint32_t E,

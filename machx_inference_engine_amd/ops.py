@@ -485,6 +485,18 @@ def rms_norm_f32w_q8(x, w, eps):
     return y, q8
 
 
+def swiglu_q8(gate, up, oai=False, alpha=1.702, limit=7.0, want_y=True):
+    """-> (y fp16 or None, block_q8_1x stream of y): silu(gate)*up, or the clamped gpt-oss form with oai=True."""
+    n = gate.numel()
+    y = torch.empty_like(gate) if want_y else None
+    q8 = torch.empty(n // 32 * Q81X_BYTES, dtype=torch.uint8, device=gate.device)
+    if oai:
+        _call("mx_swiglu_oai_q8", _f16(gate), _f16(up), _ptr(y), _ptr(q8), n, alpha, limit)
+    else:
+        _call("mx_swiglu_q8", _f16(gate), _f16(up), _ptr(y), _ptr(q8), n)
+    return y, q8
+
+
 def gated_rms_norm_q8(x, z, weight, eps):
     n_rows, hidden = x.shape
     assert x.dtype == torch.float32

@@ -99,3 +99,24 @@ def test_gated_rms_norm_q8(mx, rows, hidden):
     ref = w.astype(np.float64) * (xd / np.sqrt((xd * xd).mean(axis=1, keepdims=True) + eps)) * (zd / (1.0 + np.exp(-zd)))
     check(y_h.astype(np.float32), ref, "gated_rms_norm_q8 y", max_rel=1.5e-3)
     assert np.array_equal(host(q8), ref_q8_of(y_h).reshape(-1))
+
+
+@pytest.mark.parametrize("n", [32, 2880 * 4, 768 * 131])
+@pytest.mark.parametrize("oai", [False, True])
+def test_swiglu_q8(mx, n, oai):
+    """swiglu / swiglu_oai (src/ops/elementwise.cpp:449-492) with the fused block_q8_1x emitter: y against the
+    closed form in fp64, the stream bit-identical to quantize_q8_1 of the rounded y."""
+    g = f16(O.normal(9500 + n, (n,), 0.0, 3.0))        # sigma 3: the OAI clamp at 7 is exercised
+    u = f16(O.normal(9501 + n, (n,), 0.0, 3.0))
+    y, q8 = mx.ops.swiglu_q8(dev(g).half(), dev(u).half(), oai=oai)
+    y_h = host(y)
+    gd, ud = g.astype(np.float64), u.astype(np.float64)
+    if oai:
+        x, z = np.minimum(gd, 7.0), np.clip(ud, -7.0, 7.0)
+        ref = x / (1.0 + np.exp(-1.702 * x)) * (z + 1.0)
+    else:
+        ref = gd / (1.0 + np.exp(-gd)) * ud
+    check(y_h.astype(np.float32), ref, "swiglu%s y" % ("_oai" if oai else ""), max_rel=1.5e-3)
+    assert np.array_equal(host(q8), ref_q8_of(y_h).reshape(-1)), "q8 stream == quantize_q8_1(y)"
+    _, q8_only = mx.ops.swiglu_q8(dev(g).half(), dev(u).half(), oai=oai, want_y=False)
+    assert torch.equal(q8_only, q8)
