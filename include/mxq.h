@@ -37,7 +37,10 @@ enum {
     MX_ERR_SHAPE = 2,       /* a dimension violates the documented precondition */
     MX_ERR_ALIGN = 3,       /* a pointer violates the documented alignment */
     MX_ERR_LAUNCH = 4,      /* the HIP runtime reported an error (see mx_last_hip_error) */
-    MX_ERR_UNSUPPORTED = 5  /* valid arguments, combination not built */
+    MX_ERR_UNSUPPORTED = 5, /* valid arguments, combination not built */
+    MX_ERR_IO = 6,          /* a file could not be opened or mapped (see mx_gguf_last_error) */
+    MX_ERR_FORMAT = 7,      /* a file is not what its format prescribes (see mx_gguf_last_error) */
+    MX_ERR_NOT_FOUND = 8    /* no tensor / key of that name */
 };
 
 const char* mx_status_string(int status);
@@ -438,6 +441,44 @@ int mx_repack_q4_K_to_soa(const void* W_blocks, uint32_t K, uint32_t N, uint8_t*
                           uint16_t* q4_d, uint16_t* q4_dmin);
 int mx_repack_q6_K_to_soa(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* q6_lo, uint8_t* q6_hi, int8_t* q6_sc,
                           uint16_t* q6_d);
+
+/* ---------------------------------------------------------------- GGUF reader (host)
+ * Memory-mapped reader of GGUF v2 / v3 files, the on-disk form of every weight this library takes:
+ * GgufReader  include/ie/gguf.hpp:72-117, src/loaders/gguf_reader.cpp.  Tensor data is not copied;
+ * `data` points into the mapping (valid until mx_gguf_close) at the GGUF block layout, i.e. exactly
+ * what the AoS kernels and the mx_repack_* functions read.  Split models: open the first shard
+ * ("...-00001-of-0000N.gguf"); the other shards are mapped too and their tensors appended.
+ * Strings are not NUL-terminated: use the length.  A kv payload points at the scalar, at a string's
+ * u64 length followed by its bytes, or at an array's first element (strings in arrays likewise
+ * length-prefixed).  ggml_type ids as in ggml (Q4_0 2, Q8_0 8, Q4_K 12, Q5_K 13, Q6_K 14, MXFP4 39...);
+ * nbytes is 0 for a type this reader does not size.  */
+typedef struct {
+    const char* name;
+    uint64_t name_len;
+    uint32_t ggml_type;
+    uint32_t n_dims;
+    uint64_t shape[4];          /* shape[0] is the contiguous (K) dimension; unused dims are 1 */
+    uint64_t offset_in_data;
+    uint64_t nbytes;
+    const void* data;
+} mx_gguf_tensor_t;
+typedef struct {
+    const char* key;
+    uint64_t key_len;
+    uint32_t type;              /* 0 u8, 1 i8, 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool, 8 string, 9 array, 10 u64, 11 i64, 12 f64 */
+    uint32_t inner_type;        /* arrays: element type */
+    uint64_t n_array;           /* arrays: element count */
+    const void* payload;
+} mx_gguf_kv_t;
+int mx_gguf_open(const char* path, void** handle);
+int mx_gguf_close(void* handle);
+int mx_gguf_info(const void* handle, uint32_t* version, uint64_t* n_tensors, uint64_t* n_kv, uint64_t* alignment,
+                 uint64_t* tensor_data_offset);
+int mx_gguf_tensor(const void* handle, uint64_t i, mx_gguf_tensor_t* out);
+int mx_gguf_find_tensor(const void* handle, const char* name, uint64_t* index);
+int mx_gguf_kv(const void* handle, uint64_t i, mx_gguf_kv_t* out);
+int mx_gguf_find_kv(const void* handle, const char* key, uint64_t* index);
+const char* mx_gguf_last_error(void);   /* text of the last MX_ERR_IO / MX_ERR_FORMAT on this thread */
 
 #ifdef __cplusplus
 }

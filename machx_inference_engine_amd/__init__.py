@@ -9,4 +9,5 @@ from . import _lib
 lib = _lib.load()
 
 from . import ops  # noqa: E402
+from . import gguf  # noqa: E402,F401
 from .ops import MxError  # noqa: E402,F401

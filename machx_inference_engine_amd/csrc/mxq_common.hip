@@ -15,6 +15,9 @@ const char* mx_status_string(int status) {
         case MX_ERR_ALIGN: return "pointer violates the required alignment";
         case MX_ERR_LAUNCH: return "HIP runtime error";
         case MX_ERR_UNSUPPORTED: return "combination not built";
+        case MX_ERR_IO: return "file could not be opened or mapped";
+        case MX_ERR_FORMAT: return "file violates its format";
+        case MX_ERR_NOT_FOUND: return "no entry of that name";
     }
     return "unknown status";
 }

@@ -415,6 +415,20 @@ def repack_q6_K_to_soa(W, K, N):
     return lo, hi, sc, d
 
 
+def repack_block32_to_soa(fmt, blocks):
+    """fmt 'q8_0' -> (qs int8, d uint16); 'mxfp4' -> (qs uint8, e uint8)."""
+    blocks = _np_u8(blocks)
+    if fmt == "q8_0":
+        nb = blocks.size // 34
+        qs, d = np.empty(nb * 32, np.int8), np.empty(nb, np.uint16)
+        _host("mx_repack_q8_0_to_soa", blocks.ctypes.data, nb, qs.ctypes.data, d.ctypes.data)
+        return qs, d
+    nb = blocks.size // 17
+    qs, e = np.empty(nb * 16, np.uint8), np.empty(nb, np.uint8)
+    _host("mx_repack_mxfp4_to_soa", blocks.ctypes.data, nb, qs.ctypes.data, e.ctypes.data)
+    return qs, e
+
+
 def _host(name, *args):
     rc = getattr(lib, name)(*args)
     if rc != 0:
