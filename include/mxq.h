@@ -81,6 +81,14 @@ int mx_dequant_q4_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K
 int mx_dequant_q5_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_q6_K_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
 int mx_dequant_mxfp4_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+/* Q4_0 (Gemma-4 QAT; 18-byte blocks {fp16 d; u8 qs[16]}, w = d * (q - 8), element j in the low and j + 16
+ * in the high nibble of qs[j]; include/ie/quant_blocks.hpp:32-43):
+ *   dequant_q4_0_to_Bt / dequant_q4_0_soa_to_Bt   include/ie/ops.hpp:550-567, src/ops/gemv_q4_0.cpp:455-477
+ * (the flat forms have no counterpart in the reference and exist for symmetry with the other formats)  */
+int mx_dequant_q4_0(mx_stream_t s, const void* packed, uint16_t* out_f16, uint64_t n_elements);
+int mx_dequant_q4_0_f32(mx_stream_t s, const void* packed, float* out, uint64_t n_elements);
+int mx_dequant_q4_0_to_Bt(mx_stream_t s, const void* W, uint16_t* Bt, uint32_t K, uint32_t N);
+int mx_dequant_q4_0_soa_to_Bt(mx_stream_t s, const uint8_t* soa_qs, const uint16_t* soa_d, uint16_t* Bt, uint32_t K, uint32_t N);
 /* Transposed dequant of the repacked layouts; bit-identical to the AoS form of the same weights:
  *   dequant_q4_moe_soa_to_Bt   include/ie/dequant.hpp:72-80   one expert region as streams qs | scales | {d,dmin}
  *   dequant_q6_K_soa_to_Bt     include/ie/dequant.hpp:64-71   one expert region as streams ql | qh | scales | d
@@ -142,6 +150,28 @@ int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint
 int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W,
                                 uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* Sibling formats on the same kernels.
+ * Q4_0:
+ *   gemv_q4_0                 include/ie/ops.hpp:525-529, src/ops/gemv_q4_0.cpp:54-120   fp16 activations, GGUF blocks
+ *   gemv_q4_0_soa_q8          include/ie/ops.hpp:573-576, src/ops/gemv_q4_0.cpp:194-270  planes q4_qs[n*(K/2)+16b+j], q4_d[n*(K/32)+b]
+ *   gemv_q4_0_soa_q8_batched  include/ie/ops.hpp:597-601  (T <= 16 here; the reference stops at 8)
+ *   gemv_q4_0_soa_q8_multi    include/ie/ops.hpp:577-592: up to 3 banks of different N sharing x_q8, one launch;
+ *                             qs / d / y / N are HOST arrays of n_banks entries (device pointers, row counts)
+ *   mx_gemv_q4_0_q8_batched   int-dot over the GGUF blocks themselves (no counterpart: the reference repacks first)
+ *   fold: acc += d * (d8 * idot - 8 * s), K % 32 == 0.
+ * Q5_K (no GEMV in the reference, which dequantizes Q5_K tensors and runs the dense GEMM; include/ie/dequant.hpp:81-86):
+ *   the Q4_K kernels with the fifth bit from qh; K % 256 == 0, W 16-byte aligned.  */
+int mx_gemv_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q4_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_q4_0_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q4_qs, const uint16_t* q4_d, uint16_t* y, uint32_t K,
+                        uint32_t N);
+int mx_gemv_q4_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q4_qs, const uint16_t* q4_d, uint16_t* y,
+                                uint32_t K, uint32_t N, uint32_t T);
+int mx_gemv_q4_0_soa_q8_multi(mx_stream_t s, const void* x_q8, const uint8_t* const* qs, const uint16_t* const* d,
+                              uint16_t* const* y, const uint32_t* N, int n_banks, uint32_t K);
+int mx_gemv_q5_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q5_K_q8(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q5_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 /* Int-dot GEMV over the repacked K-quant layouts (written by the mx_repack_* host functions below):
  *   gemv_q4_K_reorder_q8     include/ie/ops.hpp:322-326, src/ops/gemv_q8dot.cpp:152-256   three-region streams
  *   gemv_q4_soa_q8           include/ie/ops.hpp:444-451, src/ops/gemv_q4_soa.cpp:160-312  natural-order planes
@@ -212,6 +242,9 @@ int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const
  * K % 256 == 0 (Q6_K), K % 128 == 0 (Q8_0); W is the GGUF block stream, 2-byte aligned.  */
 int mx_gemm_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+/* Q4_0 weights through the same kernel: gemm_q4_0 / gemm_q4_0_xmx  include/ie/ops.hpp:530-534, src/ops/gemv_q4_0.cpp,
+ * src/ops/gemm_q4k_xmx.cpp:418-522; K % 128 == 0, W 2-byte aligned.  */
+int mx_gemm_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 /* Plain dense GEMM for the dequant-to-Bt route (formats without a fused quant-GEMM: Q5_K, MXFP4):
  *   gemm_fp16          include/ie/ops.hpp:275-286, src/ops/gemm_fp16.cpp:46-178    C fp32 [M,N]
  *   gemm_fp16_onednn   include/ie/ops.hpp:460-465, src/ops/gemm_onednn.cpp:75-111  y fp16 [M,N]
@@ -434,6 +467,8 @@ int mx_repack_q8_0_to_soa(const void* blocks, uint64_t n_blocks, int8_t* qs_plan
  *   repack_q6_K_to_soa        include/ie/ops.hpp:393-399, src/ops/gemv_q6_soa.cpp:71-126
  *     q6_lo N*K/2 (low nibbles), q6_hi N*K/4 (element k = bits 2*(k&3) of byte k/4), q6_sc N*K/16 int8,
  *     q6_d N*K/256 fp16 bits; unlike the reference's, the planes need not be zeroed first  */
+/* repack_q4_0_to_soa  include/ie/ops.hpp:571-572, src/ops/gemv_q4_0.cpp:179-192: q4_qs N*K/2 bytes, q4_d N*K/32 fp16 bits */
+int mx_repack_q4_0_to_soa(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* q4_qs, uint16_t* q4_d);
 int mx_repack_q4_K_to_reorder(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* out);
 int mx_repack_moe_q4k_soa_host(const void* src, void* dst, uint32_t n_experts, uint64_t nblocks_per_expert);
 int mx_repack_moe_q6k_soa_host(const void* src, void* dst, uint32_t n_experts, uint64_t nblocks_per_expert);

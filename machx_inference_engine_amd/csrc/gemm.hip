@@ -258,6 +258,71 @@ struct GemmQ8Aos {
     }
 };
 
+// Q4_0 AoS GGUF blocks (18 B: fp16 d, 16 bytes of nibbles; element j in the low, j + 16 in the high
+// nibble of qs[j]; include/ie/quant_blocks.hpp:32-43): lane half h owns blocks 4 kc + 2h and + 1, 36
+// contiguous bytes at a 2-byte aligned address, fetched as 9 dwords.  Step S covers elements
+// 8 (S%4) .. +7 of block S/4: the low nibbles of quant words 2 (S%2), 2 (S%2) + 1 for S%4 < 2, their high
+// nibbles otherwise.  value = half(d * (q - 8)) = fma(q * 2^-24, d * 2^24, -8 d), exact in fp32.
+struct GemmQ40 {
+    struct W {
+        const uint8_t* base;
+        uint32_t row_bytes;
+    };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
+    struct Raw {
+        uint32_t w[9];
+    };
+    struct Dec {
+        float d[2], o[2];
+    };
+    static constexpr uint32_t K_ALIGN = 128;
+    static constexpr uint32_t H_COL = 8;
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)S; }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
+        const uint8_t* p = w.base + (size_t)n * w.row_bytes + (size_t)(4u * kc + 2u * h) * 18u;
+        Raw r;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint4 v = load_u4_a2(p + 16 * i);
+            r.w[4 * i] = v.x; r.w[4 * i + 1] = v.y; r.w[4 * i + 2] = v.z; r.w[4 * i + 3] = v.w;
+        }
+        r.w[8] = load_u1_a2(p + 32);
+        return r;
+    }
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t, uint32_t) {
+        Dec o;
+        o.d[0] = h2f(r.w[0] & 0xFFFFu);
+        o.d[1] = h2f(r.w[4] >> 16);
+        o.o[0] = -8.f * o.d[0];
+        o.o[1] = -8.f * o.d[1];
+        o.d[0] *= 16777216.f;
+        o.d[1] *= 16777216.f;
+        return o;
+    }
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int blk = S / 4, j = 2 * (S % 2) + HF, hi = (S % 4) / 2;   // quant word j of the block, nibble half
+        uint32_t w;
+        if (blk == 0) w = __builtin_amdgcn_alignbyte(r.w[j + 1], r.w[j], 2);   // bytes 2 + 4j .. 5 + 4j
+        else w = r.w[5 + j];                                                   // bytes 20 + 4j ..
+        const uint32_t code = (hi ? w >> 4 : w) & 0x0F0F0F0Fu;
+        const float d = dc.d[blk], o = dc.o[blk];
+        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, code, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, code, 0x0C030C02u));
+        f.u[2 * HF] = mix_pair(w01.x, w01.y, d, o);
+        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, d, o);
+    }
+    template <int S>
+    __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
+    }
+};
+
 // Q6_K (210-byte AoS blocks, 2-byte aligned): chunk kc = 128-element half c = kc%2 of block
 // kc/2.  Lane half j = lane/32 owns the 16 "l" positions 16j .. 16j+15 of that half, i.e. the
 // four 16-element groups 32s + 16j + [0,16), s = 0..3 (include/ie/dequant_ref.hpp:78-96):
@@ -713,6 +778,14 @@ int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, u
     g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
     GemmQ8Aos::Bank b{static_cast<const uint8_t*>(W), 0, K / 32 * (uint32_t)kQ8_0Bytes};
     return launch_gemm<GemmQ8Aos, GEMM_DENSE>(s, b, b, g, M);
+}
+
+int mx_gemm_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    if (int rc = check_gemm(A, W, y, M, K, N, 128, 2)) return rc;
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
+    GemmQ40::Bank b{static_cast<const uint8_t*>(W), 0, K / 32 * 18u};
+    return launch_gemm<GemmQ40, GEMM_DENSE>(s, b, b, g, M);
 }
 
 int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {

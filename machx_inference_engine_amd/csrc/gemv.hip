@@ -68,6 +68,49 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
     }
 }
 
+// Up to three matrices of different N that share one quantized activation row, in one launch: the
+// workgroups tile the concatenated row space, so small projections (GQA k / v) ride a full grid
+// (gemv_q4_0_soa_q8_multi, include/ie/ops.hpp:577-592).  T = 1.
+template <class F>
+struct GemvBanks {
+    typename F::W w[3];
+    half_t* y[3];
+    uint32_t rg_end[3];   // cumulative row-group counts
+    uint32_t n[3];
+};
+template <class F, int G>
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_multi_kernel(GemvBanks<F> bk, const uint8_t* xq8, uint32_t K, uint32_t KT, int n_banks) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G, U = 2;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    auto xrow = [&](uint32_t) { return xq8; };
+    const uint32_t n_tiles = (K + KT - 1) / KT;
+    const uint32_t total_rg = bk.rg_end[n_banks - 1];
+    ActTile act;
+    bool staged = false;
+    for (uint32_t rg = blockIdx.x; rg < total_rg; rg += gridDim.x) {
+        const int b = (rg < bk.rg_end[0]) ? 0 : (rg < bk.rg_end[1] ? 1 : 2);
+        const uint32_t N = bk.n[b];
+        const uint32_t row = (rg - (b ? bk.rg_end[b - 1] : 0u)) * ROWS_PER_WG + wave * GROUPS + grp;
+        float acc[1][1] = {{0.f}};
+        for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+            const uint32_t k0 = tile * KT, kt = (K - k0 < KT) ? K - k0 : KT;
+            typename F::Cursor cu[1] = {F::cursor(bk.w[b], row < N ? row : N - 1, k0 / 64 + gl)};
+            if (n_tiles > 1 || !staged) {
+                __syncthreads();
+                act = stage_act<F::SUM_GRAN, 1>(lds, xrow, k0, kt, KT, false);
+                __syncthreads();
+                staged = true;
+            }
+            gemv_rows<F, 1, 1, G, U>(cu, (kt + 63) / 64, (kt & 63u) != 0, gl, act, acc);
+        }
+        const float v = group_sum<G>(acc[0][0]);
+        if (lane == (uint32_t)group_sum_lane<G>(lane) && row < N) store_out(bk.y[b] + row, v);
+    }
+}
+
 // ---------------------------------------------------------------- float activations (T = 1)
 // Same unit walk; activations staged as fp32 plus per-16 sums; the fold is the
 // reference's acc += (d*sc) * sum(a*q) - (dmin*m) * sum(a)  (src/ops/gemv_q4k.cpp:119-146).
@@ -416,6 +459,85 @@ int mx_gemv_q6_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q6
 int mx_gemv_q6_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc, const uint16_t* q6_d,
                       uint16_t* y, uint32_t K, uint32_t N) {
     return mx_gemv_q6_soa_q8_batched(s, x_q8, q6_lo, q6_hi, q6_sc, q6_d, y, K, N, 1);
+}
+
+// ---------------------------------------------------------------- Q4_0 (Gemma-4 QAT) and Q5_K
+int mx_gemv_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y, K, N, 1, 32)) return rc;
+    MX_REQUIRE_PTR(W);
+    MX_REQUIRE_ALIGN(W, 2);
+    return launch_fact<FmtQ40Aos>(s, FmtQ40Aos::W{static_cast<const uint8_t*>(W), K / 32 * 18u}, reinterpret_cast<const half_t*>(A),
+                                  reinterpret_cast<half_t*>(y), K, N);
+}
+int mx_gemv_q4_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    if (int rc = check_common(x_q8, y, K, N, T, 32)) return rc;
+    MX_REQUIRE_PTR(W);
+    MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(W, 2);
+    GemvSeg<FmtQ40Aos, half_t> g{{static_cast<const uint8_t*>(W), K / 32 * 18u}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtQ40Aos, half_t>(s, g, g, 1, x_q8, K, N, T);
+}
+int mx_gemv_q4_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q4_qs, const uint16_t* q4_d, uint16_t* y, uint32_t K, uint32_t N,
+                                uint32_t T) {
+    if (int rc = check_common(x_q8, y, K, N, T, 32)) return rc;
+    MX_REQUIRE_PTR(q4_qs); MX_REQUIRE_PTR(q4_d);
+    MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(q4_qs, 16); MX_REQUIRE_ALIGN(q4_d, 2);
+    GemvSeg<FmtQ40Soa, half_t> g{{q4_qs, q4_d, K}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtQ40Soa, half_t>(s, g, g, 1, x_q8, K, N, T);
+}
+int mx_gemv_q4_0_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q4_qs, const uint16_t* q4_d, uint16_t* y, uint32_t K, uint32_t N) {
+    return mx_gemv_q4_0_soa_q8_batched(s, x_q8, q4_qs, q4_d, y, K, N, 1);
+}
+int mx_gemv_q4_0_soa_q8_multi(mx_stream_t s, const void* x_q8, const uint8_t* const* qs, const uint16_t* const* d, uint16_t* const* y,
+                              const uint32_t* N, int n_banks, uint32_t K) {
+    MX_REQUIRE_PTR(x_q8); MX_REQUIRE_PTR(qs); MX_REQUIRE_PTR(d); MX_REQUIRE_PTR(y); MX_REQUIRE_PTR(N);
+    MX_REQUIRE_SHAPE(n_banks >= 1 && n_banks <= 3 && K > 0 && K % 32 == 0);
+    MX_REQUIRE_ALIGN(x_q8, 8);
+    const uint32_t G = pick_group((K + 63) / 64);
+    const uint32_t rows_per_wg = kGemvWaves * (64 / G);
+    GemvBanks<FmtQ40Soa> bk{};
+    uint32_t total = 0;
+    for (int b = 0; b < 3; ++b) {
+        const int src = b < n_banks ? b : n_banks - 1;
+        if (b < n_banks) {
+            MX_REQUIRE_PTR(qs[b]); MX_REQUIRE_PTR(d[b]); MX_REQUIRE_PTR(y[b]);
+            MX_REQUIRE_SHAPE(N[b] > 0);
+            MX_REQUIRE_ALIGN(qs[b], 16); MX_REQUIRE_ALIGN(d[b], 2);
+            total += (N[b] + rows_per_wg - 1) / rows_per_wg;
+        }
+        bk.w[b] = {qs[src], d[src], K};
+        bk.y[b] = reinterpret_cast<half_t*>(y[src]);
+        bk.n[b] = N[src];
+        bk.rg_end[b] = total;
+    }
+    const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(FmtQ40Soa::SUM_GRAN);
+    const uint32_t KT_max = (kLdsBudget / per_elem_x32) * 32 / 256 * 256;
+    const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
+    const uint32_t KT = (K256 + n_tiles - 1) / n_tiles * 256;
+    const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu;
+    const dim3 grid(total < cap ? total : cap);
+    const uint32_t lds = act_tile_bytes(1, KT, FmtQ40Soa::SUM_GRAN);
+    const uint8_t* x = static_cast<const uint8_t*>(x_q8);
+    if (G == 16) hipLaunchKernelGGL((gemv_q8_multi_kernel<FmtQ40Soa, 16>), grid, dim3(kGemvThreads), lds, as_stream(s), bk, x, K, KT, n_banks);
+    else if (G == 32) hipLaunchKernelGGL((gemv_q8_multi_kernel<FmtQ40Soa, 32>), grid, dim3(kGemvThreads), lds, as_stream(s), bk, x, K, KT, n_banks);
+    else hipLaunchKernelGGL((gemv_q8_multi_kernel<FmtQ40Soa, 64>), grid, dim3(kGemvThreads), lds, as_stream(s), bk, x, K, KT, n_banks);
+    return launch_status();
+}
+int mx_gemv_q5_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T) {
+    if (int rc = check_common(x_q8, y, K, N, T, 256)) return rc;
+    MX_REQUIRE_PTR(W);
+    MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(W, 16);
+    GemvSeg<FmtQ5K, half_t> g{{static_cast<const uint8_t*>(W), K / 256 * 176u}, reinterpret_cast<half_t*>(y), nullptr};
+    return launch_q8<FmtQ5K, half_t>(s, g, g, 1, x_q8, K, N, T);
+}
+int mx_gemv_q5_K_q8(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return mx_gemv_q5_K_q8_batched(s, x_q8, W, y, K, N, 1);
+}
+int mx_gemv_q5_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(A, y, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(W);
+    MX_REQUIRE_ALIGN(W, 16);
+    return launch_fact<FmtQ5K>(s, FmtQ5K::W{static_cast<const uint8_t*>(W), K / 256 * 176u}, reinterpret_cast<const half_t*>(A),
+                               reinterpret_cast<half_t*>(y), K, N);
 }
 
 int mx_gemv_mxfp4_soa_q8_batched(mx_stream_t s, const void* x, const uint8_t* qs, const uint8_t* e, uint16_t* y, uint32_t K, uint32_t N,

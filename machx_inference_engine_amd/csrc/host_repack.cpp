@@ -29,6 +29,19 @@ int mx_repack_q8_0_to_soa(const void* blocks, uint64_t n_blocks, int8_t* qs_plan
     return MX_OK;
 }
 
+// block_q4_0 {fp16 d; u8 qs[16]} -> qs_plane[16*i + j], d_plane[i]   (reference: src/ops/gemv_q4_0.cpp:179-192)
+int mx_repack_q4_0_to_soa(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* q4_qs, uint16_t* q4_d) {
+    if (!W_blocks || !q4_qs || !q4_d) return MX_ERR_NULL;
+    if (K == 0 || K % 32) return MX_ERR_SHAPE;
+    const uint8_t* b = static_cast<const uint8_t*>(W_blocks);
+    const uint64_t nb = (uint64_t)N * (K / 32);
+    for (uint64_t i = 0; i < nb; ++i, b += 18) {
+        memcpy(q4_d + i, b, 2);
+        memcpy(q4_qs + 16 * i, b + 2, 16);
+    }
+    return MX_OK;
+}
+
 // block_q4_K {fp16 d; fp16 dmin; u8 scales[12]; u8 qs[128]} x nb  ->  qs x nb | scales x nb | {d,dmin} x nb
 // over all nb = N*K/256 blocks of a matrix (reference: src/ops/gemv_q8dot.cpp:134-147).
 int mx_repack_q4_K_to_reorder(const void* W_blocks, uint32_t K, uint32_t N, uint8_t* out) {

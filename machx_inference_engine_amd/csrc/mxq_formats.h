@@ -543,6 +543,161 @@ struct FmtQ8Aos {
     }
 };
 
+// ---------------------------------------------------------------- Q4_0
+// {fp16 d; u8 qs[16]} per 32 elements, element j in the low and j + 16 in the high nibble of qs[j],
+// w = d * (q - 8) (include/ie/quant_blocks.hpp:32-43).  Codes stay unsigned; the -8 goes into the
+// min term against the activation block's sum: acc += d * (d8 * idot - 8 * s), the reference's fold
+// (src/ops/gemv_q4_0.cpp:194-197).  Unit u = blocks 2u, 2u+1.
+// SoA planes: q4_qs[n*(K/2) + 16b + j], q4_d[n*(K/32) + b] (repack_q4_0_to_soa, :179-192).
+struct FmtQ40Soa {
+    struct W {
+        const uint8_t* qs;
+        const uint16_t* d;
+        uint32_t K;
+    };
+    struct Cursor {
+        const uint4* qs;
+        const uint8_t* d;
+    };
+    struct Raw {
+        uint4 qa, qb;
+        uint32_t d2;
+    };
+    static constexpr int SUM_GRAN = 32;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
+    static constexpr uint32_t K_ALIGN = 32;
+    static constexpr bool CODES_UNSIGNED = true;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {reinterpret_cast<const uint4*>(w.qs + (size_t)n * (w.K >> 1) + (size_t)u * 32u),
+                reinterpret_cast<const uint8_t*>(w.d + (size_t)n * (w.K >> 5) + 2u * u)};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool half_only = false) {
+        const uint4* p = cu.qs + (size_t)i * (G * 2);
+        const uint8_t* d = cu.d + (size_t)i * (G * 4);
+        Raw r;
+        r.qa = p[0];
+        if (half_only) {
+            r.qb = make_uint4(0, 0, 0, 0);
+            r.d2 = *reinterpret_cast<const uint16_t*>(d);
+        } else {
+            r.qb = p[1];
+            r.d2 = load_u1_a2(d);
+        }
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
+        const uint32_t a[4] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w}, b[4] = {r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o.q[0][i] = a[i] & 0x0F0F0F0Fu;
+            o.q[1][i] = (a[i] >> 4) & 0x0F0F0F0Fu;
+            o.q[2][i] = b[i] & 0x0F0F0F0Fu;
+            o.q[3][i] = (b[i] >> 4) & 0x0F0F0F0Fu;
+        }
+        o.c[0] = o.c[1] = h2f(r.d2 & 0xFFFFu);
+        o.c[2] = o.c[3] = h2f(r.d2 >> 16);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) o.m[g] = 8.f * o.c[g];
+    }
+};
+
+// Q4_0 as GGUF blocks (18 B, 2-byte aligned): one lane per block pair, 36 contiguous bytes.
+struct FmtQ40Aos {
+    struct W {
+        const uint8_t* base;
+        uint32_t row_bytes;
+    };
+    struct Cursor {
+        const uint8_t* blk;
+    };
+    typedef FmtQ40Soa::Raw Raw;
+    static constexpr int SUM_GRAN = 32;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
+    static constexpr uint32_t K_ALIGN = 32;
+    static constexpr bool CODES_UNSIGNED = true;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) { return {w.base + (size_t)n * w.row_bytes + (size_t)u * 36u}; }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool half_only = false) {
+        const uint8_t* blk = cu.blk + (size_t)i * (G * 36);
+        Raw r;
+        r.d2 = *reinterpret_cast<const uint16_t*>(blk);
+        r.qa = load_u4_a2(blk + 2);
+        if (half_only) {
+            r.qb = make_uint4(0, 0, 0, 0);
+        } else {
+            r.d2 |= (uint32_t)*reinterpret_cast<const uint16_t*>(blk + 18) << 16;
+            r.qb = load_u4_a2(blk + 20);
+        }
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) { FmtQ40Soa::decode(r, FmtQ40Soa::Cursor{}, o); }
+};
+
+// ---------------------------------------------------------------- Q5_K (AoS GGUF blocks)
+// {d, dmin, scales[12], qh[32], qs[128]} (176 B; include/ie/quant_blocks.hpp:79-85): Q4_K plus a fifth
+// bit, bit 2g + hi of qh[l] for element 64g + 32hi + l (include/ie/dequant_ref.hpp:55-75).  Units, scales
+// and fold as Q4_K; the unit also reads the whole qh (32 bytes) and picks its two bit planes.
+struct FmtQ5K {
+    struct W {
+        const uint8_t* base;
+        uint32_t row_bytes;
+    };
+    struct Cursor {
+        const uint8_t* blk;
+        uint32_t g;
+    };
+    struct Raw {
+        uint4 hdr, h0, h1, q0, q1;
+    };
+    static constexpr int SUM_GRAN = 32;
+    static constexpr bool PAIRED = true;
+    static constexpr uint32_t GROUP_OFF = 16;
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr bool CODES_UNSIGNED = true;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return u * 64u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {w.base + (size_t)n * w.row_bytes + (size_t)(u >> 2) * 176u, u & 3u};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i) {
+        const uint8_t* blk = cu.blk + (size_t)i * (G / 4 * 176);
+        const uint4* h = reinterpret_cast<const uint4*>(blk + 16);
+        const uint4* q = reinterpret_cast<const uint4*>(blk + 48 + cu.g * 32u);
+        Raw r;
+        r.hdr = *reinterpret_cast<const uint4*>(blk);
+        r.h0 = h[0];
+        r.h1 = h[1];
+        r.q0 = q[0];
+        r.q1 = q[1];
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) {
+        const uint32_t q0[4] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w}, q1[4] = {r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t h0[4] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w}, h1[4] = {r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+        const uint32_t sh = 2u * cu.g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // bit (2g) of each qh byte -> bit 4 of the low-nibble code, bit (2g+1) -> of the high-nibble code
+            o.q[0][i] = (q0[i] & 0x0F0F0F0Fu) | (((h0[i] >> sh) & 0x01010101u) << 4);
+            o.q[1][i] = (q1[i] & 0x0F0F0F0Fu) | (((h1[i] >> sh) & 0x01010101u) << 4);
+            o.q[2][i] = ((q0[i] >> 4) & 0x0F0F0F0Fu) | (((h0[i] >> (sh + 1u)) & 0x01010101u) << 4);
+            o.q[3][i] = ((q1[i] >> 4) & 0x0F0F0F0Fu) | (((h1[i] >> (sh + 1u)) & 0x01010101u) << 4);
+        }
+        uint32_t sc, mn;
+        q4k_scale_pair(r.hdr.y, r.hdr.z, r.hdr.w, (int)cu.g, sc, mn);
+        const float d = h2f(r.hdr.x & 0xFFFFu), dmin = h2f(r.hdr.x >> 16);
+        o.c[0] = o.c[1] = d * (float)(sc & 0xFFu);
+        o.c[2] = o.c[3] = d * (float)(sc >> 8);
+        o.m[0] = o.m[1] = dmin * (float)(mn & 0xFFu);
+        o.m[2] = o.m[3] = dmin * (float)(mn >> 8);
+    }
+};
+
 // ---------------------------------------------------------------- MXFP4, SoA planes
 // qs_plane[n*(K/2) + 16b + j], e_plane[n*(K/32) + b] (src/ops/gemv_mxfp4.cpp:13-16).
 // Unit u = blocks 2u, 2u+1: 32 bytes of codes (per block: low nibbles = elements

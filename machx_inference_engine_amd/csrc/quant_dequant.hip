@@ -75,7 +75,7 @@ static int quantize_launch(mx_stream_t s, const ActT* x, void* out, uint64_t n) 
 // (include/ie/dequant_ref.hpp:32-96): the fp32 result is bit-identical for every
 // association because each partial product is exact (11-bit d times <= 12-bit
 // integer); only Q4_K's final subtraction rounds, once, fused or not.
-enum { FMT_Q8_0 = 0, FMT_Q4_K = 1, FMT_Q6_K = 2, FMT_MXFP4 = 3, FMT_Q5_K = 4 };
+enum { FMT_Q8_0 = 0, FMT_Q4_K = 1, FMT_Q6_K = 2, FMT_MXFP4 = 3, FMT_Q5_K = 4, FMT_Q4_0 = 5 };
 
 template <int FMT>
 struct BlockInfo;
@@ -89,6 +89,8 @@ template <>
 struct BlockInfo<FMT_MXFP4> { static constexpr uint32_t elems = 32, bytes = kMxfp4Bytes; };
 template <>
 struct BlockInfo<FMT_Q5_K> { static constexpr uint32_t elems = 256, bytes = 176; };
+template <>
+struct BlockInfo<FMT_Q4_0> { static constexpr uint32_t elems = 32, bytes = 18; };
 
 __device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
 
@@ -151,6 +153,16 @@ __device__ __forceinline__ void dequant8(const uint8_t* b, uint32_t e0, float (&
         }
     } else if (FMT == FMT_Q6_K) {
         dequant8_q6k(b, b + 128, b + 192, b + 208, e0, y);
+    } else if (FMT == FMT_Q4_0) {
+        // {fp16 d; u8 qs[16]}: element j in the low, j + 16 in the high nibble of qs[j]; w = d * (q - 8)
+        // (include/ie/quant_blocks.hpp:32-43, src/ops/gemv_q4_0.cpp:3-8)
+        const float d = h2f(ld16(b));
+        const uint32_t hi = e0 >> 4, j0 = e0 & 15u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t byte = b[2 + j0 + i];
+            y[i] = d * (float)((int)(hi ? byte >> 4 : byte & 15u) - 8);
+        }
     } else {
         const float d = e8m0_half(b[0]);
         const uint32_t hi = e0 >> 4, j0 = e0 & 15u;
@@ -275,6 +287,18 @@ struct Mxfp4SoaView {   // qs_plane[n*(K/2) + 16b + j], e_plane[n*(K/32) + b]   
     }
 };
 
+struct Q40SoaView {     // q4_qs[n*(K/2) + 16b + j], q4_d[n*(K/32) + b]   (src/ops/gemv_q4_0.cpp:179-192,455-477)
+    const uint8_t* qs; const uint16_t* d; uint32_t K;
+    __device__ __forceinline__ void get(uint32_t n, uint32_t kg, float (&y)[8]) const {
+        const uint32_t b = kg >> 2, e0 = (kg & 3u) * 8u;
+        const float dv = h2f(d[(size_t)n * (K >> 5) + b]);
+        const uint8_t* p = qs + (size_t)n * (K >> 1) + 16u * b + (e0 & 15u);
+        const uint32_t hi = e0 >> 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = dv * (float)((int)(hi ? p[i] >> 4 : p[i] & 15u) - 8);
+    }
+};
+
 template <class V>
 __global__ __launch_bounds__(256) void dequant_bt_view_kernel(V v, half_t* Bt, uint32_t N) {
     const uint32_t n = blockIdx.x * blockDim.x + threadIdx.x;
@@ -330,6 +354,7 @@ MX_DEQ(q4_K, FMT_Q4_K)
 MX_DEQ(q5_K, FMT_Q5_K)
 MX_DEQ(q6_K, FMT_Q6_K)
 MX_DEQ(mxfp4, FMT_MXFP4)
+MX_DEQ(q4_0, FMT_Q4_0)
 #undef MX_DEQ
 
 // Transposed dequant of the repacked layouts.
@@ -354,6 +379,10 @@ int mx_dequant_q6_soa_to_Bt(mx_stream_t s, const uint8_t* q6_lo, const uint8_t* 
     MX_REQUIRE_PTR(q6_lo); MX_REQUIRE_PTR(q6_hi); MX_REQUIRE_PTR(q6_sc); MX_REQUIRE_PTR(q6_d);
     MX_REQUIRE_ALIGN(q6_lo, 4); MX_REQUIRE_ALIGN(q6_hi, 2);
     return dequant_bt_view(s, Q6KNatView{q6_lo, q6_hi, q6_sc, q6_d, K}, Bt, K, N, 256);
+}
+int mx_dequant_q4_0_soa_to_Bt(mx_stream_t s, const uint8_t* soa_qs, const uint16_t* soa_d, uint16_t* Bt, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(soa_qs); MX_REQUIRE_PTR(soa_d);
+    return dequant_bt_view(s, Q40SoaView{soa_qs, soa_d, K}, Bt, K, N, 32);
 }
 int mx_dequant_mxfp4_soa_to_Bt(mx_stream_t s, const uint8_t* qs_plane, const uint8_t* e_plane, uint16_t* Bt, uint32_t K, uint32_t N) {
     MX_REQUIRE_PTR(qs_plane); MX_REQUIRE_PTR(e_plane);

@@ -12,7 +12,7 @@ import torch
 from . import lib
 
 Q81X_BYTES, Q81S_BYTES = 40, 48
-BLOCK = {"q8_0": (32, 34), "q4_K": (256, 144), "q6_K": (256, 210), "mxfp4": (32, 17)}
+BLOCK = {"q8_0": (32, 34), "q4_K": (256, 144), "q6_K": (256, 210), "mxfp4": (32, 17), "q5_K": (256, 176), "q4_0": (32, 18)}
 
 
 class MxError(RuntimeError):
@@ -361,6 +361,56 @@ def gemv_q4_K_dual(A, W_a, W_b, K, N):
 def gemv_q4_K_down_accum(A, W, sh_g, y, K, N):
     _call("mx_gemv_q4_K_down_accum", _f16(A), _u8(W), _f16(sh_g), _f16(y), K, N)
     return y
+
+
+def gemv_q4_0(A, W, K, N, y=None):
+    y = _out(y, (N,), torch.float16, A)
+    _call("mx_gemv_q4_0", _f16(A), _u8(W), _ptr(y), K, N)
+    return y
+
+
+def gemv_q4_0_q8(x_q8, W, K, N, T=1, y=None):
+    return _gemv_q8("mx_gemv_q4_0_q8_batched", x_q8, (_u8(W),), K, N, T, y)
+
+
+def gemv_q4_0_soa_q8(x_q8, q4_qs, q4_d, K, N, T=1, y=None):
+    return _gemv_q8("mx_gemv_q4_0_soa_q8" + ("_batched" if T > 1 else ""), x_q8, (_u8(q4_qs), _ptr(q4_d)), K, N, T, y)
+
+
+def gemv_q4_0_soa_q8_multi(x_q8, banks, K):
+    """banks = [(q4_qs, q4_d, N), ...] (1 to 3) sharing x_q8 -> list of fp16 [N] outputs, one launch."""
+    import ctypes as C
+    n = len(banks)
+    ys = [torch.empty(b[2], dtype=torch.float16, device=x_q8.device) for b in banks]
+    qs = (C.c_void_p * n)(*[_u8(b[0]) for b in banks])
+    d = (C.c_void_p * n)(*[_ptr(b[1]) for b in banks])
+    yp = (C.c_void_p * n)(*[_ptr(t) for t in ys])
+    Ns = (C.c_uint32 * n)(*[b[2] for b in banks])
+    _call("mx_gemv_q4_0_soa_q8_multi", _u8(x_q8), C.cast(qs, C.c_void_p), C.cast(d, C.c_void_p), C.cast(yp, C.c_void_p), C.cast(Ns, C.c_void_p), n, K)
+    return ys
+
+
+def gemv_q5_K(A, W, K, N, y=None):
+    y = _out(y, (N,), torch.float16, A)
+    _call("mx_gemv_q5_K", _f16(A), _u8(W), _ptr(y), K, N)
+    return y
+
+
+def gemv_q5_K_q8(x_q8, W, K, N, T=1, y=None):
+    return _gemv_q8("mx_gemv_q5_K_q8" + ("_batched" if T > 1 else ""), x_q8, (_u8(W),), K, N, T, y)
+
+
+def gemm_q4_0(A, W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_q4_0", _f16(A), _u8(W), _ptr(y), M, K, N)
+    return y
+
+
+def repack_q4_0_to_soa(W, K, N):
+    W = _np_u8(W)
+    qs, d = np.empty(N * K // 2, np.uint8), np.empty(N * K // 32, np.uint16)
+    _host("mx_repack_q4_0_to_soa", W.ctypes.data, K, N, qs.ctypes.data, d.ctypes.data)
+    return qs, d
 
 
 def gemv_q4_K_reorder_q8(x_q8, W_reorder, K, N, y=None):

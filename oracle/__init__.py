@@ -13,10 +13,10 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-Q8_0, Q4_K, Q6_K, MXFP4, Q5_K = 0, 1, 2, 3, 4   # Q5_K: dequant only
-FMT_NAMES = {Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", MXFP4: "mxfp4", Q5_K: "q5_K"}
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, Q5_K: 256}
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210, MXFP4: 17, Q5_K: 176}
+Q8_0, Q4_K, Q6_K, MXFP4, Q5_K, Q4_0 = 0, 1, 2, 3, 4, 5   # Q5_K: no encoder (see synth_q5_K)
+FMT_NAMES = {Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K", MXFP4: "mxfp4", Q5_K: "q5_K", Q4_0: "q4_0"}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, Q5_K: 256, Q4_0: 32}
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210, MXFP4: 17, Q5_K: 176, Q4_0: 18}
 Q8_1X_BYTES, Q8_1S_BYTES = 40, 48
 
 
@@ -152,6 +152,16 @@ def quantize(fmt, x):
     out = np.zeros((rows, row_bytes(fmt, K)), np.uint8)
     _quant_rows(fmt, _p(x), _p(out), rows, K)
     return out
+
+
+def synth_q5_K(x, seed):
+    """Valid Q5_K blocks for tests: the Q4_K encoding of x (header, scales, nibbles) plus seeded fifth bits.
+    {d, dmin, scales[12], qh[32], qs[128]} (include/ie/quant_blocks.hpp:79-85).  -> uint8 [rows, K/256*176]."""
+    b4 = quantize(Q4_K, x)
+    rows = b4.shape[0]
+    b4 = b4.reshape(-1, 144)
+    qh = rand_bytes(seed, b4.shape[0] * 32).reshape(-1, 32)
+    return np.concatenate([b4[:, :16], qh, b4[:, 16:]], axis=1).reshape(rows, -1)
 
 
 def quantize_q8_1(x):

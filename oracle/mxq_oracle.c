@@ -17,6 +17,12 @@
  *                                            e in {0,1} denormals, 2^(e-128)), the
  *                                            reference test's exponent list; no host
  *                                            header in the reference compiles it
+ *   orc_dequant (Q4_0)                       pinned: closed forms (d = 1 -> y = nibble - 8, element j in the low
+ *                                            and j+16 in the high nibble of qs[j]); the reference holds no host
+ *                                            routine for it (device code src/ops/gemv_q4_0.cpp:3-8,455-477)
+ *   orc_quantize_row_q4_0                    NOT IN REFERENCE (fixture generator only; ggml's published
+ *                                            quantize_row_q4_0_ref recipe); pinned by round trip: error <= |d|/2
+ *                                            except the clamped extreme
  *   orc_quantize_row_q4_K / _q6_K            pinned: oracle/_ref (bit-identical blocks),
  *                                            golden fixtures, reference error bounds
  *   orc_quantize_row_q8_0                    pinned: invariants + round trip
@@ -42,7 +48,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_Q8_0 = 0, ORC_Q4_K = 1, ORC_Q6_K = 2, ORC_MXFP4 = 3, ORC_Q5_K = 4 /* dequant only */ };
+enum { ORC_Q8_0 = 0, ORC_Q4_K = 1, ORC_Q6_K = 2, ORC_MXFP4 = 3, ORC_Q5_K = 4 /* no encoder */, ORC_Q4_0 = 5 };
 
 /* ---------------------------------------------------------------- layouts
  * include/ie/quant_blocks.hpp:26-30 (Q8_0), :55-60 (MXFP4), :67-73 (Q4_K),
@@ -53,6 +59,7 @@ enum { ORC_Q8_0 = 0, ORC_Q4_K = 1, ORC_Q6_K = 2, ORC_MXFP4 = 3, ORC_Q5_K = 4 /* 
 #define Q6_K_BYTES 210
 #define Q5_K_BYTES 176
 #define MXFP4_BYTES 17
+#define Q4_0_BYTES 18
 #define Q8_1X_BYTES 40
 #define Q8_1S_BYTES 48
 
@@ -221,7 +228,17 @@ static void deq_mxfp4(const uint8_t* b, float* y) {
     }
 }
 
-ORC_API int orc_block_elems(int fmt) { return (fmt == ORC_Q8_0 || fmt == ORC_MXFP4) ? 32 : 256; }
+/* Q4_0: {fp16 d; u8 qs[16]}, w[j] = d * ((qs[j] & 15) - 8), w[j+16] = d * ((qs[j] >> 4) - 8)
+ * (include/ie/quant_blocks.hpp:32-43, src/ops/gemv_q4_0.cpp:3-8) */
+static void deq_q4_0(const uint8_t* b, float* y) {
+    const float d = orc_fp16_to_fp32(rd16(b));
+    for (int j = 0; j < 16; ++j) {
+        y[j] = d * (float)((int)(b[2 + j] & 15) - 8);
+        y[j + 16] = d * (float)((int)(b[2 + j] >> 4) - 8);
+    }
+}
+
+ORC_API int orc_block_elems(int fmt) { return (fmt == ORC_Q8_0 || fmt == ORC_MXFP4 || fmt == ORC_Q4_0) ? 32 : 256; }
 ORC_API int orc_block_bytes(int fmt) {
     switch (fmt) {
         case ORC_Q8_0: return Q8_0_BYTES;
@@ -229,6 +246,7 @@ ORC_API int orc_block_bytes(int fmt) {
         case ORC_Q6_K: return Q6_K_BYTES;
         case ORC_MXFP4: return MXFP4_BYTES;
         case ORC_Q5_K: return Q5_K_BYTES;
+        case ORC_Q4_0: return Q4_0_BYTES;
     }
     return 0;
 }
@@ -239,6 +257,7 @@ static void deq_block(int fmt, const uint8_t* b, float* y) {
         case ORC_Q6_K: deq_q6_K(b, y); break;
         case ORC_MXFP4: deq_mxfp4(b, y); break;
         case ORC_Q5_K: deq_q5_K(b, y); break;
+        case ORC_Q4_0: deq_q4_0(b, y); break;
     }
 }
 
@@ -510,6 +529,24 @@ ORC_API void orc_quantize_row_mxfp4(const float* x, void* out, int64_t k) {
     }
 }
 
+/* Q4_0 encoder.  NOT in the reference (Gemma-4 QAT GGUFs ship Q4_0).  Fixture generator only, after ggml's
+ * published quantize_row_q4_0_ref: d = (value of largest magnitude) / -8, q = min(15, trunc(x/d + 8.5)). */
+ORC_API void orc_quantize_row_q4_0(const float* x, void* out, int64_t k) {
+    uint8_t* y = (uint8_t*)out;
+    for (int64_t i = 0; i < k / 32; ++i, x += 32, y += Q4_0_BYTES) {
+        float amax = 0, mx = 0;
+        for (int j = 0; j < 32; ++j)
+            if (amax < fabsf(x[j])) { amax = fabsf(x[j]); mx = x[j]; }
+        const float d = mx / -8.f, id = d != 0.f ? 1.f / d : 0.f;
+        const uint16_t hd = orc_fp32_to_fp16(d);
+        y[0] = (uint8_t)hd; y[1] = (uint8_t)(hd >> 8);
+        for (int j = 0; j < 16; ++j) {
+            const int q0 = clampi((int)(x[j] * id + 8.5f), 0, 15), q1 = clampi((int)(x[j + 16] * id + 8.5f), 0, 15);
+            y[2 + j] = (uint8_t)(q0 | (q1 << 4));
+        }
+    }
+}
+
 ORC_API void orc_quantize_rows(int fmt, const float* x, void* out, int64_t n_rows, int64_t k) {
     const int64_t rb = k / orc_block_elems(fmt) * orc_block_bytes(fmt);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -521,6 +558,7 @@ ORC_API void orc_quantize_rows(int fmt, const float* x, void* out, int64_t n_row
             case ORC_Q4_K: orc_quantize_row_q4_K(xr, o, k); break;
             case ORC_Q6_K: orc_quantize_row_q6_K(xr, o, k); break;
             case ORC_MXFP4: orc_quantize_row_mxfp4(xr, o, k); break;
+            case ORC_Q4_0: orc_quantize_row_q4_0(xr, o, k); break;
         }
     }
 }
@@ -635,7 +673,7 @@ ORC_API void orc_gemv_q8chain(int fmt, const void* W, const void* xq8, double* y
 /* Exact integer dot of one weight row against one q8 row, per 32-element
  * block, for brute-force checks of the int-dot kernels' integer part.
  * qw = the format's integer code (Q8_0: qs; Q4_K: nibble 0..15; Q6_K: q-32;
- * MXFP4: doubled E2M1 value). */
+ * MXFP4: doubled E2M1 value; Q4_0: nibble - 8; Q5_K: 5-bit code 0..31). */
 ORC_API void orc_int_codes(int fmt, const void* row, uint32_t K, int8_t* codes) {
     const int be = orc_block_elems(fmt), bb = orc_block_bytes(fmt);
     for (uint32_t b = 0; b < K / be; ++b) {
@@ -644,6 +682,13 @@ ORC_API void orc_int_codes(int fmt, const void* row, uint32_t K, int8_t* codes) 
         if (fmt == ORC_Q8_0) memcpy(c, p + 2, 32);
         else if (fmt == ORC_MXFP4)
             for (int j = 0; j < 16; ++j) { c[j] = kMxfp4Lut[p[1 + j] & 15]; c[j + 16] = kMxfp4Lut[p[1 + j] >> 4]; }
+        else if (fmt == ORC_Q4_0)
+            for (int j = 0; j < 16; ++j) { c[j] = (int8_t)((p[2 + j] & 15) - 8); c[j + 16] = (int8_t)((p[2 + j] >> 4) - 8); }
+        else if (fmt == ORC_Q5_K)
+            for (int e = 0; e < 256; ++e) {
+                const uint8_t by = p[48 + 32 * (e >> 6) + (e & 31)];
+                c[e] = (int8_t)((((e >> 5) & 1) ? by >> 4 : by & 15) | (((p[16 + (e & 31)] >> (e >> 5)) & 1) << 4));
+            }
         else if (fmt == ORC_Q4_K)
             for (int e = 0; e < 256; ++e) { const uint8_t by = p[16 + 32 * (e >> 6) + (e & 31)]; c[e] = (int8_t)(((e >> 5) & 1) ? by >> 4 : by & 15); }
         else

@@ -8,14 +8,14 @@ import oracle as O
 from gpu_util import dev, host
 
 pytestmark = pytest.mark.gpu
-FMTS = (O.Q8_0, O.Q4_K, O.Q6_K, O.MXFP4)
+FMTS = (O.Q8_0, O.Q4_K, O.Q6_K, O.MXFP4, O.Q4_0)
 
 
 def random_blocks(fmt, seed, nb):
     """1024 seeded random blocks per format as the reference's dequant test does
     (tests/unit/dequant_test.cpp:112-150); scale fields kept finite."""
     raw = O.rand_bytes(seed, nb * O.BLOCK_BYTES[fmt]).reshape(nb, -1).copy()
-    for off in {O.Q8_0: [1], O.Q4_K: [1, 3], O.Q6_K: [209], O.MXFP4: []}[fmt]:
+    for off in {O.Q8_0: [1], O.Q4_K: [1, 3], O.Q6_K: [209], O.MXFP4: [], O.Q4_0: [1]}[fmt]:
         raw[:, off] &= 0xBB
     if fmt == O.MXFP4:  # the reference test's exponent list, then random ones below overflow
         lst = [0, 1, 2, 3, 64, 126, 127, 128, 200, 254, 255]

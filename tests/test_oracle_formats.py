@@ -140,6 +140,39 @@ def test_mxfp4_closed_forms():
     assert O.e8m0_half(0) == 2.0 ** -128 and O.e8m0_half(1) == 2.0 ** -127 and O.e8m0_half(127) == 0.5
 
 
+def test_q4_0_closed_forms_and_round_trip():
+    """Q4_0 has no host routine in the reference; pinned by its definition (include/ie/quant_blocks.hpp:32-43,
+    src/ops/gemv_q4_0.cpp:3-8): w[j] = d * ((qs[j] & 15) - 8), w[j+16] = d * ((qs[j] >> 4) - 8)."""
+    b = np.zeros(18, np.uint8)
+    b[0:2] = np.array([0x4000], np.uint16).view(np.uint8)       # d = 2.0
+    b[2:] = (np.arange(16) | ((15 - np.arange(16)) << 4)).astype(np.uint8)
+    y = O.dequant(O.Q4_0, b)
+    assert np.array_equal(y[:16], 2.0 * (np.arange(16) - 8)) and np.array_equal(y[16:], 2.0 * (7 - np.arange(16)))
+    # encoder (fixture generator): error at most |d|/2 except where x/d + 8 clamps at 15, and the extreme maps to code 0
+    x = O.normal(77, (64, 256), 0.0, 0.02)
+    w = O.quantize(O.Q4_0, x)
+    yq = O.dequant(O.Q4_0, w).reshape(x.shape)
+    d = np.abs(O.fp16_to_fp32(w.reshape(-1, 18)[:, :2].copy().view(np.uint16).ravel())).reshape(64, 8)
+    err = np.abs(yq - x).reshape(64, 8, 32)
+    inside = np.abs(x).reshape(64, 8, 32) <= 7.0 * d[:, :, None]          # codes 1..15 reach +-7 d; beyond that the code clamps
+    tol = 2.0 ** -7                                                        # d is stored as fp16, the codes were chosen with the fp32 d
+    assert (err <= d[:, :, None] * (1.0 + tol)).all() and (err[inside] <= (d[:, :, None] * (0.5 + tol) * np.ones_like(err))[inside]).all()
+    codes = O.int_codes(O.Q4_0, w[0], 256)
+    assert codes.min() >= -8 and codes.max() <= 7
+    assert np.array_equal(codes.astype(np.float32) * np.repeat(O.fp16_to_fp32(w[0].reshape(-1, 18)[:, :2].copy().view(np.uint16).ravel()), 32), yq[0])
+    # Q5_K codes: 5-bit code c with (d*sc)*c - dmin*m == dequant (include/ie/dequant_ref.hpp:55-75)
+    w5 = O.synth_q5_K(O.normal(78, (1, 512), 0.0, 0.02), 79)
+    c5 = O.int_codes(O.Q5_K, w5[0], 512).astype(np.int64)
+    assert c5.min() >= 0 and c5.max() <= 31 and c5.max() > 15
+    blk = w5[0].reshape(-1, 176)
+    for b in range(2):
+        d, dmin = O.fp16_to_fp32(blk[b, 0:4].copy().view(np.uint16))
+        for j in range(8):
+            sc, mn = O.get_scale_min_k4(j, blk[b, 4:16])
+            exp = (np.float32(d) * np.float32(sc)) * c5[256 * b + 32 * j:256 * b + 32 * j + 32].astype(np.float32) - np.float32(dmin) * np.float32(mn)
+            assert np.array_equal(exp.astype(np.float32), O.dequant(O.Q5_K, w5[0])[256 * b + 32 * j:256 * b + 32 * j + 32])
+
+
 # ---------------------------------------------------------------- encoders
 @pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K))
 def test_encoders_bit_identical_to_reference_golden(golden, fmt):
