@@ -4,6 +4,9 @@
 every call goes through the C ABI of libmxq.so (include/mxq.h).  PyTorch is
 used only for device memory and the current HIP stream.
 """
+import torch  # noqa: F401  -- before libmxq.so: the library must bind to the HIP runtime torch has loaded,
+#                      or the process ends up with two runtimes and the second one sees no device
+
 from . import _lib
 
 lib = _lib.load()
