@@ -41,6 +41,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
+    ap.add_argument("--unfused", action="store_true", help="gate and up as two launches instead of the fused gate+up launch")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-detail", action="store_true", help="skip the per-config detail table")
     ap.add_argument("--sets", type=int, default=4, help="distinct weight sets rotated through (331.7 MB each)")
@@ -92,13 +93,25 @@ def main():
             qs, d = ws[("q8_0_soa", name)]
             ops.gemv_q8_0_soa_q8(xq_, qs, d, K, N, y)
 
+    def gate_up(fmt, ws):
+        # gate and up share the activation row: one fused launch (as the reference fuses them for MXFP4 and Q4_K)
+        if fmt == "q6_K":
+            ops.gemv_q8_x2("q6_K", xq, ws[(fmt, "gate")], ws[(fmt, "up")], H, FF, y_ff[(fmt, "gate")], y_ff[(fmt, "up")])
+        else:
+            ops.gemv_q8_x2("q8_0_soa", xq, ws[("q8_0_soa", "gate")], ws[("q8_0_soa", "up")], H, FF, y_ff[(fmt, "gate")], y_ff[(fmt, "up")])
+
     def step(ws):
         for fmt in fmts:
-            gemv(fmt, xq, ws, "gate", H, FF, y_ff[(fmt, "gate")])
-            gemv(fmt, xq, ws, "up", H, FF, y_ff[(fmt, "up")])
+            if args.unfused:
+                gemv(fmt, xq, ws, "gate", H, FF, y_ff[(fmt, "gate")])
+                gemv(fmt, xq, ws, "up", H, FF, y_ff[(fmt, "up")])
+            else:
+                gate_up(fmt, ws)
             gemv(fmt, hq, ws, "down", FF, H, y_h[fmt])
 
     bytes_per_step = sum(gemv_bytes(synth.row_bytes(f, K), K, N, 1) for f in fmts for (K, N) in shapes.values())
+    if not args.unfused:
+        bytes_per_step -= len(fmts) * (H // 32) * 40   # the fused launch reads the activation row once
 
     if args.probe:
         # plain copy of known size first (the scale for FETCH_SIZE / WRITE_SIZE), then the kernels under study
@@ -164,22 +177,29 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / (5 * n_launch) * 1e3
 
-    mats = [ws[("q8_0_soa", n)] for ws in sets for n in ("gate", "up")]
-    dom_us = kernel_avg_us(lambda i: ops.gemv_q8_0_soa_q8(xq, mats[i % len(mats)][0], mats[i % len(mats)][1], H, FF, y_ff[("q8_0", "gate")]),
-                           4 * len(mats))
-    dom_bytes = gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1)
+    if args.unfused:
+        mats = [ws[("q8_0_soa", n)] for ws in sets for n in ("gate", "up")]
+        dom_us = kernel_avg_us(lambda i: ops.gemv_q8_0_soa_q8(xq, mats[i % len(mats)][0], mats[i % len(mats)][1], H, FF, y_ff[("q8_0", "gate")]),
+                               4 * len(mats))
+        dom_bytes = gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1)
+        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> K=4096 N=14336", 62483456 + 114790
+    else:
+        # the fused gate + up launch: two 4096 -> 14336 matrices, one activation row, two output rows
+        dom_us = kernel_avg_us(lambda i: gate_up("q8_0", sets[i % len(sets)]), 4 * len(sets))
+        dom_bytes = 2 * gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1) - (H // 32) * 40
+        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 124876800 + 233267
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "gemv_q8_kernel<FmtQ8Soa,T=1> K=4096 N=14336", "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt)
-                "traffic": 62483456 + 114790,
+                "traffic": dom_traffic,
                 "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 3)}
 
     out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8 dot, fp32 fold", "data": "synthetic",
            "config": {"workload": "configs[1]: decode GEMV gate/up 4096->14336 + down 14336->4096, Q6_K and Q8_0, T=1, "
-                                  "6 launches/step, %d rotating weight sets" % len(sets),
+                                  "%s, %d rotating weight sets" % ("6 launches/step" if args.unfused else "gate+up fused: 4 launches/step", len(sets)),
                       "bytes_per_step": bytes_per_step, "hip_graph": bool(graphs), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
            "roofline": roofline}
 

@@ -150,6 +150,18 @@ int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint
 int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W,
                                 uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* Fused gate + up for the other int-dot formats: y_a = W_a . x, y_b = W_b . x in one launch, both matrices [N, K].
+ * No counterpart of these names in the reference, which fuses gate/up this way for MXFP4 (gemv_mxfp4_soa_q8_x2,
+ * include/ie/ops.hpp:503-513) and for Q4_K with fp16 activations (gemv_q4_K_dual_ffn, src/ops/gemv_q4k.cpp:603-612).
+ * Each output is bit-identical to the single-matrix entry point's.  */
+int mx_gemv_q8_0_soa_q8_x2(mx_stream_t s, const void* x_q8, const int8_t* a_qs, const uint16_t* a_d, const int8_t* b_qs,
+                           const uint16_t* b_d, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N);
+int mx_gemv_q4_K_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b,
+                       uint32_t K, uint32_t N);
+int mx_gemv_q6_K_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b,
+                       uint32_t K, uint32_t N);
+int mx_gemv_q8_0_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b,
+                       uint32_t K, uint32_t N);
 /* Sibling formats on the same kernels.
  * Q4_0:
  *   gemv_q4_0                 include/ie/ops.hpp:525-529, src/ops/gemv_q4_0.cpp:54-120   fp16 activations, GGUF blocks

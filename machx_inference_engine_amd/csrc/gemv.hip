@@ -373,6 +373,13 @@ static int gemv_aos_fact(int fmt, mx_stream_t s, const ActT* A, const void* W, O
     return launch_fact<FmtQ8Aos>(s, FmtQ8Aos::W{base, K / 32 * (uint32_t)kQ8_0Bytes}, A, y, K, N);
 }
 
+// Fused gate + up for the other int-dot formats: two matrices of the same shape against one q8 row, one
+// launch (the shape of gemv_mxfp4_soa_q8_x2 above and of gemv_q4_K_dual_ffn; blockIdx.y picks the matrix).
+template <class F>
+static int gemv_x2(mx_stream_t s, const void* x, const typename F::W& wa, const typename F::W& wb, uint16_t* ya, uint16_t* yb, uint32_t K, uint32_t N) {
+    GemvSeg<F, half_t> a{wa, reinterpret_cast<half_t*>(ya), nullptr}, b{wb, reinterpret_cast<half_t*>(yb), nullptr};
+    return launch_q8<F, half_t>(s, a, b, 2, x, K, N, 1);
+}
 }  // namespace mxq
 
 using namespace mxq;
@@ -568,6 +575,32 @@ int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x, const uint8_t* gate_qs
     GemvSeg<FmtMxfp4Soa, half_t> g{{gate_qs, gate_e, K}, reinterpret_cast<half_t*>(gate_y), gate_bias};
     GemvSeg<FmtMxfp4Soa, half_t> u{{up_qs, up_e, K}, reinterpret_cast<half_t*>(up_y), up_bias};
     return launch_q8<FmtMxfp4Soa, half_t>(s, g, u, 2, x, K, N, 1);
+}
+
+int mx_gemv_q8_0_soa_q8_x2(mx_stream_t s, const void* x_q8, const int8_t* a_qs, const uint16_t* a_d, const int8_t* b_qs, const uint16_t* b_d,
+                           uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
+    if (int rc = check_common(x_q8, y_a, K, N, 1, 32)) return rc;
+    MX_REQUIRE_PTR(y_b); MX_REQUIRE_PTR(a_qs); MX_REQUIRE_PTR(a_d); MX_REQUIRE_PTR(b_qs); MX_REQUIRE_PTR(b_d);
+    MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(a_qs, 16); MX_REQUIRE_ALIGN(b_qs, 16); MX_REQUIRE_ALIGN(a_d, 2); MX_REQUIRE_ALIGN(b_d, 2);
+    return gemv_x2<FmtQ8Soa>(s, x_q8, {a_qs, a_d, K}, {b_qs, b_d, K}, y_a, y_b, K, N);
+}
+static int gemv_aos_x2(int fmt, mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
+    if (int rc = check_common(x_q8, y_a, K, N, 1, fmt == 0 ? 32 : 256)) return rc;
+    MX_REQUIRE_PTR(y_b); MX_REQUIRE_PTR(W_a); MX_REQUIRE_PTR(W_b);
+    MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(W_a, fmt == 1 ? 16 : 2); MX_REQUIRE_ALIGN(W_b, fmt == 1 ? 16 : 2);
+    const uint8_t *a = static_cast<const uint8_t*>(W_a), *b = static_cast<const uint8_t*>(W_b);
+    if (fmt == 1) return gemv_x2<FmtQ4K>(s, x_q8, {a, K / 256 * (uint32_t)kQ4KBytes}, {b, K / 256 * (uint32_t)kQ4KBytes}, y_a, y_b, K, N);
+    if (fmt == 2) return gemv_x2<FmtQ6K>(s, x_q8, {a, K / 256 * (uint32_t)kQ6KBytes}, {b, K / 256 * (uint32_t)kQ6KBytes}, y_a, y_b, K, N);
+    return gemv_x2<FmtQ8Aos>(s, x_q8, {a, K / 32 * (uint32_t)kQ8_0Bytes}, {b, K / 32 * (uint32_t)kQ8_0Bytes}, y_a, y_b, K, N);
+}
+int mx_gemv_q4_K_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
+    return gemv_aos_x2(1, s, x_q8, W_a, W_b, y_a, y_b, K, N);
+}
+int mx_gemv_q6_K_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
+    return gemv_aos_x2(2, s, x_q8, W_a, W_b, y_a, y_b, K, N);
+}
+int mx_gemv_q8_0_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
+    return gemv_aos_x2(0, s, x_q8, W_a, W_b, y_a, y_b, K, N);
 }
 
 int mx_gemv_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t K, uint32_t N) {

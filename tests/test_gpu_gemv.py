@@ -245,3 +245,20 @@ def test_gemv_q4_K_dual_ssm_gbeta(mx, K, N):
     assert np.max(np.abs(host(beta) - ref_b)) <= 1e-5
     # and the sums themselves against the float-chain oracle
     check(host(ya).astype(np.float32), O.gemv_f64(O.Q4_K, Wa, x16, K, N)[0], "alpha sums")
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+def test_gemv_q8_x2_equals_two_single_launches(mx, fmt):
+    """Fused gate + up (the launch shape of gemv_mxfp4_soa_q8_x2, include/ie/ops.hpp:503-513): each output is
+    bit-identical to the single-matrix kernel's, which is gated against the oracle above."""
+    K, N = 2048, 300
+    name = O.FMT_NAMES[fmt]
+    Wa, Wb = weights(fmt, 1400 + fmt, N, K), weights(fmt, 1410 + fmt, N, K)
+    xq = dev(O.quantize_q8_1(acts(1420, 1, K)))
+    single = getattr(mx.ops, "gemv_%s_q8" % name)
+    ya, yb = mx.ops.gemv_q8_x2(name, xq, dev(Wa), dev(Wb), K, N)
+    assert torch.equal(ya, single(xq, dev(Wa), K, N)) and torch.equal(yb, single(xq, dev(Wb), K, N))
+    if fmt == O.Q8_0:
+        sa, sb = [tuple(dev(p) for p in O.repack_q8_0_to_soa(W)) for W in (Wa, Wb)]
+        ya2, yb2 = mx.ops.gemv_q8_x2("q8_0_soa", xq, sa, sb, K, N)
+        assert torch.equal(ya2, mx.ops.gemv_q8_0_soa_q8(xq, sa[0], sa[1], K, N)) and torch.equal(yb2, mx.ops.gemv_q8_0_soa_q8(xq, sb[0], sb[1], K, N))
