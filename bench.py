@@ -238,6 +238,14 @@ def main():
         us = kernel_avg_us(lambda i: ops.gemv_q4_K_q8(aq, w1[i % len(w1)], 4096, 4096, y16), 2 * len(w1))
         detail["config1_q4_K_4096x4096_q8"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
         del w1
+        # lm_head-sized decode GEMV (the largest single GEMV of a decode step): Q6_K, 4096 -> 151936, 510 MB
+        NV = 151936
+        wl = [synth.random_weights("q6_K", NV, H, seed=700 + i, device=dev) for i in range(2)]
+        yv = torch.empty(NV, dtype=torch.float16, device=dev)
+        us = kernel_avg_us(lambda i: ops.gemv_q6_K_q8(xq, wl[i % 2], H, NV, yv), 4)
+        b = gemv_bytes(synth.row_bytes("q6_K", H), H, NV, 1)
+        detail["lm_head_q6_K_K4096_N151936_T1"] = {"us": round(us, 1), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del wl, yv
         # BASELINE config 3: prefill quant-GEMM, Q4_K, fp16 MFMA (peak 2.5 PFLOP/s dense fp16)
         MFMA_PEAK = 2500.0
         for (K, N) in ((H, FF), (FF, H)):

@@ -195,6 +195,9 @@ int parse_shard(Gguf* g, const Mapping& m, bool primary, const std::string& path
         type_size(t.ggml_type, &bytes, &elems);
         if (bytes) {
             if (t.shape[0] % elems) return fail(MX_ERR_FORMAT, path + ": tensor row length is not a whole number of blocks");
+            // no format here packs more than 8 elements into a byte: anything larger cannot lie in this file
+            // (and would overflow the size computation)
+            if (n_elem / 8 > m.size) return fail(MX_ERR_FORMAT, path + ": tensor " + std::to_string(i) + " is larger than the file");
             t.nbytes = n_elem / elems * bytes;
         }
         g->tensors.push_back(t);

@@ -94,4 +94,10 @@ def test_errors(tmp_path):
         with pytest.raises(gguf.GgufError) as e:
             gguf.GgufFile(p)
         assert e.value.status == 7, what
+    # a directory entry whose element count would overflow the size computation
+    p = tmp_path / "huge.gguf"
+    G.write_gguf(p, [], [("t", 0, (2 ** 62, 8), np.zeros(4, np.float32))])
+    with pytest.raises(gguf.GgufError) as e:
+        gguf.GgufFile(p)
+    assert e.value.status == 7
     assert lib.mx_gguf_open(None, None) == 1
