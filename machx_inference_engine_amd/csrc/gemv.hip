@@ -2,6 +2,8 @@
 // Q4_K / Q6_K / Q8_0 / MXFP4 weights: int-dot on q8 activations and the
 // float-activation variants.  Kernel structure: mxq_gemv_core.h.
 #include "mxq_gemv_core.h"
+#include <stdlib.h>
+
 #include "mxq_host.h"
 
 namespace mxq {
@@ -65,6 +67,56 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
                     store_out(seg.y + (size_t)t * N + row0 + r, v);
                 }
             }
+    }
+}
+
+// Rows much longer than a wave can cover in one step (K >= 8192) with few of them (N = 4096: the down
+// projections): the whole workgroup walks R rows at a time, thread t of 256 taking units t, t + 256, ...,
+// and the four wave sums meet in LDS.  One memory round trip per row instead of K / 64 / G of them, and
+// G / 256 times fewer rows per workgroup, so that a short matrix still fills every CU.  Single K tile only.
+template <class F, int T, int R, class OutT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, OutT> seg0, GemvSeg<F, OutT> seg1, const uint8_t* xq8, uint32_t K,
+                                                                     uint32_t N, uint32_t KT, uint32_t T_real, uint32_t q8_split) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ float red[2][kGemvWaves][R][T];
+    const GemvSeg<F, OutT>& seg = blockIdx.y ? seg1 : seg0;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const size_t q8_row_bytes = (size_t)(K / 32) * (q8_split ? kQ81sBytes : kQ81xBytes);
+    auto xrow = [&](uint32_t t) { return xq8 + (size_t)(t < T_real ? t : T_real - 1) * q8_row_bytes; };
+    const ActTile act = stage_act<F::SUM_GRAN, T>(lds, xrow, 0, K, KT, q8_split != 0);
+    __syncthreads();
+    const uint32_t n_units = (K + 63) / 64, n_rg = (N + R - 1) / R;
+    const bool half_tail = (K & 63u) != 0;
+    uint32_t par = 0;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x, par ^= 1u) {
+        const uint32_t row0 = rg * R;
+        float acc[R][T];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < T; ++t) acc[r][t] = 0.f;
+        typename F::Cursor cu[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) cu[r] = F::cursor(seg.w, (row0 + r < N) ? row0 + r : N - 1, tid);
+        gemv_rows<F, T, R, kGemvThreads, 1>(cu, n_units, half_tail, tid, act, acc);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const float v = group_sum<64>(acc[r][t]);
+                if (lane == (uint32_t)group_sum_lane<64>(lane)) red[par][wave][r][t] = v;
+            }
+        __syncthreads();   // one barrier per row group: the sums alternate between two buffers
+        if (tid < R * T) {
+            const uint32_t r = tid / T, t = tid % T;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < kGemvWaves; ++w) v += red[par][w][r][t];
+            if (row0 + r < N && t < T_real) {
+                if (seg.bias) v += seg.bias[row0 + r];
+                store_out(seg.y + (size_t)t * N + row0 + r, v);
+            }
+        }
     }
 }
 
@@ -264,6 +316,17 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
     const uint32_t KT = (K256 + n_tiles - 1) / n_tiles * 256;   // balanced tiles
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
+    if constexpr (T == 1 && F::SUM_GRAN == 16) {
+        // long rows, too few of them to give every CU its workgroups: the workgroup-wide row walk.  Measured at
+        // K = 14336, N = 4096: Q6_K 14.4 -> 12.7 us; no gain for the formats with 64-byte units or for T = 2.
+        if (n_tiles == 1 && K >= 8192 && n_rg <= 2u * (uint32_t)cu_count()) {
+            const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu / nseg;
+            dim3 gridw(N < capw ? N : capw, nseg);
+            hipLaunchKernelGGL((gemv_q8_wide_kernel<F, 1, 1, OutT>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, F::SUM_GRAN), st, s0, s1, xq8, K, N, KT,
+                               T_real, split ? 1u : 0u);
+            return launch_status();
+        }
+    }
     // A CU streams at a fixed rate (its waves' loads in flight over the memory latency), so the
     // launch is balanced per CU, not per workgroup: with a whole number of workgroups per CU
     // the dispatcher gives every CU the same number of them, and the strided row-group loop
