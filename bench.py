@@ -349,17 +349,30 @@ def main():
             omp.omp_set_num_threads(1)
         except OSError:
             omp = None
+        # Where oracle/_ref (the reference's own host code, built where the reference tree was mounted) is present,
+        # the timed loop runs the reference's ie::ref::dequant_*_buffer itself; otherwise the oracle's restatement.
+        ref = O.load_ref()
+        ybuf = np.empty(max(H, FF), np.float32)
+
+        def cpu_gemv(f, w, a, K, N):
+            if ref is not None:
+                a32 = np.ascontiguousarray(a, np.float32).ravel()
+                assert ref.ref_gemv_cpu(f, w.ctypes.data, a32.ctypes.data, ybuf.ctypes.data, K, N) == 0
+            else:
+                O.gemv_f32chain(f, w, a, K, N)
+
         while t_cpu < 10.0 and reps < 50:
             for f, w, a, K, N in host:
                 c0 = time.perf_counter()
-                O.gemv_f32chain(f, w, a, K, N)
+                cpu_gemv(f, w, a, K, N)
                 t_cpu += time.perf_counter() - c0
                 tot_b += w.nbytes
             reps += 1
-        out["cpu_baseline"] = {"value": round(tot_b / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        out["cpu_baseline"] = {"value": round(tot_b / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "reference" if ref is not None else "port",
                                "sample": "gate (4096->14336) and down (14336->4096) GEMV in Q6_K and Q8_0, T=1, %d repetitions, "
-                                         "weight bytes / time; dequant-to-fp32 + sequential fp32 dot as in the reference's "
-                                         "tests/unit/gemv_q4k_test.cpp" % reps}
+                                         "weight bytes / time; dequant-to-fp32 (%s) + sequential fp32 dot as in the reference's "
+                                         "tests/unit/gemv_q4k_test.cpp" % (reps, "the reference's ie::ref::dequant_*_buffer, oracle/_ref"
+                                                                           if ref is not None else "oracle restatement")}
         if omp is not None:
             n_thr = min(16, os.cpu_count() or 1)
             omp.omp_set_num_threads(n_thr)
