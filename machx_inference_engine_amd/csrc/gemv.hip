@@ -120,6 +120,60 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, O
     }
 }
 
+// Batched launches with long rows and few of them (T >= 2, K >= 8192, N <= 16384: the down projections in
+// a speculative-verify batch): the row-group grid alone leaves CUs idle and every workgroup restages
+// several activation tiles.  Here the grid is (row groups, K slices): a workgroup stages one slice once and
+// writes its partial sums to a per-device scratch plane; a second, tiny launch adds the slices in slice
+// order and writes y.  (A single launch with a last-arriver reduction needs device-scope fences, which on
+// this part write back the XCD's L2: measured five times slower than the two launches.)
+// The scratch is a file-scope device array: launches that overlap on one device would race on it (as the
+// reference's static per-device scratch buffers do, src/model/dense_dispatch.hpp:547-560).
+constexpr uint32_t kSplitMaxN = 16384, kSplitMaxT = 8, kSplitMaxSlices = 4;
+__device__ float g_splitk_part[kSplitMaxSlices][kSplitMaxT][kSplitMaxN];
+
+template <class F, int T, int R, int G>
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_splitk_kernel(typename F::W w, const uint8_t* xq8, uint32_t K, uint32_t N, uint32_t KS,
+                                                                       uint32_t T_real, uint32_t q8_split) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    const uint32_t rg = blockIdx.x, ks = blockIdx.y;
+    const uint32_t k0 = ks * KS, kt = (K - k0 < KS) ? K - k0 : KS;
+    const size_t q8_row_bytes = (size_t)(K / 32) * (q8_split ? kQ81sBytes : kQ81xBytes);
+    auto xrow = [&](uint32_t t) { return xq8 + (size_t)(t < T_real ? t : T_real - 1) * q8_row_bytes; };
+    const ActTile act = stage_act<F::SUM_GRAN, T>(lds, xrow, k0, kt, KS, q8_split != 0);
+    __syncthreads();
+    const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
+    float acc[R][T];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[r][t] = 0.f;
+    typename F::Cursor cu[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) cu[r] = F::cursor(w, (row0 + r < N) ? row0 + r : N - 1, k0 / 64 + gl);
+    gemv_rows<F, T, R, G, 1>(cu, (kt + 63) / 64, (kt & 63u) != 0, gl, act, acc);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const float v = group_sum<G>(acc[r][t]);
+            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N) g_splitk_part[ks][t][row0 + r] = v;
+        }
+}
+
+template <class OutT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(OutT* y, const float* bias, uint32_t N, uint32_t T_real, uint32_t n_split) {
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (row >= N || t >= T_real) return;
+    float v = 0.f;
+    for (uint32_t k = 0; k < n_split; ++k) v += g_splitk_part[k][t][row];
+    if (bias) v += bias[row];
+    store_out(y + (size_t)t * N + row, v);
+}
+
 // Up to three matrices of different N that share one quantized activation row, in one launch: the
 // workgroups tile the concatenated row space, so small projections (GQA k / v) ride a full grid
 // (gemv_q4_0_soa_q8_multi, include/ie/ops.hpp:577-592).  T = 1.
@@ -325,6 +379,22 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
             hipLaunchKernelGGL((gemv_q8_wide_kernel<F, 1, 1, OutT>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, F::SUM_GRAN), st, s0, s1, xq8, K, N, KT,
                                T_real, split ? 1u : 0u);
             return launch_status();
+        }
+    }
+    if constexpr (T >= 2) {
+        const uint32_t cus = (uint32_t)cu_count();
+        if (nseg == 1 && K >= 8192 && N <= kSplitMaxN && (n_tiles > 1 || n_rg < 2u * cus)) {
+            uint32_t n_split = (4u * cus + n_rg - 1) / n_rg;   // about four workgroups per CU
+            if (n_split < n_tiles) n_split = n_tiles;
+            if (n_split > kSplitMaxSlices) n_split = kSplitMaxSlices;
+            const uint32_t KS = (K256 + n_split - 1) / n_split * 256;
+            n_split = (K + KS - 1) / KS;
+            if (n_split >= 2 && KS <= KT_max) {
+                hipLaunchKernelGGL((gemv_q8_splitk_kernel<F, T, R, G>), dim3(n_rg, n_split), dim3(kGemvThreads), act_tile_bytes(T, KS, F::SUM_GRAN), st,
+                                   s0.w, xq8, K, N, KS, T_real, split ? 1u : 0u);
+                hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((N + 255) / 256, T_real), dim3(256), 0, st, s0.y, s0.bias, N, T_real, n_split);
+                return launch_status();
+            }
         }
     }
     // A CU streams at a fixed rate (its waves' loads in flight over the memory latency), so the

@@ -262,3 +262,19 @@ def test_gemv_q8_x2_equals_two_single_launches(mx, fmt):
         sa, sb = [tuple(dev(p) for p in O.repack_q8_0_to_soa(W)) for W in (Wa, Wb)]
         ya2, yb2 = mx.ops.gemv_q8_x2("q8_0_soa", xq, sa, sb, K, N)
         assert torch.equal(ya2, mx.ops.gemv_q8_0_soa_q8(xq, sa[0], sa[1], K, N)) and torch.equal(yb2, mx.ops.gemv_q8_0_soa_q8(xq, sb[0], sb[1], K, N))
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+@pytest.mark.parametrize("T", (2, 5, 8, 13))
+def test_gemv_q8_batched_long_rows_split_k(mx, fmt, T):
+    """Batched launches at K >= 8192 with few rows run as (row groups x K slices) plus a small reduction launch:
+    results against the q8-chain oracle, and identical from launch to launch (the slices are added in slice order)."""
+    K, N = 14336, 200
+    W = weights(fmt, 1500 + fmt, N, K)
+    xq = O.quantize_q8_1(acts(1510 + T, T, K))
+    ref = O.gemv_q8chain(fmt, W, xq, K, N)
+    first = run_q8(mx, fmt, W, xq, K, N, T)
+    for t in range(T):
+        check(first[t], ref[t], "%s K=%d T=%d row %d" % (O.FMT_NAMES[fmt], K, T, t))
+    for _ in range(3):
+        assert np.array_equal(run_q8(mx, fmt, W, xq, K, N, T), first)
