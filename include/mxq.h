@@ -137,7 +137,11 @@ int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x_q8, const uint8_t* gate
  * gemv_q6_soa_q8_batched include/ie/ops.hpp:420-426 (the reference batches Q6_K only
  *                        in its SoA form; here the GGUF AoS blocks are batched directly)
  * Q8_0 / MXFP4 batched have no reference counterpart (T >= 2 falls to dequant +
- * GEMM there, src/model/qwen35_dense.cpp:811-831).  */
+ * GEMM there, src/model/qwen35_dense.cpp:811-831).
+ * Batched launches with K >= 8192 and N <= 16384 split K over workgroups and keep their partial sums in
+ * a 2 MB per-device scratch array owned by the library (nothing is allocated): two such calls that
+ * overlap on one device (different streams) would race on it, exactly as calls sharing the reference's
+ * static per-device scratch buffers would (src/model/dense_dispatch.hpp:547-560).  */
 int mx_gemv_q4_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 /* gemv_q4_K_q8s_batched  include/ie/ops.hpp (gemv_q4_K_q8s_batched), src/ops/gemv_q8dot.cpp:483-597: the
  * activation rows are block_q8_1s (48 B, stored half sums s0/s1; 16-byte aligned) from
