@@ -49,8 +49,8 @@ def main():
                     help="counter probe for `rocprofv3 --pmc`: a few launches of the dominant kernels and of a plain copy of known size, no timing")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.stderr.write("bench.py: this build measures one GPU only (the path is data-parallel over output rows / experts; "
-                         "see DESIGN.md for how it shards); run with --gpus 1\n")
+        sys.stderr.write("bench.py: this build measures one GPU only (the path is data-parallel over output rows / experts, "
+                         "so more GPUs would each take a slice of rows or experts); run with --gpus 1\n")
         sys.exit(2)
 
     import torch
