@@ -3,7 +3,7 @@
 Run in a container where the reference tree is mounted and oracle/_ref was built
 (`make -C oracle`).  Inputs come from the oracle's counter-based RNG (seeds
 below); expected outputs come from oracle/_ref/libmxref.so, i.e. from
-ie::ref::dequant_*, ie::quantize_row_q4_K/q6_K, ie::build_moe_packing,
+ie::ref::dequant_*, ie::quantize_row_q4_K/q6_K, ie::build_moe_packing, ie::repack_moe_q{4,6}k_soa_host,
 ie::fp16_to_fp32/fp32_to_fp16 and ie::ref::get_scale_min_k4 compiled from the
 reference sources.  Only data is stored: inputs and the reference's outputs.
 
@@ -90,6 +90,14 @@ def main():
     out["dp4a_us"] = np.array([r.ref_dp4a_us(int(x), int(y), 7) for x, y in zip(a, b)], np.int32)
     out["dp4a_ss"] = np.array([r.ref_dp4a_ss(int(np.int32(x)), int(y), -3) for x, y in zip(a.view(np.int32), b)], np.int32)
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref_vectors.npz")
+    # per-expert stream repacks (ie::repack_moe_q4k_soa_host / _q6k_soa_host, include/ie/quant_soa.hpp:127-157)
+    for fmt, fn in ((O.Q4_K, r.ref_repack_moe_q4k_soa), (O.Q6_K, r.ref_repack_moe_q6k_soa)):
+        E, nb = 3, 20
+        bank = O.rand_bytes(0x50A50A + fmt, E * nb * O.BLOCK_BYTES[fmt])
+        soa = np.empty_like(bank)
+        fn(bank.ctypes.data, soa.ctypes.data, E, nb)
+        out["soa_in_%s" % O.FMT_NAMES[fmt]] = bank
+        out["soa_out_%s" % O.FMT_NAMES[fmt]] = soa
     np.savez_compressed(dst, **out)
     print("wrote", dst, os.path.getsize(dst), "bytes")
 

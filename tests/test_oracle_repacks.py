@@ -25,6 +25,17 @@ def test_stream_repack_matches_reference_host_code(fmt):
     assert np.array_equal(O.repack_kquant_streams(fmt, bank, E, nb), want)
 
 
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K))
+def test_stream_repack_matches_reference_golden(fmt):
+    """The same check against vectors written from the reference's host code (tests/golden/make_golden.py),
+    for where oracle/_ref is not built."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors.npz"))
+    name = O.FMT_NAMES[fmt]
+    assert np.array_equal(O.repack_kquant_streams(fmt, g["soa_in_" + name], 3, 20), g["soa_out_" + name])
+    assert np.array_equal(ops.repack_moe_kquant_soa("q4k" if fmt == O.Q4_K else "q6k", g["soa_in_" + name], 3, 20), g["soa_out_" + name])
+
+
 def test_stream_layout_probe():
     """One region of two Q4_K blocks: qs x 2 | scales x 2 | {d,dmin} x 2 (include/ie/quant_soa.hpp:33-41)."""
     bank = np.arange(288, dtype=np.uint16).astype(np.uint8)   # byte i = i mod 256
