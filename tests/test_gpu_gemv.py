@@ -278,3 +278,13 @@ def test_gemv_q8_batched_long_rows_split_k(mx, fmt, T):
         check(first[t], ref[t], "%s K=%d T=%d row %d" % (O.FMT_NAMES[fmt], K, T, t))
     for _ in range(3):
         assert np.array_equal(run_q8(mx, fmt, W, xq, K, N, T), first)
+
+
+@pytest.mark.parametrize("K,N,seed", [(12288, 4096, 0x6C01), (4096, 2048, 0x6C02), (12288 + 256, 1024, 0x6C03), (2304, 257, 0x6C04), (2048, 512, 0x6C05)])
+def test_gemv_q6_K_q8_reference_ktiled_shapes(mx, K, N, seed):
+    """The five shapes of the reference's K-tiled Q6_K test (tests/gemv_q6k_ktiled_test.cpp:195-208: the qwen3-8b
+    ffn_down decode shape, a fitting K, a partial last K tile, odd N, exactly one tile), against the q8-chain oracle
+    as there (:89-103)."""
+    W = weights(O.Q6_K, seed, N, K)
+    xq = O.quantize_q8_1(acts(seed + 16, 1, K))
+    check(run_q8(mx, O.Q6_K, W, xq, K, N, 1), O.gemv_q8chain(O.Q6_K, W, xq, K, N)[0], "gemv_q6_K_q8 K=%d N=%d" % (K, N))

@@ -72,7 +72,8 @@ def test_natural_order_probes():
     assert hi[49] == 0x20 and hi.sum() == 0x20                # byte 198//4, bits 2*(198&3) = 4..5, value 2
 
 
-@pytest.mark.parametrize("K,N", [(256, 3), (1024, 7)])
+# the shapes of the reference's own host-side check of this repack (tools/q4_soa_test.cpp:75-77) plus two more
+@pytest.mark.parametrize("K,N", [(256, 1), (256, 5), (512, 3), (2048, 7), (768, 4), (256, 64), (1024, 7)])
 def test_natural_order_repack_keeps_every_value(K, N):
     W4, W6 = blocks(O.Q4_K, 920, N, K), blocks(O.Q6_K, 921, N, K)
     assert np.array_equal(O.dequant_q4_soa(O.repack_q4_K_to_soa(W4)).view(np.uint32), O.dequant(O.Q4_K, W4).view(np.uint32))
