@@ -301,6 +301,22 @@ int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* do
 int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
                          const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
                          uint64_t expert_stride_bytes, uint32_t total_rows);
+/* Q4_0 expert banks (Gemma-4 MoE) and the dense W4A8 GEMM; plain projections, no epilogue:
+ *   moe_prefill_proj_q4_0_q8      include/ie/ops.hpp:166-177   block_q8_1s rows, GGUF blocks, expert e at W + e*expert_stride_bytes
+ *   moe_prefill_proj_q4_0_soa_q8  include/ie/ops.hpp:179-190   block_q8_1s rows, planes: qs_bank + e*qs_stride bytes, d_bank + e*d_stride entries
+ *   moe_prefill_proj_q4_0_xmx     include/ie/ops.hpp:192-204   fp16 rows, matrix cores (K % 128 == 0 here; the reference needs K % 256, N % 64)
+ *   gemm_q4_0_q8                  include/ie/ops.hpp:538-548   y[M,N] = q8(x)[M,K] . W, any M and any K % 32 == 0, int-dot
+ * out_packed[row, n] = half(acc); rows of expert e are [expert_offsets[e], expert_offsets[e+1]); total_rows = expert_offsets[E].  */
+int mx_moe_prefill_proj_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, const uint32_t* expert_offsets,
+                                uint16_t* out_packed, uint32_t E, uint32_t K, uint32_t N, uint64_t expert_stride_bytes,
+                                uint32_t total_rows);
+int mx_moe_prefill_proj_q4_0_soa_q8(mx_stream_t s, const void* xq8s_packed, const uint8_t* qs_bank, const uint16_t* d_bank,
+                                    const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t K, uint32_t N,
+                                    uint64_t qs_stride, uint64_t d_stride, uint32_t total_rows);
+int mx_moe_prefill_proj_q4_0_xmx(mx_stream_t s, const uint16_t* x_fp16, const void* W_q4_0, const uint32_t* expert_offsets,
+                                 uint16_t* out_packed, uint32_t E, uint32_t K, uint32_t N, uint64_t expert_stride_bytes,
+                                 uint32_t total_rows);
+int mx_gemm_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 /* Accumulate form of the down projection (the reference's first prefill path), same matrix-core kernel
  * with an atomic fp32 epilogue:
  *   moe_prefill_down_q4k / _q6k       include/ie/ops.hpp:930-954, src/ops/moe_fused.cpp:937-1085

@@ -844,6 +844,19 @@ int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* do
                                                 total_rows, kQ6KBytes, 2);
 }
 
+// moe_prefill_proj_q4_0_xmx (include/ie/ops.hpp:192-204): plain projection of expert-sorted fp16 rows through Q4_0 experts.
+int mx_moe_prefill_proj_q4_0_xmx(mx_stream_t s, const uint16_t* x_fp16, const void* W_q4_0, const uint32_t* expert_offsets, uint16_t* out_packed,
+                                 uint32_t E, uint32_t K, uint32_t N, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    if (int rc = check_gemm(x_fp16, W_q4_0, out_packed, total_rows, K, N, 128, 2)) return rc;
+    MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(E > 0 && expert_stride_bytes % 2 == 0);
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(x_fp16); g.Y = reinterpret_cast<half_t*>(out_packed); g.expert_offsets = expert_offsets;
+    g.M = total_rows; g.K = K; g.N = N; g.E = E;
+    GemmQ40::Bank b{static_cast<const uint8_t*>(W_q4_0), expert_stride_bytes, K / 32 * 18u};
+    return launch_gemm<GemmQ40, GEMM_MOE_DOWN>(s, b, b, g, total_rows);
+}
+
 // Accumulate form of the down projection (moe_prefill_down_q4k / _q6k, include/ie/ops.hpp:930-954):
 // y_fp32[sorted_token_idx[row], n] += sorted_token_w[row] * (down_e . h_row)[n], fp32 atomics.
 int mx_moe_prefill_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const int32_t* sorted_token_idx,

@@ -32,6 +32,7 @@ struct MoeArgs {
     uint32_t act_div;                // activation row of output row r is r / act_div
     uint32_t K, N, KT, n_experts;
     uint32_t q8_split;               // activation rows are block_q8_1s (48 B) instead of block_q8_1x
+    uint32_t n_rows;                 // dense mode (no topk_idx, no expert_offsets): one weight matrix, rows [0, n_rows)
 };
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
@@ -53,10 +54,14 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
         e = (uint32_t)a.topk_idx[seg];
         r_begin = seg;
         r_end = seg + 1;
-    } else {
+    } else if (a.expert_offsets) {
         e = seg;
         r_begin = a.expert_offsets[seg];
         r_end = a.expert_offsets[seg + 1];
+    } else {
+        e = 0;
+        r_begin = 0;
+        r_end = a.n_rows;
     }
     if (r_begin >= r_end || e >= a.n_experts) return;   // empty expert / invalid id: uniform for the block
     const typename F::W w0 = F::expert(bank0, e), w1 = F::expert(NW == 2 ? bank1 : bank0, e);
@@ -562,6 +567,46 @@ int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8
     MX_REQUIRE_PTR(expert_offsets);
     return moe_mxfp4_down(s, hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
                           grouped_tt(total_rows, E));
+}
+
+// ------------------------------------------------------------ Q4_0 experts (Gemma-4 MoE) and the dense W4A8 GEMM
+// Plain projections out_packed[row, n] = half(W_e[n, :] . q8(x_row)), rows partitioned by expert_offsets.
+int mx_moe_prefill_proj_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, const uint32_t* expert_offsets, uint16_t* out_packed,
+                                uint32_t E, uint32_t K, uint32_t N, uint64_t expert_stride_bytes, uint32_t total_rows) {
+    if (int rc = check_moe(xq8s_packed, out_packed, K, N, E)) return rc;
+    MX_REQUIRE_PTR(W_q4_0); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(expert_stride_bytes % 2 == 0);
+    MX_REQUIRE_ALIGN(W_q4_0, 2); MX_REQUIRE_ALIGN(xq8s_packed, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out_packed);
+    a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = 1;
+    FmtQ40Aos::Bank b{static_cast<const uint8_t*>(W_q4_0), expert_stride_bytes, K / 32 * 18u};
+    return launch_moe<FmtQ40Aos, 1, EPI_DOWN_BIAS>(s, b, b, a, E, grouped_tt(total_rows, E));
+}
+int mx_moe_prefill_proj_q4_0_soa_q8(mx_stream_t s, const void* xq8s_packed, const uint8_t* qs_bank, const uint16_t* d_bank,
+                                    const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t K, uint32_t N, uint64_t qs_stride,
+                                    uint64_t d_stride, uint32_t total_rows) {
+    if (int rc = check_moe(xq8s_packed, out_packed, K, N, E)) return rc;
+    MX_REQUIRE_PTR(qs_bank); MX_REQUIRE_PTR(d_bank); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(qs_bank, 16); MX_REQUIRE_ALIGN(d_bank, 2); MX_REQUIRE_ALIGN(xq8s_packed, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out_packed);
+    a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = 1;
+    FmtQ40Soa::Bank b{qs_bank, d_bank, qs_stride, d_stride, K};
+    return launch_moe<FmtQ40Soa, 1, EPI_DOWN_BIAS>(s, b, b, a, E, grouped_tt(total_rows, E));
+}
+// gemm_q4_0_q8: y[M, N] = q8(x)[M, K] . W[N, K]^T for any M, int-dot: the rows run as token tiles of 8 over one matrix.
+int mx_gemm_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    if (int rc = check_moe(xq8s_packed, y, K, N, 1)) return rc;
+    MX_REQUIRE_PTR(W_q4_0);
+    MX_REQUIRE_SHAPE(M > 0);
+    MX_REQUIRE_ALIGN(W_q4_0, 2); MX_REQUIRE_ALIGN(xq8s_packed, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.out = reinterpret_cast<half_t*>(y);
+    a.act_div = 1; a.K = K; a.N = N; a.n_experts = 1; a.q8_split = 1; a.n_rows = M;
+    FmtQ40Aos::Bank b{static_cast<const uint8_t*>(W_q4_0), 0, K / 32 * 18u};
+    return launch_moe<FmtQ40Aos, 1, EPI_DOWN_BIAS>(s, b, b, a, 1, M == 1 ? 1u : (M <= 4 ? 4u : 8u));
 }
 
 // ------------------------------------------------------------ row utilities

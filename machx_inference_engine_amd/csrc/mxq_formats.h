@@ -555,6 +555,14 @@ struct FmtQ40Soa {
         const uint16_t* d;
         uint32_t K;
     };
+    // expert e: qs + e*qs_stride bytes, d + e*d_stride fp16 entries (include/ie/ops.hpp:179-190)
+    struct Bank {
+        const uint8_t* qs;
+        const uint16_t* d;
+        uint64_t qs_stride, d_stride;
+        uint32_t K;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.qs + (size_t)e * b.qs_stride, b.d + (size_t)e * b.d_stride, b.K}; }
     struct Cursor {
         const uint4* qs;
         const uint8_t* d;
@@ -610,6 +618,12 @@ struct FmtQ40Aos {
         const uint8_t* base;
         uint32_t row_bytes;
     };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
     struct Cursor {
         const uint8_t* blk;
     };

@@ -416,6 +416,23 @@ def gemm_q4_0(A, W, M, K, N, y=None):
     return y
 
 
+def moe_prefill_proj_q4_0(kind, rows, W, expert_offsets, TK, E, K, N, stride, out_packed=None):
+    """kind 'q8' (rows = block_q8_1s stream, W = GGUF blocks, stride = expert_stride_bytes), 'soa_q8' (W = (qs_bank, d_bank),
+    stride = (qs_stride, d_stride)) or 'xmx' (rows = fp16 [TK, K], W = GGUF blocks)."""
+    out_packed = _out(out_packed, (TK, N), torch.float16, rows)
+    if kind == "soa_q8":
+        _call("mx_moe_prefill_proj_q4_0_soa_q8", _ptr(rows), _u8(W[0]), _ptr(W[1]), _ptr(expert_offsets), _ptr(out_packed), E, K, N, stride[0], stride[1], TK)
+    else:
+        _call("mx_moe_prefill_proj_q4_0_%s" % kind, _ptr(rows), _u8(W), _ptr(expert_offsets), _ptr(out_packed), E, K, N, stride, TK)
+    return out_packed
+
+
+def gemm_q4_0_q8(xq8s, W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, xq8s)
+    _call("mx_gemm_q4_0_q8", _ptr(xq8s), _u8(W), _ptr(y), M, K, N)
+    return y
+
+
 def repack_q4_0_to_soa(W, K, N):
     W = _np_u8(W)
     qs, d = np.empty(N * K // 2, np.uint8), np.empty(N * K // 32, np.uint16)

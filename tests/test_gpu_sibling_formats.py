@@ -89,3 +89,50 @@ def test_gemv_q5_K(mx, K, N, T):
     if T == 1:
         y16 = ops.gemv_q5_K(dev(x[0]).half(), dev(W), K, N)
         check(host(y16).astype(np.float32), O.gemv_f64(O.Q5_K, W, x, K, N)[0], "gemv_q5_K (fp16 activations)")
+
+
+@pytest.mark.parametrize("T,E,Kt,K,N", [(40, 6, 2, 736, 200), (96, 8, 2, 1024, 512)])
+def test_moe_prefill_proj_q4_0(mx, T, E, Kt, K, N):
+    """moe_prefill_proj_q4_0_q8 / _soa_q8 / _xmx (include/ie/ops.hpp:166-204): plain projections of expert-sorted rows
+    through Q4_0 experts; the int-dot forms against the q8-chain oracle expert by expert, the matrix-core form against
+    the float chain with fp16-rounded weights."""
+    ops = mx.ops
+    Ws = np.stack([weights(O.Q4_0, 6500 + e, N, K) for e in range(E)])
+    x = acts(6510, T, K)
+    rng = np.random.default_rng(6511)
+    ids = np.stack([np.sort(rng.choice(E, size=Kt, replace=False)) for _ in range(T)]).astype(np.int32)
+    off, si, wp, t2p = ops.build_moe_packing(ids, np.full(ids.shape, 0.5, np.float32), E)
+    TK = T * Kt
+    xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, K)
+    xq_s = ops.quantize_q8_1s(xp)
+    xq_x = host(ops.quantize_q8_1(xp)).reshape(TK, -1)      # same quants and d in the 40-byte layout, for the oracle
+    stride = Ws[0].size
+    got = ops.moe_prefill_proj_q4_0("q8", xq_s, dev(Ws), dev(off), TK, E, K, N, stride)
+    ref = np.zeros((TK, N), np.float64)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            ref[off[e]:off[e + 1]] = O.gemv_q8chain(O.Q4_0, Ws[e], xq_x[off[e]:off[e + 1]], K, N)
+    check(host(got).astype(np.float32).ravel(), ref.ravel(), "moe_prefill_proj_q4_0_q8")
+    planes = [ops.repack_q4_0_to_soa(Ws[e], K, N) for e in range(E)]
+    qs_bank, d_bank = np.concatenate([p[0] for p in planes]), np.concatenate([p[1] for p in planes])
+    got_soa = ops.moe_prefill_proj_q4_0("soa_q8", xq_s, (dev(qs_bank), dev(d_bank)), dev(off), TK, E, K, N, (N * K // 2, N * K // 32))
+    assert torch.equal(got_soa, got)
+    if K % 128 == 0:
+        got_x = ops.moe_prefill_proj_q4_0("xmx", xp, dev(Ws), dev(off), TK, E, K, N, stride)
+        xs = x[si]
+        ref_x = np.zeros((TK, N), np.float64)
+        for e in range(E):
+            if off[e + 1] > off[e]:
+                ref_x[off[e]:off[e + 1]] = O.gemv_f64(O.Q4_0, Ws[e], xs[off[e]:off[e + 1]], K, N, round_w_fp16=True)
+        check(host(got_x).astype(np.float32).ravel(), ref_x.ravel(), "moe_prefill_proj_q4_0_xmx")
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 64, 8), (5, 736, 130), (37, 2048, 300)])
+def test_gemm_q4_0_q8(mx, M, K, N):
+    """gemm_q4_0_q8 (include/ie/ops.hpp:538-548): int-dot GEMM over block_q8_1s rows, any M, any K % 32 == 0."""
+    W = weights(O.Q4_0, 6600 + M, N, K)
+    x = acts(6601, M, K)
+    xq_s = mx.ops.quantize_q8_1s(dev(x).half())
+    y = mx.ops.gemm_q4_0_q8(xq_s, dev(W), M, K, N)
+    ref = O.gemv_q8chain(O.Q4_0, W, O.quantize_q8_1(x), K, N)
+    check(host(y).astype(np.float32).ravel(), ref.ravel(), "gemm_q4_0_q8 M=%d" % M)
