@@ -127,20 +127,20 @@ __device__ __forceinline__ void q4k_scale_pair(uint32_t s0, uint32_t s1, uint32_
     }
 }
 
-// MXFP4 codes -> doubled E2M1 values as int8, four at a time.  `sel` holds the
-// 3 magnitude bits of four codes (one per byte), `sgn` the sign bit of each in
-// bit 0 of its byte.  LUT {0,1,2,3,4,6,8,12} / {0,-1,...,-12} via two byte
-// permutes and a per-byte select (include/ie/quant_blocks.hpp:46-54).
-__device__ __forceinline__ uint32_t mxfp4_lut4(uint32_t sel, uint32_t sgn) {
+// MXFP4 codes -> doubled E2M1 values as int8, four at a time.  `sel` holds the 3 magnitude bits of
+// four codes (one per byte); `pick` byte i is i for a positive code and 4 + i for a negative one.
+// LUT {0,1,2,3,4,6,8,12} / {0,-1,...,-12} by two byte permutes, then a third permute takes byte i from
+// the positive or the negative result (include/ie/quant_blocks.hpp:46-54).
+__device__ __forceinline__ uint32_t mxfp4_lut4(uint32_t sel, uint32_t pick) {
     const uint32_t pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
     const uint32_t neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
-    const uint32_t m = (sgn << 8) - sgn;  // 0xFF in every byte whose sign bit is set
-    return (pos & ~m) | (neg & m);
+    return __builtin_amdgcn_perm(neg, pos, pick);
 }
-// One qs dword (bytes j..j+3 of a block) -> codes of elements j..j+3 (lo) and 16+j..16+j+3 (hi)
+// One qs dword (bytes j..j+3 of a block) -> codes of elements j..j+3 (lo) and 16+j..16+j+3 (hi).
+// The sign bit of a code (bit 3 / bit 7 of its byte) lands on bit 2 of the pick byte.
 __device__ __forceinline__ void mxfp4_decode_word(uint32_t w, uint32_t& lo, uint32_t& hi) {
-    lo = mxfp4_lut4(w & 0x07070707u, (w >> 3) & 0x01010101u);
-    hi = mxfp4_lut4((w >> 4) & 0x07070707u, (w >> 7) & 0x01010101u);
+    lo = mxfp4_lut4(w & 0x07070707u, ((w >> 1) & 0x04040404u) | 0x03020100u);
+    hi = mxfp4_lut4((w >> 4) & 0x07070707u, ((w >> 5) & 0x04040404u) | 0x03020100u);
 }
 
 }  // namespace mxq
