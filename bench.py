@@ -291,10 +291,14 @@ def main():
                 b = banks[i % nrep]
                 if T == 1:    # device-side expert ids, one launch per stage
                     ops.moe_gate_up_oai_mxfp4(xq8, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, idsd, T, K4, H4, H4, E4, h_out=hbuf)
-                    ops.quantize_q8_1(hbuf, hq8)
-                    ops.moe_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
+                    if args.unfused:
+                        ops.quantize_q8_1(hbuf, hq8)
+                        ops.moe_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
+                    else:     # h quantized while the down launch stages it: same bits, one launch fewer
+                        ops.moe_down_mxfp4_f16(hbuf, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
                 else:         # expert-grouped rows, each routed expert streamed once
                     ops.moe_grouped_gate_up_oai_mxfp4(xpq, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, offd, TK, E4, H4, H4, h_packed=hbuf)
+                    # with 128 rows every workgroup would requantize all of them: the separate quantize launch is cheaper here
                     ops.quantize_q8_1(hbuf, hq8)
                     ops.moe_grouped_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, offd, TK, E4, H4, H4, out_packed=obuf)
 

@@ -438,6 +438,19 @@ int mx_moe_grouped_gate_up_oai_mxfp4(mx_stream_t s, const void* xq8_packed, cons
 int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
                               uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed,
                               uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+/* Down projections that take h as fp16 rows and quantize it while staging it (the staged tile is bit-identical to
+ * staging mx_quantize_q8_1(h)), so the quantize launch between the two expert stages disappears.  No counterpart in
+ * the reference (it launches quantize_q8_1 between swiglu and the down GEMV, src/model/gptoss.cpp:400-412).
+ * h rows 16-byte aligned; otherwise the arguments of mx_moe_down_mxfp4 / mx_moe_grouped_down_mxfp4 / mx_moe_down_q8.  */
+int mx_moe_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_f16, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
+                          uint64_t e_stride, const float* down_bias, const int32_t* topk_idx, uint16_t* out_packed, uint32_t T,
+                          uint32_t K, uint32_t E_ffn, uint32_t H, uint32_t n_experts);
+int mx_moe_grouped_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_packed_f16, const uint8_t* d_qs, const uint8_t* d_e,
+                                  uint64_t qs_stride, uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets,
+                                  uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                       uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
+                       uint32_t K, uint32_t E_ffn, uint32_t H);
 /* ---------------------------------------------------------------- MoE routing and packing on the device
  *   moe_router             include/ie/ops.hpp:780-786, src/ops/moe.cpp:22-216
  *     logits = W_gate[E,H] (fp32) . x_t, softmax, top-k, renormalise, ascending expert id; any

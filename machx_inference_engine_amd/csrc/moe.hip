@@ -33,6 +33,7 @@ struct MoeArgs {
     uint32_t K, N, KT, n_experts;
     uint32_t q8_split;               // activation rows are block_q8_1s (48 B) instead of block_q8_1x
     uint32_t n_rows;                 // dense mode (no topk_idx, no expert_offsets): one weight matrix, rows [0, n_rows)
+    const half_t* act_f16;           // when set: activation rows are fp16 [rows][K] and are quantized while they are staged
 };
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
@@ -94,7 +95,12 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
                 }
                 if (n_tiles > 1 || !staged) {
                     __syncthreads();
-                    act = stage_act<F::SUM_GRAN, TT>(lds, xrow, k0, kt, KT, a.q8_split != 0);
+                    if (a.act_f16) {
+                        auto hrow = [&](uint32_t t) { return a.act_f16 + (size_t)((t0 + (t < nt ? t : nt - 1)) / a.act_div) * K; };
+                        act = stage_act_f16<F::SUM_GRAN, TT>(lds, hrow, k0, kt, KT);
+                    } else {
+                        act = stage_act<F::SUM_GRAN, TT>(lds, xrow, k0, kt, KT, a.q8_split != 0);
+                    }
                     __syncthreads();
                     staged = true;
                 }
@@ -544,14 +550,16 @@ int mx_moe_grouped_gate_up_oai_mxfp4(mx_stream_t s, const void* xq8_packed, cons
 }
 static int moe_mxfp4_down(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
                           const float* down_bias, const int32_t* topk_idx, const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t n_seg,
-                          uint32_t E_ffn, uint32_t H, uint32_t n_experts, uint32_t tt) {
+                          uint32_t E_ffn, uint32_t H, uint32_t n_experts, uint32_t tt, bool act_is_f16 = false) {
     if (int rc = check_moe(h_q8, out_packed, E_ffn, H, n_seg)) return rc;
+    if (act_is_f16) MX_REQUIRE_ALIGN(h_q8, 16);
     MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_e);
     MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
     MX_REQUIRE_ALIGN(d_qs, 16);
     MoeArgs a{};
     a.xq8 = static_cast<const uint8_t*>(h_q8); a.topk_idx = topk_idx; a.expert_offsets = expert_offsets; a.bias0 = down_bias;
     a.out = reinterpret_cast<half_t*>(out_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
+    if (act_is_f16) a.act_f16 = static_cast<const half_t*>(h_q8);
     FmtMxfp4Soa::Bank b{d_qs, d_e, qs_stride, e_stride, E_ffn};
     return launch_moe<FmtMxfp4Soa, 1, EPI_DOWN_BIAS>(s, b, b, a, n_seg, tt);
 }
@@ -567,6 +575,35 @@ int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8
     MX_REQUIRE_PTR(expert_offsets);
     return moe_mxfp4_down(s, hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
                           grouped_tt(total_rows, E));
+}
+
+// The down projections taking h as fp16 and quantizing it while staging (same q8 values as mx_quantize_q8_1(h)): no quantize launch.
+int mx_moe_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_f16, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
+                          const float* down_bias, const int32_t* topk_idx, uint16_t* out_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H,
+                          uint32_t n_experts) {
+    MX_REQUIRE_PTR(topk_idx);
+    return moe_mxfp4_down(s, h_f16, d_qs, d_e, qs_stride, e_stride, down_bias, topk_idx, nullptr, out_packed, T * K, E_ffn, H, n_experts, 1, true);
+}
+int mx_moe_grouped_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_packed_f16, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
+                                  uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E,
+                                  uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    MX_REQUIRE_PTR(expert_offsets);
+    return moe_mxfp4_down(s, h_packed_f16, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
+                          grouped_tt(total_rows, E), true);
+}
+int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                       const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
+    const uint32_t n_experts = 0xFFFFFFFFu;
+    if (int rc = check_moe(h_f16, y_packed, E_ffn, H, T * K)) return rc;
+    MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(topk_w);
+    MX_REQUIRE_SHAPE(qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(d_qs, 16); MX_REQUIRE_ALIGN(h_f16, 16);
+    MoeArgs a{};
+    a.act_f16 = reinterpret_cast<const half_t*>(h_f16); a.xq8 = reinterpret_cast<const uint8_t*>(h_f16); a.topk_idx = topk_idx;
+    a.route_w = reinterpret_cast<const half_t*>(topk_w); a.out = reinterpret_cast<half_t*>(y_packed); a.act_div = 1; a.K = E_ffn; a.N = H;
+    a.n_experts = n_experts;
+    FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
+    return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, T * K, 1);
 }
 
 // ------------------------------------------------------------ Q4_0 experts (Gemma-4 MoE) and the dense W4A8 GEMM

@@ -89,6 +89,66 @@ __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t 
     return ActTile{qs, hdr, KT_alloc};
 }
 
+// The same tile from fp16 rows, quantized on the way in: d = amax/127, q = round-half-away(v * 127/amax),
+// s = d * float(sum q) per 32-element block, exactly quantize_q8_1 (src/ops/gemv_q8dot.cpp:94-124), so the
+// staged tile is bit-identical to staging the quantizer's output.  A thread takes 16 elements; the two
+// threads of a block (adjacent lanes) exchange their maxima and sums.  `hrow(t)` -> first element of row t.
+template <int SUM_GRAN, int T, class RowFn>
+__device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc) {
+    uint4* qs = reinterpret_cast<uint4*>(lds);
+    uint8_t* hdr = lds + (size_t)T * KT_alloc;
+    const uint32_t halves = (kt + 63) / 64 * 4;
+    const uint32_t total = (uint32_t)T * halves, total_up = (total + blockDim.x - 1) / blockDim.x * blockDim.x;
+    for (uint32_t i = threadIdx.x; i < total_up; i += blockDim.x) {   // whole passes: both threads of a block stay converged
+        const bool in = i < total;
+        const uint32_t t = in ? i / halves : 0, hb = in ? i - t * halves : 0;
+        const bool live = in && hb * 16 < kt;
+        float v[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = 0.f;
+        if (live) {
+            const half_t* p = hrow(t) + k0 + hb * 16;
+            const uint4 a = reinterpret_cast<const uint4*>(p)[0], b = reinterpret_cast<const uint4*>(p)[1];
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                v[2 * j] = h2f(w[j] & 0xFFFFu);
+                v[2 * j + 1] = h2f(w[j] >> 16);
+            }
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(v[j]));
+        amax = fmaxf(amax, __shfl_xor(amax, 1));
+        const float d = amax / 127.0f, inv = amax > 0.f ? 127.0f / amax : 0.f;
+        uint32_t q[4];
+        int s16 = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t pk = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int qi = (int)roundf(v[4 * j + b] * inv);
+                s16 += qi;
+                pk |= (uint32_t)(qi & 0xFF) << (8 * b);
+            }
+            q[j] = pk;
+        }
+        const int s32 = s16 + __shfl_xor(s16, 1);
+        if (!in) continue;
+        qs[(size_t)t * (KT_alloc / 16) + hb] = make_uint4(q[0], q[1], q[2], q[3]);
+        if (SUM_GRAN == 16) {
+            reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 16) + hb] = make_float2(d, d * (float)s16);
+        } else if ((hb & 1u) == 0) {
+            if (SUM_GRAN == 32)
+                reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = make_float2(d, d * (float)s32);
+            else
+                reinterpret_cast<float*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = d;
+        }
+    }
+    return ActTile{qs, hdr, KT_alloc};
+}
+
 __device__ __forceinline__ int dot16(const uint32_t (&w)[4], const uint4& x, int c) {
     c = dot4(w[0], x.x, c);
     c = dot4(w[1], x.y, c);

@@ -217,6 +217,14 @@ def moe_down_q8(h_q8, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_
     return y_packed
 
 
+def moe_down_q8_f16(h_f16, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_ffn, H, y_packed=None):
+    """moe_down_q8 on fp16 h rows [T*K][E_ffn], quantized while they are staged (no quantize launch)."""
+    y_packed = _out(y_packed, (T * K, H), torch.float16, h_f16)
+    _call("mx_moe_down_q8_f16", _f16(h_f16), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(topk_idx), _f16(topk_w), _ptr(y_packed),
+          T, K, E_ffn, H)
+    return y_packed
+
+
 def moe_reduce_q8(y_packed, T, K, H, y=None):
     y = _out(y, (T, H), torch.float16, y_packed)
     _call("mx_moe_reduce_q8", _f16(y_packed), _ptr(y), T, K, H)
@@ -323,6 +331,14 @@ def moe_down_mxfp4(h_q8, d_qs, d_e, qs_stride, e_stride, down_bias, topk_idx, T,
     return out_packed
 
 
+def moe_down_mxfp4_f16(h_f16, d_qs, d_e, qs_stride, e_stride, down_bias, topk_idx, T, K, E_ffn, H, n_experts, out_packed=None):
+    """moe_down_mxfp4 on fp16 h rows [T*K][E_ffn], quantized while they are staged (no quantize launch)."""
+    out_packed = _out(out_packed, (T * K, H), torch.float16, h_f16)
+    _call("mx_moe_down_mxfp4_f16", _f16(h_f16), _u8(d_qs), _u8(d_e), qs_stride, e_stride, _ptr(down_bias), _ptr(topk_idx),
+          _ptr(out_packed), T, K, E_ffn, H, n_experts)
+    return out_packed
+
+
 def moe_grouped_gate_up_oai_mxfp4(xq8_packed, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, expert_offsets, TK, E, H,
                                   E_ffn, alpha=1.702, limit=7.0, h_packed=None):
     h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8_packed)
@@ -335,6 +351,14 @@ def moe_grouped_down_mxfp4(hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias
     out_packed = _out(out_packed, (TK, H), torch.float16, hq8_packed)
     _call("mx_moe_grouped_down_mxfp4", _u8(hq8_packed), _u8(d_qs), _u8(d_e), qs_stride, e_stride, _ptr(down_bias), _ptr(expert_offsets),
           _ptr(out_packed), E, H, E_ffn, TK)
+    return out_packed
+
+
+def moe_grouped_down_mxfp4_f16(h_packed_f16, d_qs, d_e, qs_stride, e_stride, down_bias, expert_offsets, TK, E, H, E_ffn, out_packed=None):
+    """moe_grouped_down_mxfp4 on fp16 packed h rows [TK][E_ffn], quantized while they are staged."""
+    out_packed = _out(out_packed, (TK, H), torch.float16, h_packed_f16)
+    _call("mx_moe_grouped_down_mxfp4_f16", _f16(h_packed_f16), _u8(d_qs), _u8(d_e), qs_stride, e_stride, _ptr(down_bias),
+          _ptr(expert_offsets), _ptr(out_packed), E, H, E_ffn, TK)
     return out_packed
 
 

@@ -95,6 +95,9 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     assert np.array_equal(hq_h, O.quantize_q8_1(h_h))
     out = ops.moe_down_mxfp4(hq, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(ids.ravel()), T, Kt, EF, H, E)
     out_h = host(out).astype(np.float32)
+    # h taken as fp16 and quantized while staged: the same q8 tile, so the same bits out
+    out_f = ops.moe_down_mxfp4_f16(h, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(ids.ravel()), T, Kt, EF, H, E)
+    assert np.array_equal(host(out_f), host(out)), "down on fp16 h != quantize + down"
     hrb = EF // 32 * 40
     inf = np.float16(np.inf)
     lo, hi = [], []
@@ -124,6 +127,8 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     hpq = ops.quantize_q8_1(hp)
     op = ops.moe_grouped_down_mxfp4(hpq, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(off), TK, E, H, EF)
     check_rows(host(op)[t2p], host(out), "grouped down == decode rows")
+    op_f = ops.moe_grouped_down_mxfp4_f16(hp, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(off), TK, E, H, EF)
+    assert np.array_equal(host(op_f), host(op)), "grouped down on fp16 h != quantize + grouped down"
     y2 = torch.zeros((T, H), dtype=torch.float16, device="cuda")
     ops.moe_prefill_reduce(op, dev(t2p.astype(np.uint32)), dev(wp).half(), y2, T, Kt, H)
     check_rows(host(y2), host(y), "grouped layer output == decode layer output")
@@ -154,6 +159,8 @@ def test_moe_q8_0_decode_and_grouped(mx, T, H, EF, E, Kt):
     yp_ref = np.stack([f16(w.ravel()[s]) * O.gemv_q8chain(O.Q8_0, Wd[ids.ravel()[s]], hq_h[s * hrb:(s + 1) * hrb], EF, H)[0]
                        for s in range(T * Kt)])
     check(host(yp).astype(np.float32), yp_ref, "moe_down_q8")
+    yp_f = ops.moe_down_q8_f16(h, dev(dq), dev(dd), dqs_st, dd_st, idsd, w16, T, Kt, EF, H)
+    assert np.array_equal(host(yp_f), host(yp)), "down on fp16 h != quantize + down"
     y = ops.moe_reduce_q8(yp, T, Kt, H)
     check(host(y).astype(np.float32), host(yp).astype(np.float32).reshape(T, Kt, H).sum(axis=1), "moe_reduce_q8")
     # grouped form == decode form, row for row
