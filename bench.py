@@ -215,8 +215,9 @@ def main():
                 if fmt == "q4_K":
                     ws_l = [synth.random_weights(fmt, N, K, seed=77 + i, device=dev) for i in range(12)]
                 else:
-                    ws_l = [ws[(fmt, "gate" if name == "gate_up" else "down")] for ws in sets] + \
-                           ([ws[(fmt, "up")] for ws in sets] if name == "gate_up" else [])
+                    # every matrix of every set, whatever its shape: the buffers are whole blocks and the same size for
+                    # (K, N) and (N, K), and a dozen of them (0.6-0.75 GB) cannot stay in the 256 MB Infinity Cache
+                    ws_l = [ws[(fmt, n)] for ws in sets for n in ("gate", "up", "down")]
                 for T in (1, 2, 4, 8):
                     xs = torch.randn((T, K), device=dev, generator=g).half()
                     xsq = ops.quantize_q8_1(xs)

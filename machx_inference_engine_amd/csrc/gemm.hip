@@ -33,7 +33,6 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kBM = 128;            // tokens per workgroup tile (NI = 4 token tiles of 32); NI = 2 serves dense launches with too few tiles
 constexpr int kBK = 128;            // K chunk
 constexpr int kWaveN = 64;          // weight rows per wave (2 MFMA tiles)
 constexpr int kGemmThreads = 256;
@@ -509,90 +508,80 @@ __device__ __forceinline__ void mma_chunk(const typename QF::Raw (&raw)[2], cons
     }
 }
 
-// NI = 32-token tiles per workgroup tile: 4 (128 tokens, two workgroups per CU), or 2 (64 tokens,
-// three per CU) for dense launches whose 128-token tiles would leave CUs without work.
-template <class QF, int MODE, int NI>
-__global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
-    extern __shared__ __align__(16) uint8_t lds_raw[];
-    constexpr uint32_t BM = 32u * NI, ABUF = BM * kBK * 2u;   // tokens per tile, bytes of one A chunk in LDS
-    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
-    constexpr uint32_t BN = GATE_UP ? 4 * 32 : 4 * kWaveN;   // output columns per workgroup
+// vmcnt(N) with every other counter left alone
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
 
-    // ---- which tile: XCD-aware order (workgroup i runs on XCD i % 8; each XCD walks a
-    // contiguous range of tiles, 4 token tiles x consecutive column tiles at a time)
-    // Expert-grouped tiles are uneven (dead tiles past the real count, 1-4 live token sub-tiles),
-    // so they are dealt round-robin over the XCDs instead of in contiguous ranges.
-    const uint32_t total = g.tiles_m * g.tiles_n;
-    const uint32_t per_xcd = (total + 7) / 8;
-    const uint32_t linear = (MODE == GEMM_DENSE) ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
-    if ((MODE == GEMM_DENSE && (blockIdx.x >> 3) >= per_xcd) || linear >= total) return;
-    uint32_t tm, tn;
-    {
-        constexpr uint32_t GM = 4;
-        const uint32_t grp = linear / (GM * g.tiles_n), in = linear - grp * (GM * g.tiles_n);
-        const uint32_t rows_here = (g.tiles_m - grp * GM < GM) ? g.tiles_m - grp * GM : GM;
-        tn = in / rows_here;
-        tm = grp * GM + in - tn * rows_here;
-    }
-    uint32_t e = 0, row_lo = 0, row_hi = g.M;
-    if (MODE != GEMM_DENSE) {
-        // tm-th 128-row tile over all experts: wave 0 scans the per-expert tile counts, 64 experts at a time
-        __shared__ uint32_t s_tile[3];
-        const uint32_t ln = threadIdx.x & 63u;
-        if (threadIdx.x < 64) {
-            uint32_t base = 0;
-            bool found = false;
-            for (uint32_t e0 = 0; e0 < g.E && !found; e0 += 64) {
-                const uint32_t ee = e0 + ln;
-                const uint32_t lo = ee < g.E ? g.expert_offsets[ee] : 0u, hi = ee < g.E ? g.expert_offsets[ee + 1] : 0u;
-                const uint32_t nt = (hi - lo + BM - 1) / BM;
-                uint32_t incl = nt;
+template <class QF, int NA>
+struct TileCtx {
+    typename QF::W w0, w1;
+    uint32_t wrow0, wrow1, h;
+    const uint8_t* a_glb;
+    uint32_t a_dst;
+    const uint8_t* lds_raw;
+    uint32_t frag0, n_chunks, mi;
+};
+
+// Chunk c out of register set P; meanwhile (`more`) the A rows of chunk c+1 and the weights of chunk c+DEPTH are requested.
+template <class QF, bool PARTIAL, int NA, int DEPTH, int P>
+__device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint32_t (&a_off)[2 * NA], typename QF::Raw (&raw)[DEPTH + 1][2],
+                                           float16_t (&acc)[NA][2], uint32_t c, bool more) {
+    constexpr int NSET = DEPTH + 1, PN = (P + DEPTH) % NSET, NL = 2 * NA;
+    constexpr uint32_t ABUF = 32u * NA * kBK * 2u;
+    constexpr int W_LOADS_MIN = 2 * (int)((sizeof(typename QF::Raw) + 15) / 16);
+    if (more) {
+        const uint8_t* a_next = t.a_glb + (size_t)(c + 1) * (kBK * 2u);
+        const uint32_t dst = t.a_dst + ((c + 1) & 1u) * ABUF;
 #pragma unroll
-                for (int d = 1; d < 64; d <<= 1) {
-                    const uint32_t v = (uint32_t)__shfl_up((int)incl, d);
-                    if (ln >= (uint32_t)d) incl += v;
-                }
-                const uint32_t excl = base + incl - nt;
-                const bool hit = tm >= excl && tm < excl + nt;
-                if (hit) {
-                    s_tile[0] = ee;
-                    s_tile[1] = lo + (tm - excl) * BM;
-                    s_tile[2] = hi;
-                }
-                found = __ballot(hit) != 0ull;
-                base += (uint32_t)__shfl((int)incl, 63);
-            }
-            if (!found && ln == 0) s_tile[0] = 0xFFFFFFFFu;
-        }
-        __syncthreads();
-        e = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[0]);
-        if (e == 0xFFFFFFFFu) return;
-        row_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[1]);
-        row_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[2]);
-    } else {
-        row_lo = tm * BM;
+        for (int j = 0; j < NL; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
+        const uint32_t cn = (c + DEPTH < t.n_chunks) ? c + DEPTH : t.n_chunks - 1;   // past the end: the last chunk again, unused
+        raw[PN][0] = QF::load(t.w0, t.wrow0, cn, t.h);
+        raw[PN][1] = QF::load(t.w1, t.wrow1, cn, t.h);
+        __builtin_amdgcn_sched_barrier(0);   // the scheduler must not sink these loads towards their uses
     }
-    const typename QF::W w0 = QF::expert(bank0, e), w1 = QF::expert(GATE_UP ? bank1 : bank0, e);
+    typename QF::Dec dec[2];
+    dec[0] = QF::prepare(raw[P][0], c, t.h);
+    dec[1] = QF::prepare(raw[P][1], c, t.h);
+    mma_chunk<QF, PARTIAL, NA>(raw[P], dec, t.lds_raw, (c & 1u) * ABUF + t.frag0, acc, t.mi);
+    if (more) {
+        wait_vmcnt<(DEPTH > 1 ? W_LOADS_MIN : 0)>();   // A rows of chunk c+1 are in LDS (DEPTH > 1: the newest weight loads stay in flight)
+        __syncthreads();
+    }
+}
 
+// One output tile: accumulators, A staging, the K loop and the epilogue.  NA = 32-token tiles this instance
+// keeps accumulators for and stages (the tile's live rows fit in 32 NA rows); PIPE = the hand-pipelined chunk
+// (needs NA = 4 and a full tile); DEPTH = how many K chunks ahead the weight words are requested.
+//
+// Software pipeline over K chunks: at the top of chunk c the A rows of chunk c+1 start their way into the
+// other LDS buffer, then the weight words of chunk c+DEPTH into registers.  Memory returns in order, the A
+// rows come from L2 while the weights come from HBM.  With DEPTH = 1 both have one chunk of MFMAs to arrive,
+// which covers the latency when a chunk carries 64 MFMAs per wave; a tile with one or two live token tiles
+// finishes a chunk in a fraction of the memory latency, so it keeps two chunks of weights in flight.  At the
+// end of chunk c the A rows of chunk c+1 must be in LDS: they are older than the weight loads issued after
+// them in the same iteration, of which there are at least 2 ceil(sizeof(Raw) / 16) (a load instruction
+// brings at most 16 bytes per lane), so waiting until at most that many loads are outstanding is enough
+// whatever the compiler made of QF::load.
+template <class QF, int MODE, bool PIPE, int NA, int DEPTH>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::W& w0, const typename QF::W& w1, const uint32_t (&wrow)[2],
+                                          uint32_t row_lo, uint32_t row_hi, uint32_t n_base, uint8_t* lds_raw) {
+    static_assert(DEPTH == 1 || DEPTH == 2, "prefetch depth");
+    static_assert(!PIPE || NA == 4, "the pipelined chunk is written for four token tiles");
+    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
+    constexpr bool PARTIAL = MODE != GEMM_DENSE && !PIPE;
+    constexpr uint32_t BM = 32u * NA;
+    constexpr int NL = 2 * NA;   // 1 KB loads per wave per chunk
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 31u, h = lane >> 5;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t n_base = tn * BN + wave * (GATE_UP ? 32 : kWaveN);
-    // weight rows of the two MFMA column tiles of this wave (gate/up: same row in two matrices)
-    uint32_t wrow[2];
-    wrow[0] = n_base + r;
-    wrow[1] = GATE_UP ? n_base + r : n_base + 32 + r;
-    if (wrow[0] >= g.N) wrow[0] = g.N - 1;
-    if (wrow[1] >= g.N) wrow[1] = g.N - 1;
-
     const uint32_t n_chunks = g.K / kBK;
-    constexpr bool PARTIAL = MODE != GEMM_DENSE;
     const uint32_t live_rows = (row_hi - row_lo) >= BM ? BM : row_hi - row_lo;
     const uint32_t mi = (live_rows + 31u) / 32u;
 
-    // A staging: wave w brings rows 32w .. 32w+31 of the chunk, 4 rows (1 KB) per load; lane L
-    // fills LDS slot (row 4j + L/16, column L%16) of that 1 KB with global column
-    // (L%16) ^ (row & 15).  Rows past the end of the tile re-read its last row (never used).
-    constexpr int NL = 2 * NI;   // 1 KB loads per wave per chunk
+    // A staging: wave w brings rows (BM/4) w .. of the chunk, 4 rows (1 KB) per load; lane L fills LDS slot
+    // (row 4j + L/16, column L%16) of that 1 KB with global column (L%16) ^ (row & 15).  Rows past the end of
+    // the tile re-read its last row (never used).
     uint32_t a_off[NL];
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
@@ -606,55 +595,58 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     // step-0 fragment address of this lane inside an A buffer
     const uint32_t frag0 = r * 256u + (((QF::H_COL * h) ^ (r & 15u)) << 4);
 
-    float16_t acc[NI][2];
+    float16_t acc[NA][2];
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+    for (int i = 0; i < NA; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // Software pipeline over K chunks: at the top of chunk c the A rows of chunk c+1 start
-    // their way into the other LDS buffer and the weight words of chunk c+1 into registers;
-    // both have the whole chunk (64 MFMAs per wave) to arrive.  The A rows are requested
-    // first: memory returns in order, and they come from L2 while the weights come from HBM.
-    typename QF::Raw raw[2];
+    // Weight words of DEPTH + 1 chunks live in registers: chunk c sits in set c % (DEPTH + 1).  The loop is unrolled
+    // over the sets so that no set is ever copied into another (a register copy of loaded data waits for the load).
+    constexpr int NSET = DEPTH + 1;
+    typename QF::Raw raw[NSET][2];
 #pragma unroll
     for (int j = 0; j < NL; ++j) load_to_lds16(a_glb, a_off[j], a_dst + 1024u * j);
-    raw[0] = QF::load(w0, wrow[0], 0, h);
-    raw[1] = QF::load(w1, wrow[1], 0, h);
-    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+    raw[0][0] = QF::load(w0, wrow[0], 0, h);
+    raw[0][1] = QF::load(w1, wrow[1], 0, h);
+    wait_vmcnt<0>();
     __syncthreads();
-
-    for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
-        const uint8_t* a_next = a_glb + (size_t)(c + 1) * (kBK * 2u);
-        const uint32_t dst = a_dst + ((c + 1) & 1u) * ABUF;
 #pragma unroll
-        for (int j = 0; j < NL; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
-        typename QF::Raw nxt[2];
-        nxt[0] = QF::load(w0, wrow[0], c + 1, h);
-        nxt[1] = QF::load(w1, wrow[1], c + 1, h);
-        __builtin_amdgcn_sched_barrier(0);   // the scheduler must not sink these loads towards their uses
-        typename QF::Dec dec[2];
-        dec[0] = QF::prepare(raw[0], c, h);
-        dec[1] = QF::prepare(raw[1], c, h);
-        mma_chunk<QF, PARTIAL, NI>(raw, dec, lds_raw, (c & 1u) * ABUF + frag0, acc, mi);
-        raw[0] = nxt[0];
-        raw[1] = nxt[1];
-        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): A rows of chunk c+1 are in LDS
-        __syncthreads();
-    }
-    {
-        const uint32_t c = n_chunks - 1;
-        typename QF::Dec dec[2];
-        dec[0] = QF::prepare(raw[0], c, h);
-        dec[1] = QF::prepare(raw[1], c, h);
-        mma_chunk<QF, PARTIAL, NI>(raw, dec, lds_raw, (c & 1u) * ABUF + frag0, acc, mi);
+    for (int d = 1; d < DEPTH; ++d) {
+        const uint32_t cd = (uint32_t)d < n_chunks ? (uint32_t)d : n_chunks - 1;
+        raw[d][0] = QF::load(w0, wrow[0], cd, h);
+        raw[d][1] = QF::load(w1, wrow[1], cd, h);
     }
 
+    const TileCtx<QF, NA> ctx{w0, w1, wrow[0], wrow[1], h, a_glb, a_dst, lds_raw, frag0, n_chunks, mi};
+#define CHUNK(P, c, more) gemm_chunk<QF, PARTIAL, NA, DEPTH, P>(ctx, a_off, raw, acc, c, more)
+    if constexpr (DEPTH == 1) {
+        // two sets, and the set just loaded is copied into set 0 at the end of a chunk, where it has to have arrived anyway
+        for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
+            CHUNK(0, c, true);
+            raw[0][0] = raw[1][0];
+            raw[0][1] = raw[1][1];
+        }
+        CHUNK(0, n_chunks - 1, false);
+    } else {
+        uint32_t c = 0;
+        for (; c + 3 < n_chunks; c += 3) {
+            CHUNK(0, c, true);
+            CHUNK(1, c + 1, true);
+            CHUNK(2, c + 2, true);
+        }
+        const uint32_t left = n_chunks - c;   // 1..3
+        CHUNK(0, c, left > 1);
+        if (left > 1) CHUNK(1, c + 1, left > 2);
+        if (left > 2) CHUNK(2, c + 2, false);
+    }
+
+#undef CHUNK
     // ---- epilogue.  MFMA C layout: lane holds column n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4.
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+    for (int i = 0; i < NA; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t row = row_lo + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
@@ -678,12 +670,104 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
         }
 }
 
+// NI = 32-token tiles per workgroup tile: 4 (128 tokens, two workgroups per CU), or 2 (64 tokens,
+// three per CU) for dense launches whose 128-token tiles would leave CUs without work.
+template <class QF, int MODE, int NI>
+__global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
+    extern __shared__ __align__(16) uint8_t lds_raw[];
+    constexpr uint32_t BM = 32u * NI;   // tokens per tile
+    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
+    constexpr uint32_t BN = GATE_UP ? 4 * 32 : 4 * kWaveN;   // output columns per workgroup
+
+    // ---- which tile: XCD-aware order (workgroup i runs on XCD i % 8; each XCD walks a
+    // contiguous range of tiles, 4 token tiles x consecutive column tiles at a time)
+    // Expert-grouped tiles are uneven (dead tiles past the real count, 1-4 live token sub-tiles),
+    // so they are dealt round-robin over the XCDs instead of in contiguous ranges.
+    const uint32_t total = g.tiles_m * g.tiles_n;
+    const uint32_t per_xcd = (total + 7) / 8;
+    const uint32_t linear = (MODE == GEMM_DENSE) ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    if ((MODE == GEMM_DENSE && (blockIdx.x >> 3) >= per_xcd) || linear >= total) return;
+    uint32_t tm, tn;
+    {
+        constexpr uint32_t GM = 4;
+        const uint32_t grp = linear / (GM * g.tiles_n), in = linear - grp * (GM * g.tiles_n);
+        const uint32_t rows_here = (g.tiles_m - grp * GM < GM) ? g.tiles_m - grp * GM : GM;
+        tn = in / rows_here;
+        tm = grp * GM + in - tn * rows_here;
+    }
+    uint32_t e = 0, row_lo = 0, row_hi = g.M;
+    if (MODE != GEMM_DENSE) {
+        // Tile order over all experts: every full BM-row tile first (expert by expert), then the experts' partial last
+        // tiles.  Full tiles cost the most, so the workgroups dispatched last are the cheap ones and the launch ends
+        // without a few full tiles running alone.  Wave 0 scans the per-expert counts, 64 experts at a time; pass 0
+        // walks the full tiles, pass 1 the partial ones.
+        __shared__ uint32_t s_tile[3];
+        const uint32_t ln = threadIdx.x & 63u;
+        if (threadIdx.x < 64) {
+            uint32_t base = 0;
+            bool found = false;
+            for (uint32_t pass = 0; pass < 2 && !found; ++pass)
+                for (uint32_t e0 = 0; e0 < g.E && !found; e0 += 64) {
+                    const uint32_t ee = e0 + ln;
+                    const uint32_t lo = ee < g.E ? g.expert_offsets[ee] : 0u, hi = ee < g.E ? g.expert_offsets[ee + 1] : 0u;
+                    const uint32_t full = (hi - lo) / BM;
+                    const uint32_t nt = pass == 0 ? full : ((hi - lo) % BM ? 1u : 0u);
+                    uint32_t incl = nt;
+#pragma unroll
+                    for (int d = 1; d < 64; d <<= 1) {
+                        const uint32_t v = (uint32_t)__shfl_up((int)incl, d);
+                        if (ln >= (uint32_t)d) incl += v;
+                    }
+                    const uint32_t excl = base + incl - nt;
+                    const bool hit = tm >= excl && tm < excl + nt;
+                    if (hit) {
+                        s_tile[0] = ee;
+                        s_tile[1] = lo + (pass == 0 ? tm - excl : full) * BM;
+                        s_tile[2] = hi;
+                    }
+                    found = __ballot(hit) != 0ull;
+                    base += (uint32_t)__shfl((int)incl, 63);
+                }
+            if (!found && ln == 0) s_tile[0] = 0xFFFFFFFFu;
+        }
+        __syncthreads();
+        e = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[0]);
+        if (e == 0xFFFFFFFFu) return;
+        row_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[1]);
+        row_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[2]);
+    } else {
+        row_lo = tm * BM;
+    }
+    const typename QF::W w0 = QF::expert(bank0, e), w1 = QF::expert(GATE_UP ? bank1 : bank0, e);
+
+    const uint32_t tid = threadIdx.x, r = tid & 31u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t n_base = tn * BN + wave * (GATE_UP ? 32 : kWaveN);
+    // weight rows of the two MFMA column tiles of this wave (gate/up: same row in two matrices)
+    uint32_t wrow[2];
+    wrow[0] = n_base + r;
+    wrow[1] = GATE_UP ? n_base + r : n_base + 32 + r;
+    if (wrow[0] >= g.N) wrow[0] = g.N - 1;
+    if (wrow[1] >= g.N) wrow[1] = g.N - 1;
+
+    if constexpr (MODE == GEMM_DENSE) {
+        gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
+    } else {
+        // expert-grouped tiles: a full one takes the same pipelined chunk as the dense GEMM; one with at most 64
+        // live rows keeps half the accumulators and spends the registers on a second chunk of weights in flight
+        const uint32_t live = row_hi - row_lo;
+        if (live >= BM) gemm_tile<QF, MODE, true, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
+        else if (live <= 64u) gemm_tile<QF, MODE, false, 2, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
+        else gemm_tile<QF, MODE, false, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
+    }
+}
+
 // ---------------------------------------------------------------- host side
 template <class QF, int MODE, int NI>
 static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
     constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU) ? 128 : 256, BM = 32u * NI, lds = 2u * BM * kBK * 2u;
     g.tiles_n = (g.N + BN - 1) / BN;
-    g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + BM - 1) / BM : (rows_bound + BM - 1) / BM + g.E;
+    g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + BM - 1) / BM : rows_bound / BM + g.E;   // grouped: an upper bound, workgroups past the real count leave at once
     const uint64_t total = (uint64_t)g.tiles_m * g.tiles_n;
     const uint64_t grid = (total + 7) / 8 * 8;
     if (grid > 0x7FFFFFFFull) return MX_ERR_SHAPE;

@@ -4,6 +4,8 @@
 #include "mxq_gemv_core.h"
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "mxq_host.h"
 
 namespace mxq {
@@ -362,7 +364,9 @@ static uint32_t pick_group(uint32_t units) {
 template <class F, int T, int G, class OutT>
 static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8,
                         uint32_t K, uint32_t N, uint32_t T_real, bool split) {
-    constexpr int R = GemvShape<T, F::SUM_GRAN>::R, U = GemvShape<T, F::SUM_GRAN>::U;
+    // GGUF Q8_0 blocks are 17 dword loads per unit: one unit in flight (measured at T = 1 against two: K = 4096,
+    // N = 14336 18.1 -> 15.8 us; K = 14336, N = 4096 18.1 -> 16.6 us)
+    constexpr int R = GemvShape<T, F::SUM_GRAN>::R, U = std::is_same<F, FmtQ8Aos>::value ? 1 : GemvShape<T, F::SUM_GRAN>::U;
     constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
     const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);   // LDS bytes per 32 activation elements
     const uint32_t KT_max = (kLdsBudget / (per_elem_x32 * T)) * 32 / 256 * 256;
