@@ -256,7 +256,18 @@ def main():
                 yg = torch.empty((T, N), dtype=torch.float16, device=dev)
                 us = kernel_avg_us(lambda i: ops.gemm_q4_K(a16, wq, T, K, N, yg), 4)
                 tf = 2.0 * T * N * K / us / 1e6
-                detail["config3_gemm_q4_K_T%d_K%d_N%d" % (T, K, N)] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
+                ent = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
+                if T >= 2048:
+                    # the same product the reference's way on this box: dequantize W to an fp16 [K, N] matrix, then the
+                    # vendor library's fp16 GEMM (rocBLAS here, oneDNN there); and that GEMM alone
+                    bt = ops.dequant_to_Bt("q4_K", wq, K, N)
+                    us_g = kernel_avg_us(lambda i: ops.gemm_fp16(a16, bt, T, N, K, torch.float16, yg), 4)
+                    us_2 = kernel_avg_us(lambda i: (ops.dequant_to_Bt("q4_K", wq, K, N, bt), ops.gemm_fp16(a16, bt, T, N, K, torch.float16, yg)), 4)
+                    ent["vendor_fp16_gemm_us"] = round(us_g, 1)
+                    ent["vendor_fp16_gemm_TFLOPs"] = round(2.0 * T * N * K / us_g / 1e6, 1)
+                    ent["dequant_plus_vendor_gemm_us"] = round(us_2, 1)
+                    del bt
+                detail["config3_gemm_q4_K_T%d_K%d_N%d" % (T, K, N)] = ent
                 del a16, yg
             del wq
         # BASELINE config 4: MXFP4 MoE decode at gpt-oss-20b shape (E=32, top-4, H=EF=2880), T=1 and T=32
