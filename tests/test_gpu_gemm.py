@@ -157,6 +157,50 @@ def test_moe_grouped_gemm_q8(mx, T, E, Kt, H, EF):
     assert np.abs(a - b).max() / np.sqrt(np.mean(b * b)) < 0.2   # q8 activation noise through silu(g)*u
 
 
+@pytest.mark.parametrize("H,EF", [(640, 256), (384, 128)])
+def test_moe_grouped_gemm_q8_tile_boundaries(mx, H, EF):
+    """Expert row counts on both sides of every tile class of the grouped kernel (empty, 1, 31..33, 63..65,
+    127..129, 192/193, 256) and K depths of 1, 2, 3 and 5 chunks (the small-tile path walks K three chunks at a time)."""
+    ops = mx.ops
+    counts = np.array([0, 1, 63, 64, 65, 127, 128, 129, 192, 193, 256, 0, 31, 33, 32], np.int64)
+    E, Kt = len(counts), 1
+    ids = np.repeat(np.arange(E), counts).astype(np.int32)
+    ids = ids[np.random.default_rng(11).permutation(ids.size)].reshape(-1, 1)
+    T = ids.shape[0]
+    w = O.uniform(12, (T, 1), 0.5, 1.5).astype(np.float32)
+    mk = lambda seed, N, K: np.stack([O.quantize(O.Q8_0, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
+    Wg, Wu, Wd = mk(3100, EF, H), mk(4100, EF, H), mk(5100, H, EF)
+    gq, gd = O.repack_q8_0_to_soa(Wg)
+    uq, ud = O.repack_q8_0_to_soa(Wu)
+    dq, dd = O.repack_q8_0_to_soa(Wd)
+    x = f16(O.normal(6100, (T, H)))
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    assert np.array_equal(np.diff(off.astype(np.int64)), counts)
+    xp = ops.moe_gather_rows(dev(x).half(), dev(si), T, H)
+    hp = ops.moe_gemm_gate_up_silu_q8(xp, dev(gq), dev(gd), dev(uq), dev(ud), EF * H, EF * H // 32, dev(off), T, E, H, EF)
+    hp_h = host(hp).astype(np.float32)
+    xs = x[si]
+    h_ref = np.zeros((T, EF), np.float32)
+    o_ref = np.zeros((T, H), np.float64)
+    for e in range(E):
+        if counts[e]:
+            rows = slice(off[e], off[e + 1])
+            g = O.gemv_f64(O.Q8_0, Wg[e], xs[rows], H, EF, round_w_fp16=True)
+            u = O.gemv_f64(O.Q8_0, Wu[e], xs[rows], H, EF, round_w_fp16=True)
+            h_ref[rows] = O.swiglu_np(g.astype(np.float32), u.astype(np.float32))
+            o_ref[rows] = O.gemv_f64(O.Q8_0, Wd[e], hp_h[rows], EF, H, round_w_fp16=True) * f16(wp[rows])[:, None]
+    check(hp_h, h_ref, "grouped gate_up silu, boundary row counts")
+    op = ops.moe_gemm_down_q8(hp, dev(dq), dev(dd), H * EF, H * EF // 32, dev(off), dev(wp).half(), T, E, H, EF)
+    check(host(op).astype(np.float32), o_ref, "grouped down, boundary row counts")
+    # per expert as well: a wrong row range shows up as one expert's rows being off, which a global norm can hide
+    op_h = host(op).astype(np.float64)
+    for e in range(E):
+        if counts[e]:
+            rows = slice(off[e], off[e + 1])
+            err = np.abs(op_h[rows] - o_ref[rows]).max() / max(np.sqrt(np.mean(o_ref[rows] ** 2)), 1e-30)
+            assert err < 5e-2, (e, counts[e], err)
+
+
 @pytest.mark.parametrize("T,E,Kt,H,EF", [(64, 8, 2, 256, 256), (300, 16, 4, 512, 256)])
 def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
     """Q4_K gate/up + Q4_K or Q6_K down expert banks (AoS, expert-major) through the grouped GEMM
