@@ -188,12 +188,19 @@ def main():
         dom_us = kernel_avg_us(lambda i: gate_up("q8_0", sets[i % len(sets)]), 4 * len(sets))
         dom_bytes = 2 * gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1) - (H // 32) * 40
         dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 124876800 + 233267
+    # yardstick: a pure read of the same number of bytes with the same launch geometry (rotating buffers, no arithmetic)
+    n_read = (dom_bytes + 15) // 16 * 16
+    rd = [torch.empty(n_read, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(8)]
+    read_us = kernel_avg_us(lambda i: ops.probe_stream_read(rd[i % len(rd)]), 4 * len(rd))
+    del rd
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt)
                 "traffic": dom_traffic,
-                "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 3)}
+                "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 3),
+                # not part of the fraction above: what a read-only kernel reaches on the same bytes on this device
+                "stream_read_same_bytes": {"avg_launch_us": round(read_us, 3), "GBps": round(n_read / read_us / 1e3, 1)}}
 
     out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),

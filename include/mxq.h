@@ -47,6 +47,11 @@ const char* mx_status_string(int status);
 int mx_last_hip_error(void);  /* hipError_t of the last MX_ERR_LAUNCH on this thread */
 int mx_version(void);
 
+/* Measurement aid, no counterpart in the reference: reads n_bytes (a multiple of 16, 16-byte aligned) once with the
+ * launch geometry of the decode GEMV and no arithmetic, so that a GEMV launch can be priced against a pure read of
+ * the same bytes on the same device.  `sink` may be NULL (a word that is practically never written).  */
+int mx_probe_stream_read(mx_stream_t s, const void* src, uint64_t n_bytes, uint32_t* sink);
+
 /* ---------------------------------------------------------------- activation quantizers
  * quantize_q8_1   include/ie/ops.hpp:301-304, src/ops/gemv_q8dot.cpp:94-124
  * quantize_q8_1s  include/ie/ops.hpp:307-310, src/ops/gemv_q8dot.cpp:57-91

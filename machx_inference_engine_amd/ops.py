@@ -77,6 +77,12 @@ def quantize_q8_1s(x, out_q8=None):
     return out_q8
 
 
+def probe_stream_read(buf, n_bytes=None):
+    """Pure read of `buf` (or its first n_bytes) with the decode GEMV's launch geometry: the bandwidth yardstick."""
+    n = buf.numel() * buf.element_size() if n_bytes is None else n_bytes
+    _call("mx_probe_stream_read", _ptr(buf), n, None)
+
+
 # ---------------------------------------------------------------- dequant
 def dequant(fmt, packed, n_elements, out=None, dtype=torch.float16):
     out = _out(out, (n_elements,), dtype, packed)
