@@ -107,6 +107,20 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
             for (int r = 0; r < R; ++r) cu[r] = F::cursor(seg.w, (row0 + r < N) ? row0 + r : N - 1, k0 / 64 + gl);
             const uint32_t n_units = (kt + 63) / 64;
             const bool half_tail = (kt & 63u) != 0;
+            if (T == 1 && n_tiles == 1 && !staged && (half_tail ? n_units - 1 : n_units) / G >= (uint32_t)U) {
+                // first row group of a single-tile launch: the first round of weights is requested before the
+                // activation row is staged (a long row stages for a microsecond or two before its first load otherwise)
+                typename F::Raw pre[U][R];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int r = 0; r < R; ++r) pre[u][r] = load_unit<F, G>(cu[r], u, false);
+                act = stage_act<F::SUM_GRAN, T>(lds, xrow, k0, kt, KT, q8_split != 0);
+                __syncthreads();
+                staged = true;
+                gemv_rows<F, T, R, G, U>(cu, n_units, half_tail, gl, act, acc, pre);
+                continue;
+            }
             if (n_tiles > 1 || !staged) {
                 __syncthreads();
                 act = stage_act<F::SUM_GRAN, T>(lds, xrow, k0, kt, KT, q8_split != 0);

@@ -213,12 +213,19 @@ __device__ __forceinline__ void gemv_step(const typename F::Raw (&raw)[R], const
 // all U*R loads issued before the first use; the ragged rest is predicated.
 // cu[r] must point at unit (tile_first_unit + gl) of row r.  `n_units` counts
 // 64-element units including a trailing half unit (`half_tail`: K % 64 == 32).
+// `pre` (optional): the U*R units of the first full iteration, already requested by the caller (before it staged
+// the activations, say); only used when there is a full iteration (n_whole / G >= U).
 template <class F, int T, int R, int G, int U>
 __device__ __forceinline__ void gemv_rows(const typename F::Cursor (&cu)[R], uint32_t n_units, bool half_tail, uint32_t gl,
-                                          const ActTile& act, float (&acc)[R][T]) {
+                                          const ActTile& act, float (&acc)[R][T], const typename F::Raw (*pre)[R] = nullptr) {
     const uint32_t n_whole = half_tail ? n_units - 1 : n_units;
     const uint32_t full = n_whole / G;
     uint32_t it = 0;
+    if (pre && U <= full) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) gemv_step<F, T, R>(pre[u], cu, gl + u * G, act, acc);
+        it = U;
+    }
     for (; it + U <= full; it += U) {
         typename F::Raw raw[U][R];
 #pragma unroll

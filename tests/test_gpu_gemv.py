@@ -288,3 +288,15 @@ def test_gemv_q6_K_q8_reference_ktiled_shapes(mx, K, N, seed):
     W = weights(O.Q6_K, seed, N, K)
     xq = O.quantize_q8_1(acts(seed + 16, 1, K))
     check(run_q8(mx, O.Q6_K, W, xq, K, N, 1), O.gemv_q8chain(O.Q6_K, W, xq, K, N)[0], "gemv_q6_K_q8 K=%d N=%d" % (K, N))
+
+
+def test_probe_stream_read(mx):
+    """The bandwidth yardstick: launches on any 16-byte multiple, rejects what it cannot read whole."""
+    buf = torch.empty(1 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+    for n in (16, 4096 + 16, 1 << 20):
+        mx.ops.probe_stream_read(buf, n)
+    torch.cuda.synchronize()
+    with pytest.raises(mx.ops.MxError):
+        mx.ops.probe_stream_read(buf, 24)          # not a multiple of 16
+    with pytest.raises(mx.ops.MxError):
+        mx.ops.probe_stream_read(buf[8:], 16)      # misaligned
