@@ -187,7 +187,7 @@ def main():
         # the fused gate + up launch: two 4096 -> 14336 matrices, one activation row, two output rows
         dom_us = kernel_avg_us(lambda i: gate_up("q8_0", sets[i % len(sets)]), 4 * len(sets))
         dom_bytes = 2 * gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1) - (H // 32) * 40
-        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 124876800 + 233267
+        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 124885402 + 233882
     # yardstick: a pure read of the same number of bytes with the same launch geometry (rotating buffers, no arithmetic)
     n_read = (dom_bytes + 15) // 16 * 16
     rd = [torch.empty(n_read, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(8)]

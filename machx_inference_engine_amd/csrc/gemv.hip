@@ -19,6 +19,12 @@ struct GemvSeg {
     const float* bias;
 };
 
+// Formats whose T = 1 kernels hold a second set of units in registers (requested ahead of the row group being
+// summed, or ahead of the activation staging): the ones where that was measured to pay and that stay within the
+// 128 VGPRs the four-workgroups-per-CU launch wants.  Q6_K loses on both counts (82 -> 129 VGPRs).
+template <class F>
+constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value;
+
 // Persistent workgroups: each stages the activation tile(s) and then streams
 // its share of row groups.  With a single K-tile (every decode shape at T <= 2)
 // the activation is staged once per workgroup.
@@ -37,12 +43,11 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
     const uint32_t n_tiles = (K + KT - 1) / KT;
     ActTile act;
     bool staged = false;
-    if (F::SUM_GRAN != 16 && K == 64u * G && n_tiles == 1) {
+    if (kPrefetchAcrossRows<F> && K == 64u * G && n_tiles == 1) {
         // One unit per lane and row (K = 4096 with 64 lanes per row, ...): a row is a single round of loads, so the
         // loads of the next row group are issued before the dot products and the lane-group sum of this one;
         // otherwise every wave would sit with nothing in flight from its last load's arrival to its store.
-        // Measured on 4096 -> 14336: Q8_0 planes 13.2 -> 12.4 us, Q4_K 8.6 -> 8.4 us.  Q6_K stays on the plain loop:
-        // its 48 MB launch gains 2 % but a 510 MB one loses 3 %.
+        // Measured on 4096 -> 14336: Q8_0 planes 13.2 -> 12.4 us, Q4_K 8.6 -> 8.4 us.
         // The first row group's weights are requested before the activation row is staged: they do not depend on it.
         typename F::Cursor cn[R];
         typename F::Raw nxt[R];
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
             for (int r = 0; r < R; ++r) cu[r] = F::cursor(seg.w, (row0 + r < N) ? row0 + r : N - 1, k0 / 64 + gl);
             const uint32_t n_units = (kt + 63) / 64;
             const bool half_tail = (kt & 63u) != 0;
-            if (T == 1 && n_tiles == 1 && !staged && (half_tail ? n_units - 1 : n_units) / G >= (uint32_t)U) {
+            if (T == 1 && kPrefetchAcrossRows<F> && n_tiles == 1 && !staged && (half_tail ? n_units - 1 : n_units) / G >= (uint32_t)U) {
                 // first row group of a single-tile launch: the first round of weights is requested before the
                 // activation row is staged (a long row stages for a microsecond or two before its first load otherwise)
                 typename F::Raw pre[U][R];
