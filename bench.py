@@ -234,6 +234,27 @@ def main():
                     detail["%s_%s_T%d" % (fmt, name, T)] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1),
                                                             "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
                 del ws_l
+        # one decode FFN (fp16 x in, fp16 y out) as the reference's launch chain and as the two fused launches
+        xf = torch.randn(H, device=dev, generator=g).half()
+        xq_b = torch.empty(H // 32 * 40, dtype=torch.uint8, device=dev)
+        hq_b = torch.empty(FF // 32 * 40, dtype=torch.uint8, device=dev)
+        g_b, u_b, h_b = (torch.empty(FF, dtype=torch.float16, device=dev) for _ in range(3))
+        y_b = torch.empty(H, dtype=torch.float16, device=dev)
+        for fmt, key in (("q8_0_soa", "q8_0_soa"), ("q6_K", "q6_K")):
+            def chain(i):
+                ws = sets[i % len(sets)]
+                ops.quantize_q8_1(xf, xq_b)
+                ops.gemv_q8_x2(fmt, xq_b, ws[(key, "gate")], ws[(key, "up")], H, FF, g_b, u_b)
+                ops.swiglu_q8(g_b, u_b, out=(h_b, hq_b))
+                gemv(key.replace("_soa", ""), hq_b, ws, "down", FF, H, y_b)
+
+            def fused(i):
+                ws = sets[i % len(sets)]
+                ops.gemv_x2_silu(fmt, xf, ws[(key, "gate")], ws[(key, "up")], H, FF, h_b)
+                ops.gemv_f16q8(fmt, h_b, ws[(key, "down")], FF, H, y_b)
+
+            us_c, us_f = kernel_avg_us(chain, 2 * len(sets)), kernel_avg_us(fused, 2 * len(sets))
+            detail["ffn_decode_%s_T1" % fmt] = {"chain_4_launches_us": round(us_c, 2), "fused_2_launches_us": round(us_f, 2)}
         # BASELINE config 1: Q4_K 4096x4096, fp32 activations, fp32 out (9.4 MB: cache resident unless rotated)
         w1 = [synth.random_weights("q4_K", 4096, 4096, seed=500 + i, device=dev) for i in range(40)]
         a32 = torch.randn(4096, device=dev, generator=g)

@@ -171,6 +171,28 @@ int mx_gemv_q6_K_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const v
                        uint32_t K, uint32_t N);
 int mx_gemv_q8_0_q8_x2(mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b,
                        uint32_t K, uint32_t N);
+
+/* Decode FFN forms (T = 1), no counterpart in the reference, which launches gemv, gemv, swiglu and quantize_q8_1
+ * separately (src/model/dense_dispatch.hpp:562-754, src/ops/elementwise.cpp:449-466).
+ * *_x2_silu: h[n] = half(silu(half(g[n])) * half(u[n])) with g, u the two GEMVs on the same activation row, the
+ *   bits of mx_gemv_*_q8_x2 followed by the fp16 output of mx_swiglu_q8.  x is the q8 row (block_q8_1x,
+ *   x_is_f16 = 0) or the fp16 row (x_is_f16 = 1: quantized while it is staged, the values of mx_quantize_q8_1,
+ *   16-byte aligned).
+ * *_f16q8: y = W . q8(x) on an fp16 activation row quantized while it is staged: the bits of mx_quantize_q8_1
+ *   followed by mx_gemv_*_q8.  K up to one LDS tile (32,768 elements for Q6_K, more for the other formats).  */
+int mx_gemv_q8_0_soa_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const int8_t* g_qs, const uint16_t* g_d,
+                             const int8_t* u_qs, const uint16_t* u_d, uint16_t* h, uint32_t K, uint32_t N);
+int mx_gemv_q4_K_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h,
+                         uint32_t K, uint32_t N);
+int mx_gemv_q6_K_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h,
+                         uint32_t K, uint32_t N);
+int mx_gemv_q8_0_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h,
+                         uint32_t K, uint32_t N);
+int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y,
+                           uint32_t K, uint32_t N);
+int mx_gemv_q4_K_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q6_K_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N);
+int mx_gemv_q8_0_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N);
 /* Sibling formats on the same kernels.
  * Q4_0:
  *   gemv_q4_0                 include/ie/ops.hpp:525-529, src/ops/gemv_q4_0.cpp:54-120   fp16 activations, GGUF blocks

@@ -592,6 +592,78 @@ static int gemv_x2(mx_stream_t s, const void* x, const typename F::W& wa, const 
     GemvSeg<F, half_t> a{wa, reinterpret_cast<half_t*>(ya), nullptr}, b{wb, reinterpret_cast<half_t*>(yb), nullptr};
     return launch_q8<F, half_t>(s, a, b, 2, x, K, N, 1);
 }
+// Decode FFN forms (T = 1, one K tile): NW = 2 walks row n of the gate and of the up matrix together and writes
+// h[n] = half(silu(half(g)) * half(u)), the rounding points of the three-launch chain gemv, gemv, swiglu
+// (src/ops/elementwise.cpp:449-466 on fp16 g and u); NW = 1 is the plain GEMV.  XF16: the activation row arrives
+// as fp16 and is quantized to q8 while it is staged (the same values as quantize_q8_1, so the same output bits),
+// which removes the quantize launch in front of the GEMV.
+template <class F, int NW, int G, int U, bool XF16>
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_ffn_kernel(typename F::W w0, typename F::W w1, const void* x, half_t* y, uint32_t K, uint32_t N,
+                                                                    uint32_t KT) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    ActTile act;
+    if (XF16) {
+        auto hrow = [&](uint32_t) { return static_cast<const half_t*>(x); };
+        act = stage_act_f16<F::SUM_GRAN, 1>(lds, hrow, 0, K, KT);
+    } else {
+        auto xrow = [&](uint32_t) { return static_cast<const uint8_t*>(x); };
+        act = stage_act<F::SUM_GRAN, 1>(lds, xrow, 0, K, KT, false);
+    }
+    __syncthreads();
+    const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    const uint32_t n_units = (K + 63) / 64;
+    const bool half_tail = (K & 63u) != 0;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
+        const uint32_t n = rg * ROWS_PER_WG + wave * GROUPS + grp;
+        const uint32_t nc = n < N ? n : N - 1;
+        typename F::Cursor cu[NW];
+        cu[0] = F::cursor(w0, nc, gl);
+        if (NW == 2) cu[NW - 1] = F::cursor(w1, nc, gl);
+        float acc[NW][1];
+#pragma unroll
+        for (int r = 0; r < NW; ++r) acc[r][0] = 0.f;
+        gemv_rows<F, 1, NW, G, U>(cu, n_units, half_tail, gl, act, acc);
+        const float v0 = group_sum<G>(acc[0][0]);
+        const float v1 = (NW == 2) ? group_sum<G>(acc[NW - 1][0]) : 0.f;
+        if (lane == (uint32_t)group_sum_lane<G>(lane) && n < N) {
+            if (NW == 2) {
+                const float g = (float)(half_t)v0, u = (float)(half_t)v1;
+                y[n] = (half_t)((g / (1.f + __expf(-g))) * u);
+            } else {
+                y[n] = (half_t)v0;
+            }
+        }
+    }
+}
+
+template <class F, int NW, bool XF16>
+static int launch_ffn(mx_stream_t s, const typename F::W& w0, const typename F::W& w1, const void* x, uint16_t* y, uint32_t K, uint32_t N) {
+    const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);
+    const uint32_t KT = (K + 255) / 256 * 256;
+    if ((uint64_t)KT / 32 * per_elem_x32 > kLdsBudget) return MX_ERR_SHAPE;   // the activation row has to fit one LDS tile
+    const uint32_t G = pick_group((K + 63) / 64);
+    const uint32_t rows_per_wg = kGemvWaves * (64 / G);
+    const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg, cap = (uint32_t)cu_count() * kWgsPerCu;
+    const dim3 grid(n_rg < cap ? n_rg : cap), block(kGemvThreads);
+    const uint32_t lds = act_tile_bytes(1, KT, F::SUM_GRAN);
+    half_t* yh = reinterpret_cast<half_t*>(y);
+    constexpr int U = std::is_same<F, FmtQ8Aos>::value ? 1 : 2;
+    if (G == 16) hipLaunchKernelGGL((gemv_q8_ffn_kernel<F, NW, 16, U, XF16>), grid, block, lds, as_stream(s), w0, w1, x, yh, K, N, KT);
+    else if (G == 32) hipLaunchKernelGGL((gemv_q8_ffn_kernel<F, NW, 32, U, XF16>), grid, block, lds, as_stream(s), w0, w1, x, yh, K, N, KT);
+    else hipLaunchKernelGGL((gemv_q8_ffn_kernel<F, NW, 64, U, XF16>), grid, block, lds, as_stream(s), w0, w1, x, yh, K, N, KT);
+    return launch_status();
+}
+template <class F, int NW>
+static int launch_ffn_x(mx_stream_t s, const typename F::W& w0, const typename F::W& w1, const void* x, int x_is_f16, uint16_t* y, uint32_t K, uint32_t N) {
+    if (int rc = check_common(x, y, K, N, 1, F::K_ALIGN)) return rc;
+    MX_REQUIRE_ALIGN(x, x_is_f16 ? 16 : 8);
+    return x_is_f16 ? launch_ffn<F, NW, true>(s, w0, w1, x, y, K, N) : launch_ffn<F, NW, false>(s, w0, w1, x, y, K, N);
+}
+
 // Streaming-read yardstick: the same persistent launch geometry as the decode GEMV (workgroups per CU x CUs,
 // 256 threads, 16-byte loads, four in flight per thread) with no arithmetic, so that a GEMV launch can be
 // priced against what a pure read of the same bytes achieves on the same device.
@@ -897,6 +969,54 @@ int mx_gemv_mxfp4_soa_f16(mx_stream_t s, const uint16_t* A, const uint8_t* qs, c
     MX_REQUIRE_PTR(e);
     MX_REQUIRE_ALIGN(qs, 16);
     return launch_fact<FmtMxfp4Soa>(s, FmtMxfp4Soa::W{qs, e, K}, reinterpret_cast<const half_t*>(A), reinterpret_cast<half_t*>(y), K, N);
+}
+
+// ---- decode FFN forms: fused gate + up + SwiGLU, and GEMVs that take the fp16 activation row
+int mx_gemv_q8_0_soa_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
+                             const uint16_t* u_d, uint16_t* h, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d);
+    MX_REQUIRE_ALIGN(g_qs, 16); MX_REQUIRE_ALIGN(u_qs, 16); MX_REQUIRE_ALIGN(g_d, 2); MX_REQUIRE_ALIGN(u_d, 2);
+    return launch_ffn_x<FmtQ8Soa, 2>(s, {g_qs, g_d, K}, {u_qs, u_d, K}, x, x_is_f16, h, K, N);
+}
+static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, const void* W0, const void* W1, uint16_t* y, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(W0); MX_REQUIRE_PTR(W1);
+    MX_REQUIRE_SHAPE(K % (fmt == 0 ? 32u : 256u) == 0);
+    MX_REQUIRE_ALIGN(W0, fmt == 1 ? 16 : 2); MX_REQUIRE_ALIGN(W1, fmt == 1 ? 16 : 2);
+    const uint8_t *a = static_cast<const uint8_t*>(W0), *b = static_cast<const uint8_t*>(W1);
+    if (fmt == 1) {
+        const FmtQ4K::W wa{a, K / 256 * (uint32_t)kQ4KBytes}, wb{b, K / 256 * (uint32_t)kQ4KBytes};
+        return nw == 2 ? launch_ffn_x<FmtQ4K, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ4K, 1>(s, wa, wb, x, x_is_f16, y, K, N);
+    }
+    if (fmt == 2) {
+        const FmtQ6K::W wa{a, K / 256 * (uint32_t)kQ6KBytes}, wb{b, K / 256 * (uint32_t)kQ6KBytes};
+        return nw == 2 ? launch_ffn_x<FmtQ6K, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ6K, 1>(s, wa, wb, x, x_is_f16, y, K, N);
+    }
+    const FmtQ8Aos::W wa{a, K / 32 * (uint32_t)kQ8_0Bytes}, wb{b, K / 32 * (uint32_t)kQ8_0Bytes};
+    return nw == 2 ? launch_ffn_x<FmtQ8Aos, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ8Aos, 1>(s, wa, wb, x, x_is_f16, y, K, N);
+}
+int mx_gemv_q4_K_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h, uint32_t K, uint32_t N) {
+    return ffn_aos(1, 2, s, x, x_is_f16, gate_W, up_W, h, K, N);
+}
+int mx_gemv_q6_K_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h, uint32_t K, uint32_t N) {
+    return ffn_aos(2, 2, s, x, x_is_f16, gate_W, up_W, h, K, N);
+}
+int mx_gemv_q8_0_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h, uint32_t K, uint32_t N) {
+    return ffn_aos(0, 2, s, x, x_is_f16, gate_W, up_W, h, K, N);
+}
+int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(qs_W); MX_REQUIRE_PTR(d_W);
+    MX_REQUIRE_ALIGN(qs_W, 16); MX_REQUIRE_ALIGN(d_W, 2);
+    const FmtQ8Soa::W w{qs_W, d_W, K};
+    return launch_ffn_x<FmtQ8Soa, 1>(s, w, w, x_f16, 1, y, K, N);
+}
+int mx_gemv_q4_K_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return ffn_aos(1, 1, s, x_f16, 1, W, W, y, K, N);
+}
+int mx_gemv_q6_K_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return ffn_aos(2, 1, s, x_f16, 1, W, W, y, K, N);
+}
+int mx_gemv_q8_0_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N) {
+    return ffn_aos(0, 1, s, x_f16, 1, W, W, y, K, N);
 }
 
 int mx_probe_stream_read(mx_stream_t s, const void* src, uint64_t n_bytes, uint32_t* sink) {

@@ -403,6 +403,28 @@ def gemv_q8_x2(fmt, x_q8, W_a, W_b, K, N, y_a=None, y_b=None):
     return y_a, y_b
 
 
+def gemv_x2_silu(fmt, x, W_gate, W_up, K, N, h=None):
+    """h = silu(W_gate . x) * (W_up . x) in one launch (decode, T = 1); x = the q8 row (uint8 tensor) or the fp16 row.
+    fmt as gemv_q8_x2.  Same bits as gemv_q8_x2 + swiglu (and quantize_q8_1 in front when x is fp16)."""
+    x_is_f16 = 1 if x.dtype == torch.float16 else 0
+    h = _out(h, (N,), torch.float16, x)
+    if fmt == "q8_0_soa":
+        _call("mx_gemv_q8_0_soa_x2_silu", _ptr(x), x_is_f16, _u8(W_gate[0]), _ptr(W_gate[1]), _u8(W_up[0]), _ptr(W_up[1]), _ptr(h), K, N)
+    else:
+        _call("mx_gemv_%s_x2_silu" % fmt, _ptr(x), x_is_f16, _u8(W_gate), _u8(W_up), _ptr(h), K, N)
+    return h
+
+
+def gemv_f16q8(fmt, x_f16, W, K, N, y=None):
+    """y = W . q8(x) with the fp16 row x quantized while it is staged: quantize_q8_1 + gemv_*_q8 in one launch (T = 1)."""
+    y = _out(y, (N,), torch.float16, x_f16)
+    if fmt == "q8_0_soa":
+        _call("mx_gemv_q8_0_soa_f16q8", _f16(x_f16), _u8(W[0]), _ptr(W[1]), _ptr(y), K, N)
+    else:
+        _call("mx_gemv_%s_f16q8" % fmt, _f16(x_f16), _u8(W), _ptr(y), K, N)
+    return y
+
+
 def gemv_q4_0(A, W, K, N, y=None):
     y = _out(y, (N,), torch.float16, A)
     _call("mx_gemv_q4_0", _f16(A), _u8(W), _ptr(y), K, N)
@@ -606,11 +628,15 @@ def rms_norm_f32w_q8(x, w, eps):
     return y, q8
 
 
-def swiglu_q8(gate, up, oai=False, alpha=1.702, limit=7.0, want_y=True):
-    """-> (y fp16 or None, block_q8_1x stream of y): silu(gate)*up, or the clamped gpt-oss form with oai=True."""
+def swiglu_q8(gate, up, oai=False, alpha=1.702, limit=7.0, want_y=True, out=None):
+    """-> (y fp16 or None, block_q8_1x stream of y): silu(gate)*up, or the clamped gpt-oss form with oai=True.
+    out = (y, q8) reuses caller buffers."""
     n = gate.numel()
-    y = torch.empty_like(gate) if want_y else None
-    q8 = torch.empty(n // 32 * Q81X_BYTES, dtype=torch.uint8, device=gate.device)
+    if out is not None:
+        y, q8 = out
+    else:
+        y = torch.empty_like(gate) if want_y else None
+        q8 = torch.empty(n // 32 * Q81X_BYTES, dtype=torch.uint8, device=gate.device)
     if oai:
         _call("mx_swiglu_oai_q8", _f16(gate), _f16(up), _ptr(y), _ptr(q8), n, alpha, limit)
     else:

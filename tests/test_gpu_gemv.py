@@ -11,6 +11,10 @@ from gpu_util import check, dev, host, weights
 pytestmark = pytest.mark.gpu
 
 
+def f16(a):
+    return np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
+
+
 def acts(seed, T, K):
     """fp32 N(0,1) activations rounded to fp16 (what the fp16 entry points see)."""
     return O.round_fp16(O.normal(seed, (T, K), 0.0, 1.0))
@@ -262,6 +266,50 @@ def test_gemv_q8_x2_equals_two_single_launches(mx, fmt):
         sa, sb = [tuple(dev(p) for p in O.repack_q8_0_to_soa(W)) for W in (Wa, Wb)]
         ya2, yb2 = mx.ops.gemv_q8_x2("q8_0_soa", xq, sa, sb, K, N)
         assert torch.equal(ya2, mx.ops.gemv_q8_0_soa_q8(xq, sa[0], sa[1], K, N)) and torch.equal(yb2, mx.ops.gemv_q8_0_soa_q8(xq, sb[0], sb[1], K, N))
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+@pytest.mark.parametrize("K,N", [(2048, 320), (4096, 1056), (1280, 96)])
+def test_decode_ffn_forms_equal_the_launch_chain(mx, fmt, K, N):
+    """gate + up + SwiGLU in one launch, and GEMVs that quantize the fp16 activation row while staging it: the bits of
+    quantize_q8_1 -> gemv x2 -> swiglu and of quantize_q8_1 -> gemv, whose parts are gated against the oracle above.
+    K = 2048 / 4096 / 1280 walk 32, 64 and 16 lanes per row (1280 leaves lanes of the last round without a unit)."""
+    ops = mx.ops
+    name = O.FMT_NAMES[fmt]
+    Wg, Wu = weights(fmt, 1600 + fmt, N, K), weights(fmt, 1610 + fmt, N, K)
+    x16 = dev(acts(1620 + K, 1, K)).half()
+    xq = ops.quantize_q8_1(x16)
+    forms = [(name, dev(Wg), dev(Wu))]
+    if fmt == O.Q8_0:
+        forms.append(("q8_0_soa",) + tuple(tuple(dev(p) for p in O.repack_q8_0_to_soa(W)) for W in (Wg, Wu)))
+    for nm, g_w, u_w in forms:
+        g, u = ops.gemv_q8_x2(nm, xq, g_w, u_w, K, N)
+        h_chain, hq_chain = ops.swiglu_q8(g, u)
+        h1 = ops.gemv_x2_silu(nm, xq, g_w, u_w, K, N)
+        h2 = ops.gemv_x2_silu(nm, x16.reshape(-1), g_w, u_w, K, N)
+        assert torch.equal(h1, h_chain), "%s: fused gate/up/silu on the q8 row != the three launches" % nm
+        assert torch.equal(h2, h_chain), "%s: fused gate/up/silu on the fp16 row != the four launches" % nm
+        single = (lambda w: ops.gemv_q8_0_soa_q8(xq, w[0], w[1], K, N)) if nm == "q8_0_soa" else (lambda w: getattr(ops, "gemv_%s_q8" % nm)(xq, w, K, N))
+        assert torch.equal(ops.gemv_f16q8(nm, x16.reshape(-1), g_w, K, N), single(g_w)), "%s: gemv on the fp16 row != quantize + gemv" % nm
+    # and the fused result against the oracle chain directly (q8-chain dots, fp16 roundings of g and u, SwiGLU)
+    xq_h = host(xq)
+    g_ref = f16(O.gemv_q8chain(fmt, Wg, xq_h, K, N)[0]).astype(np.float32)
+    u_ref = f16(O.gemv_q8chain(fmt, Wu, xq_h, K, N)[0]).astype(np.float32)
+    check(host(h1).astype(np.float32), O.swiglu_np(g_ref, u_ref), "fused gate/up/silu vs oracle", max_rel=3e-3)
+
+
+def test_decode_ffn_forms_reject_bad_arguments(mx):
+    ops = mx.ops
+    K, N = 512, 64
+    W = dev(weights(O.Q4_K, 1700, N, K))
+    x16 = dev(acts(1701, 1, K)).half().reshape(-1)
+    with pytest.raises(ops.MxError):
+        ops.gemv_f16q8("q4_K", x16, W, K + 32, N)                      # K not a multiple of 256
+    with pytest.raises(ops.MxError):
+        ops.gemv_f16q8("q4_K", x16[4:], W, K, N)                       # fp16 row not 16-byte aligned
+    big = 65536
+    with pytest.raises(ops.MxError):
+        ops.gemv_f16q8("q6_K", torch.zeros(big, dtype=torch.float16, device="cuda"), torch.zeros(big // 256 * 210, dtype=torch.uint8, device="cuda"), big, 1)   # row longer than one LDS tile
 
 
 @pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
