@@ -43,11 +43,12 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
     const uint32_t n_tiles = (K + KT - 1) / KT;
     ActTile act;
     bool staged = false;
-    if (kPrefetchAcrossRows<F> && K == 64u * G && n_tiles == 1) {
+    if (T <= 2 && kPrefetchAcrossRows<F> && K == 64u * G && n_tiles == 1) {
         // One unit per lane and row (K = 4096 with 64 lanes per row, ...): a row is a single round of loads, so the
         // loads of the next row group are issued before the dot products and the lane-group sum of this one;
         // otherwise every wave would sit with nothing in flight from its last load's arrival to its store.
-        // Measured on 4096 -> 14336: Q8_0 planes 13.2 -> 12.4 us, Q4_K 8.6 -> 8.4 us.
+        // Measured on 4096 -> 14336: Q8_0 planes 13.2 -> 12.4 us (T = 2: 14.2 -> 13.0), Q4_K 8.6 -> 8.4 us (T = 2:
+        // 10.2 -> 9.2).  Batches of four and more lose (the second set of units costs occupancy next to R x T sums).
         // The first row group's weights are requested before the activation row is staged: they do not depend on it.
         typename F::Cursor cn[R];
         typename F::Raw nxt[R];
