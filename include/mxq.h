@@ -275,7 +275,12 @@ int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uin
  *   dequant_q4_K_to_Bt + gemm_fp16(_onednn)      src/model/dense_dispatch.hpp:658-693
  * K % 256 == 0 (Q4_K), K % 128 == 0 (Q8_0 planes); A and W 16-byte aligned.
  * mx_gemm_q8_0_soa takes the SoA planes of gemv_q8_0_soa_q8 (the reference runs Q8_0 prefill
- * as dequant_q8_0_soa_to_Bt + gemm_fp16, src/model/qwen35_dense.cpp:811-831).  */
+ * as dequant_q8_0_soa_to_Bt + gemm_fp16, src/model/qwen35_dense.cpp:811-831).
+ * A launch whose 128-token tiles would cover at most half of the CUs (a short batch against a narrow
+ * matrix) and whose K is at least 2048 is cut into 2..8 K slices; their fp32 partial sums go through a
+ * 16 MB per-device scratch array owned by the library (nothing is allocated) and are added in slice
+ * order by a second small launch: two such calls that overlap on one device race on it, as the
+ * reference's static per-device scratch buffers would (src/model/dense_dispatch.hpp:547-560).  */
 int mx_gemm_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M,
                      uint32_t K, uint32_t N);

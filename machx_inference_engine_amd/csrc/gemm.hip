@@ -414,9 +414,27 @@ struct GemmArgs {
     float* y_acc;                     //   and the fp32 [T, N] buffer w * acc is atomically added into (Y unused)
     uint32_t M, K, N, E;
     uint32_t tiles_m, tiles_n;        // dense tile grid; grouped: tiles_m is an upper bound
+    uint32_t k_split;                 // dense only: K slices per output tile (above 1: fp32 partial sums go to g_gemm_splitk_acc)
 };
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
+
+// Dense launches with too few output tiles for the chip (a short batch against a narrow matrix) cut K into up to
+// eight slices: every slice writes its fp32 partial sums to its own plane of this per-device scratch, and a last
+// launch adds the planes in slice order and rounds to fp16 (so the result does not depend on which slice finished
+// first).  Launches that overlap on one device would race on it, as with the reference's static per-device scratch
+// buffers (src/model/dense_dispatch.hpp:547-560).
+constexpr uint32_t kGemmSplitElems = 4u << 20;   // slices * M * N <= 4 Mi partial sums (16 MB)
+constexpr uint32_t kGemmSplitMax = 8;
+__device__ float g_gemm_splitk_acc[kGemmSplitElems];
+
+__global__ __launch_bounds__(256) void gemm_splitk_store_kernel(half_t* y, uint32_t n, uint32_t k_split) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = g_gemm_splitk_acc[i];
+    for (uint32_t k = 1; k < k_split; ++k) v += g_gemm_splitk_acc[(size_t)k * n + i];
+    y[i] = (half_t)v;
+}
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
@@ -522,6 +540,7 @@ struct TileCtx {
     uint32_t a_dst;
     const uint8_t* lds_raw;
     uint32_t frag0, n_chunks, mi;
+    uint32_t c0;   // first chunk of this K slice (chunk numbers below are slice-local)
 };
 
 // Chunk c out of register set P; meanwhile (`more`) the A rows of chunk c+1 and the weights of chunk c+DEPTH are requested.
@@ -537,13 +556,13 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
 #pragma unroll
         for (int j = 0; j < NL; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
         const uint32_t cn = (c + DEPTH < t.n_chunks) ? c + DEPTH : t.n_chunks - 1;   // past the end: the last chunk again, unused
-        raw[PN][0] = QF::load(t.w0, t.wrow0, cn, t.h);
-        raw[PN][1] = QF::load(t.w1, t.wrow1, cn, t.h);
+        raw[PN][0] = QF::load(t.w0, t.wrow0, t.c0 + cn, t.h);
+        raw[PN][1] = QF::load(t.w1, t.wrow1, t.c0 + cn, t.h);
         __builtin_amdgcn_sched_barrier(0);   // the scheduler must not sink these loads towards their uses
     }
     typename QF::Dec dec[2];
-    dec[0] = QF::prepare(raw[P][0], c, t.h);
-    dec[1] = QF::prepare(raw[P][1], c, t.h);
+    dec[0] = QF::prepare(raw[P][0], t.c0 + c, t.h);
+    dec[1] = QF::prepare(raw[P][1], t.c0 + c, t.h);
     mma_chunk<QF, PARTIAL, NA>(raw[P], dec, t.lds_raw, (c & 1u) * ABUF + t.frag0, acc, t.mi);
     if (more) {
         wait_vmcnt<(DEPTH > 1 ? W_LOADS_MIN : 0)>();   // A rows of chunk c+1 are in LDS (DEPTH > 1: the newest weight loads stay in flight)
@@ -566,7 +585,8 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
 // whatever the compiler made of QF::load.
 template <class QF, int MODE, bool PIPE, int NA, int DEPTH>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::W& w0, const typename QF::W& w1, const uint32_t (&wrow)[2],
-                                          uint32_t row_lo, uint32_t row_hi, uint32_t n_base, uint8_t* lds_raw) {
+                                          uint32_t row_lo, uint32_t row_hi, uint32_t n_base, uint8_t* lds_raw, uint32_t c0 = 0,
+                                          uint32_t n_chunks_slice = 0, uint32_t ks = 0) {
     static_assert(DEPTH == 1 || DEPTH == 2, "prefetch depth");
     static_assert(!PIPE || NA == 4, "the pipelined chunk is written for four token tiles");
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
@@ -575,7 +595,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
     constexpr int NL = 2 * NA;   // 1 KB loads per wave per chunk
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 31u, h = lane >> 5;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t n_chunks = g.K / kBK;
+    const uint32_t n_chunks = n_chunks_slice ? n_chunks_slice : g.K / kBK;   // chunks of this K slice (all of K unless split)
     const uint32_t live_rows = (row_hi - row_lo) >= BM ? BM : row_hi - row_lo;
     const uint32_t mi = (live_rows + 31u) / 32u;
 
@@ -589,7 +609,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
         const uint32_t Rc = R < live_rows ? R : live_rows - 1u;
         a_off[j] = Rc * (g.K * 2u) + (((lane & 15u) ^ (R & 15u)) << 4);
     }
-    const uint8_t* a_glb = reinterpret_cast<const uint8_t*>(g.A + (size_t)row_lo * g.K);
+    const uint8_t* a_glb = reinterpret_cast<const uint8_t*>(g.A + (size_t)row_lo * g.K) + (size_t)c0 * (kBK * 2u);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds_raw;
     const uint32_t a_dst = lds_base + wave * (BM / 4u) * 256u;   // this wave's quarter of the rows inside an A buffer
     // step-0 fragment address of this lane inside an A buffer
@@ -609,18 +629,18 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
     typename QF::Raw raw[NSET][2];
 #pragma unroll
     for (int j = 0; j < NL; ++j) load_to_lds16(a_glb, a_off[j], a_dst + 1024u * j);
-    raw[0][0] = QF::load(w0, wrow[0], 0, h);
-    raw[0][1] = QF::load(w1, wrow[1], 0, h);
+    raw[0][0] = QF::load(w0, wrow[0], c0, h);
+    raw[0][1] = QF::load(w1, wrow[1], c0, h);
     wait_vmcnt<0>();
     __syncthreads();
 #pragma unroll
     for (int d = 1; d < DEPTH; ++d) {
         const uint32_t cd = (uint32_t)d < n_chunks ? (uint32_t)d : n_chunks - 1;
-        raw[d][0] = QF::load(w0, wrow[0], cd, h);
-        raw[d][1] = QF::load(w1, wrow[1], cd, h);
+        raw[d][0] = QF::load(w0, wrow[0], c0 + cd, h);
+        raw[d][1] = QF::load(w1, wrow[1], c0 + cd, h);
     }
 
-    const TileCtx<QF, NA> ctx{w0, w1, wrow[0], wrow[1], h, a_glb, a_dst, lds_raw, frag0, n_chunks, mi};
+    const TileCtx<QF, NA> ctx{w0, w1, wrow[0], wrow[1], h, a_glb, a_dst, lds_raw, frag0, n_chunks, mi, c0};
 #define CHUNK(P, c, more) gemm_chunk<QF, PARTIAL, NA, DEPTH, P>(ctx, a_off, raw, acc, c, more)
     if constexpr (DEPTH == 1) {
         // two sets, and the set just loaded is copied into set 0 at the end of a chunk, where it has to have arrived anyway
@@ -663,6 +683,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
                     if (MODE == GEMM_MOE_DOWN && g.route_w) o *= (float)g.route_w[row];
                     if (MODE == GEMM_MOE_DOWN && g.y_acc)
                         __hip_atomic_fetch_add(g.y_acc + (size_t)g.row_token[row] * g.N + n, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else if (MODE == GEMM_DENSE && g.k_split > 1)
+                        g_gemm_splitk_acc[((size_t)ks * g.M + row) * g.N + n] = o;
                     else
                         g.Y[(size_t)row * g.N + n] = (half_t)o;
                 }
@@ -683,10 +705,12 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     // contiguous range of tiles, 4 token tiles x consecutive column tiles at a time)
     // Expert-grouped tiles are uneven (dead tiles past the real count, 1-4 live token sub-tiles),
     // so they are dealt round-robin over the XCDs instead of in contiguous ranges.
-    const uint32_t total = g.tiles_m * g.tiles_n;
+    const uint32_t ksplit = (MODE == GEMM_DENSE) ? g.k_split : 1u;   // workgroups per output tile (K slices)
+    const uint32_t total = g.tiles_m * g.tiles_n * ksplit;
     const uint32_t per_xcd = (total + 7) / 8;
-    const uint32_t linear = (MODE == GEMM_DENSE) ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
-    if ((MODE == GEMM_DENSE && (blockIdx.x >> 3) >= per_xcd) || linear >= total) return;
+    const uint32_t lin_ks = (MODE == GEMM_DENSE) ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    if ((MODE == GEMM_DENSE && (blockIdx.x >> 3) >= per_xcd) || lin_ks >= total) return;
+    const uint32_t linear = lin_ks / ksplit, ks = lin_ks - linear * ksplit;
     uint32_t tm, tn;
     {
         constexpr uint32_t GM = 4;
@@ -751,8 +775,11 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     if (wrow[1] >= g.N) wrow[1] = g.N - 1;
 
     if constexpr (MODE == GEMM_DENSE) {
-        gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
+        const uint32_t n_all = g.K / kBK, per = (n_all + ksplit - 1) / ksplit;
+        const uint32_t c0 = ks * per, c1 = (c0 + per < n_all) ? c0 + per : n_all;
+        gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, c0, c1 - c0, ks);
     } else {
+        (void)ks;
         // expert-grouped tiles: a full one takes the same pipelined chunk as the dense GEMM; one with at most 64
         // live rows keeps half the accumulators and spends the registers on a second chunk of weights in flight
         const uint32_t live = row_hi - row_lo;
@@ -768,7 +795,8 @@ static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const type
     constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU) ? 128 : 256, BM = 32u * NI, lds = 2u * BM * kBK * 2u;
     g.tiles_n = (g.N + BN - 1) / BN;
     g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + BM - 1) / BM : rows_bound / BM + g.E;   // grouped: an upper bound, workgroups past the real count leave at once
-    const uint64_t total = (uint64_t)g.tiles_m * g.tiles_n;
+    if (MODE != GEMM_DENSE || g.k_split == 0) g.k_split = 1;
+    const uint64_t total = (uint64_t)g.tiles_m * g.tiles_n * g.k_split;
     const uint64_t grid = (total + 7) / 8 * 8;
     if (grid > 0x7FFFFFFFull) return MX_ERR_SHAPE;
     static bool attr_set = false;   // LDS at the 64 KB default limit: opt in once per kernel
@@ -800,8 +828,42 @@ static int gemm_cu_count() {
 template <class QF, int MODE>
 static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
     if constexpr (MODE == GEMM_DENSE) {
+        const uint64_t cus = (uint64_t)gemm_cu_count();
         const uint64_t tiles128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 255) / 256);
-        if (g.M > 64 && 2 * tiles128 <= (uint64_t)gemm_cu_count()) return launch_gemm_ni<QF, MODE, 2>(s, b0, b1, g, rows_bound);
+        const uint64_t tiles64 = (uint64_t)((g.M + 63) / 64) * ((g.N + 255) / 256);
+        const uint64_t mn = (uint64_t)g.M * g.N, n_chunks = g.K / kBK;
+        // K slices a tiling could take: until every CU has a workgroup, each slice at least 8 chunks deep, the partial
+        // sums within the scratch
+        auto slices = [&](uint64_t tiles) {
+            uint64_t k = tiles ? cus / tiles : 1;
+            if (k > kGemmSplitMax) k = kGemmSplitMax;
+            if (k > n_chunks / 8) k = n_chunks / 8;
+            if (k * mn > kGemmSplitElems) k = kGemmSplitElems / mn;
+            return k < 1 ? (uint64_t)1 : k;
+        };
+        bool ni2 = false;
+        uint64_t k_split = 1;
+        if (2 * tiles128 <= cus) {
+            // 128-token tiles would leave half the CUs idle.  They stay (they do twice the matrix work per dequantized
+            // weight) when K slices alone fill three quarters of the chip; otherwise 64-token tiles, sliced as well.
+            // Measured at K = 14336, N = 4096: T = 128 94 -> 39 us, T = 512 162 -> 111 us.
+            const uint64_t k4 = slices(tiles128);
+            if (4 * tiles128 * k4 >= 3 * cus || g.M <= 64) {
+                k_split = k4;
+            } else {
+                ni2 = true;
+                k_split = slices(tiles64);
+            }
+        }
+        if (k_split >= 2) {
+            const uint32_t per = (uint32_t)((n_chunks + k_split - 1) / k_split);
+            g.k_split = (uint32_t)((n_chunks + per - 1) / per);   // no empty slice
+            const int rc = ni2 ? launch_gemm_ni<QF, MODE, 2>(s, b0, b1, g, rows_bound) : launch_gemm_ni<QF, MODE, 4>(s, b0, b1, g, rows_bound);
+            if (rc != MX_OK) return rc;
+            hipLaunchKernelGGL(gemm_splitk_store_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, as_stream(s), g.Y, (uint32_t)mn, g.k_split);
+            return launch_status();
+        }
+        if (ni2) return launch_gemm_ni<QF, MODE, 2>(s, b0, b1, g, rows_bound);
     }
     return launch_gemm_ni<QF, MODE, 4>(s, b0, b1, g, rows_bound);
 }
