@@ -31,6 +31,23 @@ def test_gemm_q4_K(mx, M, K, N):
         check(one[0], ref[1], "row 1 alone")
 
 
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+@pytest.mark.parametrize("M,K,N", [(8, 4096, 512), (64, 2048, 260), (200, 3072, 768), (512, 7168, 256)])
+def test_gemm_k_slices(mx, fmt, M, K, N):
+    """Launches with too few output tiles for the chip run as K slices plus a launch that adds the slices in order:
+    4 slices of 128-token tiles (M <= 64), 2..8 slices of 64-token tiles, a last slice shorter than the others
+    (K = 3072: 24 chunks in 3 slices; K = 7168: 56 chunks in 7).  Against the oracle, and the same bits from launch to launch."""
+    W = weights(fmt, 2100 + N, N, K)
+    A = f16(O.normal(2101 + M, (M, K)))
+    ref = O.gemv_f64(fmt, W, A, K, N, round_w_fp16=True)
+    fn = getattr(mx.ops, "gemm_%s" % O.FMT_NAMES[fmt])
+    a_d, w_d = dev(A).half(), dev(W)
+    got = fn(a_d, w_d, M, K, N)
+    check(host(got).astype(np.float32), ref, "gemm %s M=%d K=%d N=%d" % (O.FMT_NAMES[fmt], M, K, N))
+    for _ in range(3):
+        assert torch.equal(fn(a_d, w_d, M, K, N), got), "K-sliced GEMM differs from launch to launch"
+
+
 @pytest.mark.parametrize("M,K,N", [(128, 128, 256), (260, 768, 2048), (77, 2048, 768)])
 def test_gemm_q8_0_soa(mx, M, K, N):
     W = weights(O.Q8_0, 2100 + N, N, K)
