@@ -79,11 +79,17 @@ def test_config3_gemm_full_size(mx, K, N):
     ref = O.gemv_f64(O.Q4_K, W_rows, A[toks], K, len(rows), round_w_fp16=True)
     got = host(Y).astype(np.float32)[np.ix_(toks, rows)]
     check(got, ref, "gemm_q4_K T=%d K=%d N=%d sampled" % (T, K, N))
-    # token rows are independent: a single-token GEMM reproduces its row up to fp32 summation order
+    # token rows are independent: a single-token GEMM reproduces its row up to fp32 summation order (a launch this
+    # small runs as K slices whose partial sums are added afterwards): within one fp16 ulp of the value or of the row's rms
     t = int(toks[3])
     y1 = host(ops.gemm_q4_K(Ad[t:t + 1], W, 1, K, N)).astype(np.float32)[0]
     yt = host(Y[t]).astype(np.float32)
-    assert np.array_equal(y1, yt), "same tile schedule for any M: identical accumulation order"
+    rms = float(np.sqrt(np.mean(yt.astype(np.float64) ** 2)))
+    assert np.all(np.abs(y1 - yt) <= np.maximum(np.abs(yt), rms) * 2.0 ** -9), "a token row depends on the batch it is in"
+    # full 128-token tiles of a batch that is not sliced keep the accumulation order: identical bits
+    Y3 = ops.gemm_q4_K(Ad[:1024], W, 1024, K, N) if N > 8192 else None
+    if Y3 is not None:
+        assert torch.equal(Y3, Y[:1024])
     # and the last, partial token tile (T not a multiple of 128) leaves the others untouched
     Y2 = ops.gemm_q4_K(Ad[:T - 37], W, T - 37, K, N)
     assert torch.equal(Y2, Y[:T - 37])
