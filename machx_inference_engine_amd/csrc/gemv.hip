@@ -148,6 +148,69 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
     }
 }
 
+// Long rows with few of them, one token (the 14336 -> 4096 down projections): a launch with at most two workgroups per
+// CU, where a lane group walks its row in several rounds.  The plain walk loads a round, waits, sums, loads the next:
+// every wave has nothing in flight while it sums.  Here two rounds of U units rotate through two register sets
+// (never copied), so one round is always in flight while the other is summed, and both are requested before the
+// activation row is staged.  Twice the registers for units, which a launch this sparse can afford.
+template <class F, int G, class OutT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_deep_kernel(GemvSeg<F, OutT> seg, const uint8_t* xq8, uint32_t K, uint32_t N, uint32_t KT,
+                                                                     uint32_t q8_split) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int GROUPS = 64 / G, U = 2, R = 1, T = 1;
+    constexpr int ROWS_PER_WG = kGemvWaves * GROUPS;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t grp = lane / G, gl = lane % G;
+    auto xrow = [&](uint32_t) { return xq8; };
+    const uint32_t n_rg = (N + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    const uint32_t n_units = (K + 63) / 64;
+    const bool half_tail = (K & 63u) != 0;
+    const uint32_t n_whole = half_tail ? n_units - 1 : n_units;
+    const uint32_t nb = n_whole / G / U;   // full rounds of U units per lane
+    ActTile act;
+    bool staged = false;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x) {
+        const uint32_t row = rg * ROWS_PER_WG + wave * GROUPS + grp;
+        typename F::Cursor cu[R];
+        cu[0] = F::cursor(seg.w, row < N ? row : N - 1, gl);
+        typename F::Raw a[U][R], b[U][R];
+        auto fetch = [&](typename F::Raw (&dst)[U][R], uint32_t round) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) dst[u][0] = load_unit<F, G>(cu[0], round * U + u, false);
+        };
+        auto sum = [&](const typename F::Raw (&src)[U][R], uint32_t round, float (&acc)[R][T]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) gemv_step<F, T, R>(src[u], cu, gl + (round * U + u) * G, act, acc);
+        };
+        if (nb >= 1) fetch(a, 0);
+        if (nb >= 2) fetch(b, 1);
+        if (!staged) {
+            act = stage_act<F::SUM_GRAN, T>(lds, xrow, 0, K, KT, q8_split != 0);
+            __syncthreads();
+            staged = true;
+        }
+        float acc[R][T] = {{0.f}};
+        uint32_t k = 0;
+        for (; k + 2 <= nb; k += 2) {
+            sum(a, k, acc);
+            if (k + 2 < nb) fetch(a, k + 2);
+            sum(b, k + 1, acc);
+            if (k + 3 < nb) fetch(b, k + 3);
+        }
+        if (k < nb) sum(a, k, acc);
+        for (uint32_t it = nb * U; it * G + gl < n_units; ++it) {   // the ragged rest, predicated
+            typename F::Raw raw[R];
+            raw[0] = load_unit<F, G>(cu[0], it, half_tail && (it * G + gl == n_units - 1));
+            gemv_step<F, T, R>(raw, cu, gl + it * G, act, acc);
+        }
+        float v = group_sum<G>(acc[0][0]);
+        if (lane == (uint32_t)group_sum_lane<G>(lane) && row < N) {
+            if (seg.bias) v += seg.bias[row];
+            store_out(seg.y + row, v);
+        }
+    }
+}
+
 // Rows much longer than a wave can cover in one step (K >= 8192) with few of them (N = 4096: the down
 // projections): the whole workgroup walks R rows at a time, thread t of 256 taking units t, t + 256, ...,
 // and the four wave sums meet in LDS.  One memory round trip per row instead of K / 64 / G of them, and
@@ -475,6 +538,14 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
                 hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((N + 255) / 256, T_real), dim3(256), 0, st, s0.y, s0.bias, N, T_real, n_split);
                 return launch_status();
             }
+        }
+    }
+    if constexpr (T == 1 && kPrefetchAcrossRows<F>) {
+        // long rows, at most two workgroups per CU, at least two full rounds per lane: the two-round rotation
+        if (nseg == 1 && n_tiles == 1 && n_rg <= 2u * (uint32_t)cu_count() && ((K & 63u) ? (K + 63) / 64 - 1 : (K + 63) / 64) / G >= 4u) {
+            hipLaunchKernelGGL((gemv_q8_deep_kernel<F, G, OutT>), dim3(n_rg), dim3(kGemvThreads), act_tile_bytes(1, KT, F::SUM_GRAN), st, s0, xq8, K, N, KT,
+                               split ? 1u : 0u);
+            return launch_status();
         }
     }
     // A CU streams at a fixed rate (its waves' loads in flight over the memory latency), so the
