@@ -298,6 +298,24 @@ def test_decode_ffn_forms_equal_the_launch_chain(mx, fmt, K, N):
     check(host(h1).astype(np.float32), O.swiglu_np(g_ref, u_ref), "fused gate/up/silu vs oracle", max_rel=3e-3)
 
 
+@pytest.mark.parametrize("fmt,K", [(O.Q4_K, 14336), (O.Q8_0, 14336), (O.Q8_0, 14368), (O.Q8_0, 8192 + 96), (O.Q4_K, 8192)])
+def test_gemv_long_rows_few_of_them(mx, fmt, K):
+    """T = 1 on long rows with few of them takes the kernel that keeps two rounds of loads rotating; K = 14368 and 8288
+    leave a half unit and lanes without a unit in the last round.  Against the q8-chain oracle, AoS and SoA forms."""
+    N = 300
+    W = weights(fmt, 1800 + fmt, N, K)
+    xq = O.quantize_q8_1(acts(1810 + K, 1, K))
+    ref = O.gemv_q8chain(fmt, W, xq, K, N)
+    name = O.FMT_NAMES[fmt]
+    got = getattr(mx.ops, "gemv_%s_q8" % name)(dev(xq), dev(W), K, N)
+    check(host(got).astype(np.float32), ref[0], "gemv_%s_q8 K=%d N=%d" % (name, K, N))
+    if fmt == O.Q8_0:
+        qs, d = (dev(p) for p in O.repack_q8_0_to_soa(W))
+        got2 = mx.ops.gemv_q8_0_soa_q8(dev(xq), qs, d, K, N)
+        check(host(got2).astype(np.float32), ref[0], "gemv_q8_0_soa_q8 K=%d N=%d" % (K, N))
+        assert torch.equal(got, got2)
+
+
 def test_decode_ffn_forms_reject_bad_arguments(mx):
     ops = mx.ops
     K, N = 512, 64
