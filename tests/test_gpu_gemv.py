@@ -316,6 +316,24 @@ def test_gemv_long_rows_few_of_them(mx, fmt, K):
         assert torch.equal(got, got2)
 
 
+@pytest.mark.parametrize("K,N", [(1312, 96), (4128, 64), (14368, 32)])
+def test_decode_ffn_forms_half_unit_tail(mx, K, N):
+    """Q8_0 rows whose length is an odd number of 32-element blocks (a half unit at the end of the row), fp16 row
+    quantized while staged: the same bits as the launch chain, AoS and SoA."""
+    ops = mx.ops
+    Wg, Wu = weights(O.Q8_0, 1900 + K, N, K), weights(O.Q8_0, 1910 + K, N, K)
+    x16 = dev(acts(1920 + K, 1, K)).half().reshape(-1)
+    xq = ops.quantize_q8_1(x16)
+    for nm, g_w, u_w in (("q8_0", dev(Wg), dev(Wu)),
+                         ("q8_0_soa",) + tuple(tuple(dev(p) for p in O.repack_q8_0_to_soa(W)) for W in (Wg, Wu))):
+        g, u = ops.gemv_q8_x2(nm, xq, g_w, u_w, K, N)
+        h_chain, _ = ops.swiglu_q8(g, u)
+        assert torch.equal(ops.gemv_x2_silu(nm, x16, g_w, u_w, K, N), h_chain)
+        assert torch.equal(ops.gemv_x2_silu(nm, xq, g_w, u_w, K, N), h_chain)
+        assert torch.equal(ops.gemv_f16q8(nm, x16, g_w, K, N), g)
+    check(host(g).astype(np.float32), O.gemv_q8chain(O.Q8_0, Wg, host(xq), K, N)[0], "gate K=%d" % K)
+
+
 def test_decode_ffn_forms_reject_bad_arguments(mx):
     ops = mx.ops
     K, N = 512, 64
