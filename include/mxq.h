@@ -402,17 +402,20 @@ int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W,
                            uint64_t expert_stride_bytes, int soa, uint32_t T);
 /* Int-dot grouped kernels for K-quant expert banks (soa as above), expert-sorted rows partitioned by
  * expert_offsets[E+1] (total_rows = expert_offsets[E], known to the host from the packing):
- *   moe_prefill_gate_up_silu_q4k_q8       include/ie/ops.hpp:912-919, src/ops/moe_fused.cpp:546-725   block_q8_1x rows
- *   moe_prefill_gate_up_silu_q6k_q8       src/ops/moe_qwen3.cpp:52-551 (include/ie/moe_qwen3.hpp)      block_q8_1x rows
+ * Every entry of the family takes block_q8_1s rows (48 B {d, s0, s1, pad, qs[32]} from mx_quantize_q8_1s, 16-byte
+ * aligned): the reference kernels read the header as one float4 and fold the min term on s0 + s1
+ * (src/ops/moe_fused.cpp:559-566,672-687; the "block_q8_1x" of the comment above that kernel is stale).
+ *   moe_prefill_gate_up_silu_q4k_q8       include/ie/ops.hpp:912-919, src/ops/moe_fused.cpp:546-725
+ *   moe_prefill_gate_up_silu_q6k_q8       src/ops/moe_qwen3.cpp:330-551 (include/ie/moe_qwen3.hpp)
  *   moe_prefill_down_packed_q4k_q8/_q6k_q8, moe_prefill_down_q{4,6}k_q8_gen
- *                                         include/ie/ops.hpp:993-1006, src/ops/moe_fused.cpp:1603-1924  block_q8_1s rows
+ *                                         include/ie/ops.hpp:993-1006, src/ops/moe_fused.cpp:1603-1924
  *     out_packed[row, n] = half(down_e . h_row), unweighted (moe_prefill_reduce applies the weights);
  *     any E_ffn % 256 == 0 (the reference's register-resident variant needs E_ffn == 512).
   */
-int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W,
+int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8s_packed, const void* gate_W, const void* up_W,
                                        const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
                                        uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
-int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W,
+int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8s_packed, const void* gate_W, const void* up_W,
                                        const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
                                        uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 int mx_moe_prefill_down_packed_q4k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W,

@@ -187,6 +187,7 @@ __global__ __launch_bounds__(kGemvThreads) void moe_fact_kernel(typename F::Bank
             for (uint32_t j = 0; j < n_act; ++j) {
                 const uint32_t slot = (MODE == FACT_DOWN) ? seg * a.K_top + j : seg;
                 const uint32_t e = (uint32_t)a.topk_idx[slot];
+                if (e >= 0x80000000u) continue;   // negative id: the slot contributes nothing (uniform for the block); the signature carries no expert count
                 const typename F::W w0 = F::expert(bank0, e), w1 = F::expert(NW == 2 ? bank1 : bank0, e);
                 typename F::Cursor c0 = F::cursor(w0, n, k0 / 64 + gl), c1 = F::cursor(w1, n, k0 / 64 + gl);
                 const float* xj = xa + (size_t)j * KT;
@@ -409,7 +410,7 @@ extern "C" {
 int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d,
                            uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
                            uint32_t E_ffn) {
-    const uint32_t n_experts = 0xFFFFFFFFu;   // the reference signature carries no expert count: ids are trusted
+    const uint32_t n_experts = 0x80000000u;   // the reference signature carries no expert count: only negative ids can be told apart (their slots are skipped)
     if (int rc = check_moe(x_q8, h_out, H, E_ffn, T * K)) return rc;
     MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d); MX_REQUIRE_PTR(topk_idx);
     MX_REQUIRE_SHAPE(K > 0 && n_experts > 0 && qs_stride % 16 == 0);
@@ -422,7 +423,7 @@ int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, 
 }
 int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
                    const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
-    const uint32_t n_experts = 0xFFFFFFFFu;
+    const uint32_t n_experts = 0x80000000u;
     if (int rc = check_moe(h_q8, y_packed, E_ffn, H, T * K)) return rc;
     MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(topk_w);
     MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
@@ -451,19 +452,22 @@ int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W,
     return moe_decode_fact<FmtQ6K, FACT_DOWN>(s, h, down_W, down_W, topk_idx, topk_w, y_out, E_ffn, H, K_top, T, expert_stride_bytes);
 }
 // ------------------------------------------------------------ K-quant experts, grouped rows, int-dot
-int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
+// Every entry of this family reads block_q8_1s rows (48 B: {d, s0, s1, pad, qs[32]}), as the reference kernels do
+// (src/ops/moe_fused.cpp:559-566,672-687: header as one float4, quants at +16 B, min term on s0 + s1;
+// src/ops/moe_qwen3.cpp:346); their callers quantize with quantize_q8_1s (src/model/qwen3moe.cpp:563,588).
+int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8s_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
                                        uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa,
                                        uint32_t total_rows) {
     if (soa)
-        return moe_grouped_kquant<FmtQ4KStr, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
-    return moe_grouped_kquant<FmtQ4K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+        return moe_grouped_kquant<FmtQ4KStr, 2, EPI_SILU>(s, xq8s_packed, true, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+    return moe_grouped_kquant<FmtQ4K, 2, EPI_SILU>(s, xq8s_packed, true, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
 }
-int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
+int mx_moe_prefill_gate_up_silu_q6k_q8(mx_stream_t s, const void* xq8s_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
                                        uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa,
                                        uint32_t total_rows) {
     if (soa)
-        return moe_grouped_kquant<FmtQ6KStr, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
-    return moe_grouped_kquant<FmtQ6K, 2, EPI_SILU>(s, xq8_packed, false, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+        return moe_grouped_kquant<FmtQ6KStr, 2, EPI_SILU>(s, xq8s_packed, true, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+    return moe_grouped_kquant<FmtQ6K, 2, EPI_SILU>(s, xq8s_packed, true, gate_W, up_W, expert_stride_bytes, expert_offsets, h_packed, E, H, E_ffn, total_rows);
 }
 int mx_moe_prefill_down_packed_q4k_q8(mx_stream_t s, const void* hq8s_packed, const void* down_W, const uint32_t* expert_offsets, uint16_t* out_packed,
                                       uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
@@ -593,7 +597,7 @@ int mx_moe_grouped_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_packed_f16, c
 }
 int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
                        const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
-    const uint32_t n_experts = 0xFFFFFFFFu;
+    const uint32_t n_experts = 0x80000000u;
     if (int rc = check_moe(h_f16, y_packed, E_ffn, H, T * K)) return rc;
     MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(topk_w);
     MX_REQUIRE_SHAPE(qs_stride % 16 == 0);

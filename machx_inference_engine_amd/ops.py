@@ -278,11 +278,11 @@ def moe_decode_down_kquant(fmt, h, down_W, topk_idx, topk_w, H, E_ffn, K_top, ex
     return y_out
 
 
-def moe_prefill_gate_up_silu_kquant_q8(fmt, xq8_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None,
+def moe_prefill_gate_up_silu_kquant_q8(fmt, xq8s_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None,
                                        soa=False):
-    """fmt in ('q4k', 'q6k'); xq8_packed: block_q8_1x rows."""
-    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8_packed)
-    _call("mx_moe_prefill_gate_up_silu_%s_q8" % fmt, _ptr(xq8_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
+    """fmt in ('q4k', 'q6k'); xq8s_packed: block_q8_1s rows (quantize_q8_1s), as the reference kernels read them."""
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, xq8s_packed)
+    _call("mx_moe_prefill_gate_up_silu_%s_q8" % fmt, _ptr(xq8s_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
           expert_stride_bytes, int(soa), TK)
     return h_packed
 

@@ -59,6 +59,7 @@ _q8_1s = _sig("orc_quantize_q8_1s", None, _vp, _vp, _i64)
 _gemv_f32 = _sig("orc_gemv_f32chain", None, C.c_int, _vp, _vp, _vp, _u32, _u32, _u32)
 _gemv_f64 = _sig("orc_gemv_f64", None, C.c_int, _vp, _vp, _vp, _u32, _u32, _u32, C.c_int)
 _gemv_q8 = _sig("orc_gemv_q8chain", None, C.c_int, _vp, _vp, _vp, _u32, _u32, _u32)
+_gemv_q8s = _sig("orc_gemv_q8schain", None, C.c_int, _vp, _vp, _vp, _u32, _u32, _u32)
 _int_codes = _sig("orc_int_codes", None, C.c_int, _vp, _u32, _vp)
 _route = _sig("orc_route_from_logits", None, _vp, _u32, _u32, _vp, _vp)
 _pack = _sig("orc_build_moe_packing", None, _vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp)
@@ -221,6 +222,15 @@ def gemv_q8chain(fmt, W, xq8, K, N):
     T = xq8.size // (K // 32 * Q8_1X_BYTES)
     y = np.empty((T, N), np.float64)
     _gemv_q8(fmt, _p(W), _p(xq8), _p(y), K, N, T)
+    return y
+
+
+def gemv_q8schain(fmt, W, xq8s, K, N):
+    """xq8s: block_q8_1s stream of T rows -> y [T,N] fp64; the K-quant min terms use the stored half sums."""
+    W, xq8s = _c(W, np.uint8), _c(xq8s, np.uint8)
+    T = xq8s.size // (K // 32 * Q8_1S_BYTES)
+    y = np.empty((T, N), np.float64)
+    _gemv_q8s(fmt, _p(W), _p(xq8s), _p(y), K, N, T)
     return y
 
 
@@ -389,13 +399,20 @@ def parity(got, ref, abs_floor=0.0):
               tests/unit/q8dot_test.cpp:112-135)
     cos     : cosine similarity
     max_abs_over_rms : max |g-r| / rms(r)
+    n_under_rms_floor / n_under_abs_floor : elements whose |r| lies below 1 % of the RMS / below abs_floor
+              (their error was divided by the floor, not by |r|)
     """
     g = np.asarray(got, np.float64).ravel()
     r = np.asarray(ref, np.float64).ravel()
     rms = float(np.sqrt(np.mean(r * r))) if r.size else 0.0
     if rms == 0.0:
-        return {"max_rel": float(np.max(np.abs(g))) if g.size else 0.0, "cos": 1.0, "max_abs_over_rms": 0.0, "rms": 0.0}
+        return {"max_rel": float(np.max(np.abs(g))) if g.size else 0.0, "cos": 1.0, "max_abs_over_rms": 0.0, "rms": 0.0,
+                "n": int(r.size), "n_under_rms_floor": int(r.size), "n_under_abs_floor": int(r.size)}
     err = np.abs(g - r)
-    return {"max_rel": float(np.max(err / np.maximum(np.abs(r), max(1e-2 * rms, abs_floor)))),
+    floor = max(1e-2 * rms, abs_floor)
+    return {"max_rel": float(np.max(err / np.maximum(np.abs(r), floor))),
             "cos": float(np.dot(g, r) / (np.linalg.norm(g) * np.linalg.norm(r) + 1e-300)),
-            "max_abs_over_rms": float(err.max() / rms), "rms": rms}
+            "max_abs_over_rms": float(err.max() / rms), "rms": rms, "n": int(r.size),
+            # how many elements were compared against a floored denominator instead of their own magnitude
+            "n_under_rms_floor": int(np.sum(np.abs(r) < 1e-2 * rms)),
+            "n_under_abs_floor": int(np.sum(np.abs(r) < abs_floor)) if abs_floor > 0 else 0}

@@ -33,6 +33,9 @@
  *                                            s0+s1==s, half-away rounding), brute force
  *   orc_gemv_* / orc_gemm_*                  pinned: brute-force int64 dots on tiny
  *                                            shapes, linearity, identity weights
+ *   orc_gemv_q8schain                        pinned: equals orc_gemv_q8chain on rows whose stored sums are d * sum(q);
+ *                                            closed forms with doctored sums (scale 0 / min 1 -> -(s0 + s1) per
+ *                                            sub-block; Q6_K d = sc = 1, zero quants -> -32 * s_half per group)
  *   orc_route_from_logits                    pinned: textbook softmax/top-k brute force
  *   orc_build_moe_packing                    pinned: oracle/_ref (ie::build_moe_packing)
  *                                            + permutation invariants
@@ -667,6 +670,62 @@ ORC_API void orc_gemv_q8chain(int fmt, const void* W, const void* xq8, double* y
                 y[(size_t)t * N + n] = acc;
             }
         }
+        free(w);
+    }
+}
+/* q8_1s-chain: the int-dot fold with the STORED half sums of block_q8_1s rows {d, s0, s1, pad, qs[32]}, the form the
+ * reference's expert-grouped K-quant kernels evaluate:
+ *   Q4_K  y += (d*sc)*(d8*idot) - (dmin*m)*(s0 + s1)   per 32-element sub-block (src/ops/moe_fused.cpp:672-687;
+ *         batched dense form with one half sum per lane, src/ops/gemv_q8dot.cpp:552-567)
+ *   Q6_K  y += (d*sc16)*(d8*idot_u - 32*s_half)        per 16-element group, idot_u over the unsigned 6-bit codes
+ *         (src/ops/moe_fused.cpp:1882-1891)
+ * Formats without a min term never read the sums: d_w * d8 * idot per block.  Accumulated in double.
+ * xq8s = T rows of K/32 block_q8_1s. */
+ORC_API void orc_int_codes(int fmt, const void* row, uint32_t K, int8_t* codes);
+ORC_API void orc_gemv_q8schain(int fmt, const void* W, const void* xq8s, double* y, uint32_t K, uint32_t N, uint32_t T) {
+    const size_t rb = (size_t)K / orc_block_elems(fmt) * orc_block_bytes(fmt);
+#pragma omp parallel
+    {
+        int8_t* codes = (int8_t*)malloc((size_t)K);
+        float* w = (float*)malloc((size_t)K * sizeof(float));
+#pragma omp for schedule(static)
+        for (uint32_t n = 0; n < N; ++n) {
+            const uint8_t* row = (const uint8_t*)W + n * rb;
+            orc_int_codes(fmt, row, K, codes);
+            if (fmt != ORC_Q4_K && fmt != ORC_Q6_K) orc_dequant(fmt, row, K, w);
+            for (uint32_t t = 0; t < T; ++t) {
+                const uint8_t* xb = (const uint8_t*)xq8s + (size_t)t * (K / 32) * Q8_1S_BYTES;
+                double acc = 0.0;
+                for (uint32_t b = 0; b < K / 32; ++b, xb += Q8_1S_BYTES) {
+                    float hdr[4];
+                    memcpy(hdr, xb, 16);
+                    const int8_t* q = (const int8_t*)(xb + 16);
+                    const double d8 = hdr[0];
+                    if (fmt == ORC_Q4_K) {
+                        const uint8_t* blk = row + (size_t)(b / 8) * Q4_K_BYTES;
+                        uint8_t sc, mn;
+                        orc_get_scale_min_k4((int)(b % 8), blk + 4, &sc, &mn);
+                        const float d1 = orc_fp16_to_fp32(rd16(blk)) * (float)sc, m1 = orc_fp16_to_fp32(rd16(blk + 2)) * (float)mn;
+                        long idot = 0;
+                        for (int i = 0; i < 32; ++i) idot += (long)codes[b * 32 + i] * q[i];
+                        acc += (double)d1 * (d8 * (double)idot) - (double)m1 * ((double)hdr[1] + (double)hdr[2]);
+                    } else if (fmt == ORC_Q6_K) {
+                        const uint8_t* blk = row + (size_t)(b / 8) * Q6_K_BYTES;
+                        const float d = orc_fp16_to_fp32(rd16(blk + 208));
+                        for (int hf = 0; hf < 2; ++hf) {
+                            const float c = d * (float)(int8_t)blk[192 + (b % 8) * 2 + hf];
+                            long idot_u = 0;
+                            for (int i = 0; i < 16; ++i) idot_u += (long)(codes[b * 32 + hf * 16 + i] + 32) * q[hf * 16 + i];
+                            acc += (double)c * (d8 * (double)idot_u - 32.0 * (double)hdr[1 + hf]);
+                        }
+                    } else {
+                        for (int i = 0; i < 32; ++i) acc += (double)w[b * 32 + i] * d8 * (double)q[i];
+                    }
+                }
+                y[(size_t)t * N + n] = acc;
+            }
+        }
+        free(codes);
         free(w);
     }
 }

@@ -31,7 +31,8 @@ def weights(fmt, seed, N, K, std=0.02):
 def check(got, ref, what, max_rel=GATE_MAX_REL, cos=GATE_COS, abs_floor=2.0 ** -14):
     """abs_floor: 2^-14 for fp16 outputs (default; subnormal halfs carry absolute precision), 0 for fp32 outputs."""
     p = O.parity(got, ref, abs_floor)
-    msg = "%s: max_rel=%.3e cos=%.7f max_abs/rms=%.3e" % (what, p["max_rel"], p["cos"], p["max_abs_over_rms"])
+    msg = "%s: max_rel=%.3e cos=%.7f max_abs/rms=%.3e (%d of %d under the 1%%-rms floor, %d under the 2^-14 floor)" % (
+        what, p["max_rel"], p["cos"], p["max_abs_over_rms"], p["n_under_rms_floor"], p["n"], p["n_under_abs_floor"])
     print(msg, flush=True)
     assert np.isfinite(np.asarray(got, np.float64)).all(), what + ": non-finite output"
     assert p["max_rel"] <= max_rel and p["cos"] >= cos, msg

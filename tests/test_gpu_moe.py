@@ -12,14 +12,24 @@ from gpu_util import check, dev, host
 pytestmark = pytest.mark.gpu
 
 
+_EXPERTS = {}
+
+
 def make_experts(fmt, seed, E, N, K):
-    """E experts of [N, K] weights -> (AoS blocks [E, N, row_bytes], SoA planes)."""
-    W = np.stack([O.quantize(fmt, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
-    if fmt == O.MXFP4:
-        qs, sc = O.repack_mxfp4_to_soa(W)
-        return W, qs, sc, N * K // 2, N * K // 32
-    qs, sc = O.repack_q8_0_to_soa(W)
-    return W, qs, sc, N * K, N * K // 32
+    """E experts of [N, K] weights -> (AoS blocks [E, N, row_bytes], SoA planes).  Kept per (fmt, seed, shape): the
+    full-size cases share their banks."""
+    key = (fmt, seed, E, N, K)
+    if key not in _EXPERTS:
+        W = np.stack([O.quantize(fmt, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
+        if fmt == O.MXFP4:
+            qs, sc = O.repack_mxfp4_to_soa(W)
+            _EXPERTS[key] = (W, qs, sc, N * K // 2, N * K // 32)
+        else:
+            qs, sc = O.repack_q8_0_to_soa(W)
+            _EXPERTS[key] = (W, qs, sc, N * K, N * K // 32)
+        if N * K * E < (1 << 24):
+            return _EXPERTS.pop(key)
+    return _EXPERTS[key]
 
 
 def route(seed, T, E, k):
@@ -49,7 +59,7 @@ CHAIN_GATE = 2e-3
 
 
 def ref_gate_up_oai(Wg, Wu, bg, bu, e, xq_row, K, N):
-    """-> (lo, hi) envelope of half(swiglu_oai(g16, u16)) over the admissible roundings of the two
+    """-> (lo, hi, g16, u16): envelope of half(swiglu_oai(g16, u16)) over the admissible roundings of the two
     intermediates: the fp32 device sums may sit on the other side of an fp16 rounding boundary than
     the fp64 oracle sums, and swiglu_oai's (up + 1) factor can amplify that ulp without bound in
     relative terms, so the stage is checked against the set of results the reference chain can
@@ -59,7 +69,30 @@ def ref_gate_up_oai(Wg, Wu, bg, bu, e, xq_row, K, N):
     inf = np.float16(np.inf)
     outs = [f16(O.swiglu_oai_np(gg.astype(np.float32), uu.astype(np.float32)))
             for gg in (np.nextafter(g, -inf), g, np.nextafter(g, inf)) for uu in (np.nextafter(u, -inf), u, np.nextafter(u, inf))]
-    return np.min(outs, axis=0), np.max(outs, axis=0)
+    return np.min(outs, axis=0), np.max(outs, axis=0), g.astype(np.float32), u.astype(np.float32)
+
+
+def ulp16(v):
+    """Spacing of fp16 at |v| (normal range)."""
+    return 2.0 ** (np.floor(np.log2(np.maximum(np.abs(v).astype(np.float64), 2.0 ** -14))) - 10)
+
+
+def explained_outliers(got, centre, budget, what, min_frac):
+    """The envelope says WHETHER every element is a value the reference chain can produce; this says HOW FAR the
+    results sit from the chain evaluated in fp64: the share of elements within the 1e-3 gate is printed and bounded
+    below, and each element beyond the gate must be explained by its own cancellation, i.e. lie within the first-order
+    effect `budget` of one-ulp moves of the fp16 intermediates (large only where z + 1 or acc + bias nearly cancels)."""
+    r = centre.astype(np.float64)
+    rms = float(np.sqrt(np.mean(r * r)))
+    den = np.maximum(np.abs(r), max(1e-2 * rms, 2.0 ** -14))
+    rel = np.abs(got.astype(np.float64) - r) / den
+    out = rel > 1e-3
+    frac = 1.0 - out.mean()
+    worst = float((rel[out] / (budget / den)[out]).max()) if out.any() else 0.0
+    print("%s: %.4f %% of %d elements within 1e-3 of the fp64 chain; %d beyond, largest error / explained budget = %.2f"
+          % (what, 100 * frac, rel.size, int(out.sum()), worst), flush=True)
+    assert frac >= min_frac, (what, frac)
+    assert np.all(rel[out] <= 1.5 * (budget / den)[out]), (what, "an element beyond the gate is not explained by cancellation")
 
 
 def check_envelope(got, lo, hi, what):
@@ -70,10 +103,11 @@ def check_envelope(got, lo, hi, what):
     assert ok.all(), (what, np.argwhere(~ok)[:5], got[~ok][:5], lo[~ok][:5], hi[~ok][:5])
 
 
-@pytest.mark.parametrize("T,H,EF,E,Kt", [(1, 2880, 2880, 32, 4), (3, 512, 320, 6, 2), (32, 704, 384, 8, 4)])
+@pytest.mark.parametrize("T,H,EF,E,Kt", [(1, 2880, 2880, 32, 4), (3, 512, 320, 6, 2), (32, 704, 384, 8, 4), (32, 2880, 2880, 32, 4)])
 def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     """gpt-oss style layer: gate/up (+bias, swiglu_oai) -> quantize -> down (+bias) -> weighted reduce.
-    T=1, H=EF=2880, E=32, top-4 is BASELINE config 4's decode case at full size."""
+    H=EF=2880, E=32, top-4 at T=1 and T=32 are BASELINE config 4's two cases at full size (every packed row of
+    both is recomputed by the oracle)."""
     ops = mx.ops
     Wg, gq, ge, qs_st, e_st = make_experts(O.MXFP4, 100, E, EF, H)
     Wu, uq, ue, _, _ = make_experts(O.MXFP4, 200, E, EF, H)
@@ -89,7 +123,15 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     h_h = host(h).astype(np.float32)
     env = [ref_gate_up_oai(Wg, Wu, bg, bu, ids[t, k], xq[t * rb:(t + 1) * rb], H, EF) for t in range(T) for k in range(Kt)]
     check_envelope(h_h, np.stack([e[0] for e in env]), np.stack([e[1] for e in env]), "moe gate_up swiglu_oai (decode) T=%d" % T)
-    check(h_h, np.stack([(e[0] + e[1]) / 2 for e in env]), "  ... and against the envelope centre", max_rel=1.0, cos=0.99999)
+    g16, u16 = np.stack([e[2] for e in env]).astype(np.float64), np.stack([e[3] for e in env]).astype(np.float64)
+    centre = f16(O.swiglu_oai_np(g16.astype(np.float32), u16.astype(np.float32)))
+    check(h_h, centre, "  ... cosine against the fp64 chain", max_rel=1.0, cos=0.99999)
+    # first-order effect of one-ulp moves of g16 and u16 plus the output's own rounding
+    xg, z = np.minimum(g16, 7.0), np.clip(u16, -7.0, 7.0)
+    sg = 1.0 / (1.0 + np.exp(-1.702 * xg))
+    glu, dglu = xg * sg, np.where(g16 < 7.0, sg * (1.0 + 1.702 * xg * (1.0 - sg)), 0.0)
+    budget = ulp16(g16) * np.abs(dglu) * np.abs(z + 1.0) + np.where(np.abs(u16) < 7.0, ulp16(u16), 0.0) * np.abs(glu) + ulp16(centre)
+    explained_outliers(h_h, centre, budget, "moe gate_up swiglu_oai (decode) T=%d" % T, 0.99)
     hq = ops.quantize_q8_1(h)
     hq_h = host(hq)
     assert np.array_equal(hq_h, O.quantize_q8_1(h_h))
@@ -100,13 +142,17 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     assert np.array_equal(host(out_f), host(out)), "down on fp16 h != quantize + down"
     hrb = EF // 32 * 40
     inf = np.float16(np.inf)
-    lo, hi = [], []
+    lo, hi, ctr, a16s = [], [], [], []
     for s_ in range(T * Kt):   # out = half(half(acc) + bias): envelope over half(acc) moving by one ulp (the sum can cancel)
         a16 = f16(O.gemv_q8chain(O.MXFP4, Wd[ids.ravel()[s_]], hq_h[s_ * hrb:(s_ + 1) * hrb], EF, H)[0]).astype(np.float16)
         c = [f16(v.astype(np.float32) + bd[ids.ravel()[s_]]) for v in (np.nextafter(a16, -inf), a16, np.nextafter(a16, inf))]
         lo.append(np.min(c, axis=0))
         hi.append(np.max(c, axis=0))
+        ctr.append(c[1])
+        a16s.append(a16.astype(np.float32))
     check_envelope(out_h, np.stack(lo), np.stack(hi), "moe down + bias (decode)")
+    ctr = np.stack(ctr)
+    explained_outliers(out_h, ctr, ulp16(np.stack(a16s)) + ulp16(ctr), "moe down + bias (decode) T=%d" % T, 0.99)
     y = torch.zeros((T, H), dtype=torch.float16, device="cuda")
     ident = dev(np.arange(T * Kt, dtype=np.uint32))
     ops.moe_prefill_reduce(out, ident, dev(w.ravel()).half(), y, T, Kt, H)
@@ -238,8 +284,9 @@ def test_moe_decode_kquant_fp16_activations(mx, T, E, Kt, H, EF):
 
 @pytest.mark.parametrize("T,E,Kt,H,EF", [(40, 8, 2, 512, 256), (200, 32, 4, 256, 768)])
 def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
-    """moe_prefill_gate_up_silu_q4k_q8 / _q6k_q8 (block_q8_1x rows) and moe_prefill_down_packed_q4k_q8 /
-    _q6k_q8 (block_q8_1s rows) against the q8-chain oracle, expert by expert."""
+    """moe_prefill_gate_up_silu_q4k_q8 / _q6k_q8 and moe_prefill_down_packed_q4k_q8 / _q6k_q8, all on block_q8_1s rows
+    (the layout the reference kernels read, src/ops/moe_fused.cpp:559-566,672-687), against the q8_1s-chain oracle
+    (min terms on the stored half sums), expert by expert."""
     ops = mx.ops
     mk = lambda F, seed, N, K: np.stack([O.quantize(F, O.normal(seed + e, (N, K), 0.0, 0.02)) for e in range(E)])
     x = f16(O.normal(8600, (T, H)))
@@ -248,8 +295,9 @@ def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
     TK = T * Kt
     counts = np.diff(off.astype(np.int64))
     xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
-    xq = ops.quantize_q8_1(xp)
+    xq = ops.quantize_q8_1s(xp)
     xq_h = host(xq).reshape(TK, -1)
+    assert np.array_equal(xq_h.ravel(), O.quantize_q8_1s(host(xp).astype(np.float32)))
     h_keep = None
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wg, Wu = mk(F, 8700, EF, H), mk(F, 8800, EF, H)
@@ -260,13 +308,13 @@ def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
         for e in range(E):
             if counts[e]:
                 rows = slice(off[e], off[e + 1])
-                g = O.gemv_q8chain(F, Wg[e], xq_h[rows], H, EF)
-                u = O.gemv_q8chain(F, Wu[e], xq_h[rows], H, EF)
+                g = O.gemv_q8schain(F, Wg[e], xq_h[rows], H, EF)
+                u = O.gemv_q8schain(F, Wu[e], xq_h[rows], H, EF)
                 h_ref[rows] = O.swiglu_np(g.astype(np.float32), u.astype(np.float32))
-        check(host(hp).astype(np.float32), h_ref, "grouped gate_up silu %s int-dot" % fmt)
+        check(host(hp).astype(np.float32), h_ref, "grouped gate_up silu %s int-dot (q8_1s rows)" % fmt)
         h_keep = hp
     hq = ops.quantize_q8_1s(h_keep)
-    hq_x = host(ops.quantize_q8_1(h_keep)).reshape(TK, -1)   # same quants and d in the 40-byte layout for the oracle
+    hq_h = host(hq).reshape(TK, -1)
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wd = mk(F, 8900, H, EF)
         op = ops.moe_prefill_down_packed_kquant_q8(fmt, hq, dev(Wd), dev(off), TK, E, H, EF, Wd[0].size)
@@ -276,7 +324,7 @@ def test_moe_grouped_kquant_int_dot(mx, T, E, Kt, H, EF):
         for e in range(E):
             if counts[e]:
                 rows = slice(off[e], off[e + 1])
-                o_ref[rows] = O.gemv_q8chain(F, Wd[e], hq_x[rows], EF, H)
+                o_ref[rows] = O.gemv_q8schain(F, Wd[e], hq_h[rows], EF, H)
         check(host(op).astype(np.float32), o_ref, "grouped down packed %s int-dot (q8_1s rows)" % fmt)
 
 

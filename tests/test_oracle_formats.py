@@ -345,3 +345,121 @@ def test_dp4a_semantics_golden(golden):
     bs = b.view(np.int8).reshape(-1, 4).astype(np.int64)
     assert np.array_equal((ab * bs).sum(axis=1) + 7, golden["dp4a_us"])
     assert np.array_equal((a.view(np.int8).reshape(-1, 4).astype(np.int64) * bs).sum(axis=1) - 3, golden["dp4a_ss"])
+
+
+# ---------------------------------------------------------------- activation epilogues
+def _both_swiglu(g, u):
+    """The C and the numpy restatement of swiglu on the same scalars."""
+    return float(O.swiglu([g], [u])[0]), float(O.swiglu_np(np.float32([g]), np.float32([u]))[0])
+
+
+def _both_oai(g, u, alpha=1.702, limit=7.0):
+    return (float(O._swiglu_oai(float(g), float(u), float(alpha), float(limit))),
+            float(O.swiglu_oai_np(np.float32([g]), np.float32([u]), alpha, limit)[0]))
+
+
+def test_swiglu_known_answers():
+    """swiglu = (g * sigmoid(g)) * u (src/ops/elementwise.cpp:449-466).  Expected values are literals
+    (sigmoid(1) = 0.7310585786300049, ...), not a retyped formula: a dropped factor, sigmoid(-g) for
+    sigmoid(g) or swapped operands each fail one line."""
+    cases = [((0.0, 3.0), 0.0),                        # silu(0) = 0 whatever u
+             ((1.0, 1.0), 0.7310585786300049),          # silu(1)
+             ((1.0, -2.0), -1.4621171572600098),        # linear in u, sign kept
+             ((-1.0, 2.0), -0.5378828427399902),        # silu(-1) = -0.26894142..., not +
+             ((30.0, 0.5), 15.0),                       # large gate: g * u
+             ((-30.0, 1.0), -2.8072868906517896e-12),   # large negative gate: -> -0
+             ((2.0, 0.0), 0.0)]
+    for (g, u), want in cases:
+        for got in _both_swiglu(g, u):
+            assert got == pytest.approx(want, rel=2e-6, abs=1e-18), (g, u, got, want)
+    # not symmetric in its operands
+    assert _both_swiglu(2.0, 1.0)[0] != pytest.approx(_both_swiglu(1.0, 2.0)[0], rel=1e-3)
+
+
+def test_swiglu_oai_known_answers():
+    """swiglu_oai: x = min(gate, limit) (clamped ABOVE only), z = clamp(up, -limit, limit),
+    out = (x * sigmoid(alpha x)) * (z + 1), alpha = 1.702, limit = 7 (src/ops/elementwise.cpp:468-492)."""
+    x7 = 6.999953128303318        # 7 * sigmoid(1.702 * 7)
+    cases = [((8.0, 0.0), x7),                          # gate above the limit -> x = 7 exactly
+             ((7.0, 0.0), x7),
+             ((100.0, 0.0), x7),
+             ((-8.0, 0.0), -9.766428865730381e-06),     # gate below -limit is NOT clamped (clamped would give -4.687e-05)
+             ((8.0, 8.0), x7 * 8.0),                    # up above the limit -> z = 7, factor 8
+             ((8.0, -8.0), x7 * -6.0),                  # up below -limit -> z = -7, factor -6
+             ((8.0, 100.0), x7 * 8.0),
+             ((3.0, -1.0), 0.0),                        # z + 1 = 0
+             ((1.0, 0.0), 0.8457957659328212),          # sigmoid(1.702): pins alpha
+             ((0.5, 1.0), 2 * 0.35038843660638014),     # (z + 1) = 2
+             ((-2.5, 0.5), 1.5 * -0.03498616504857008),
+             ((0.0, 5.0), 0.0)]
+    for (g, u), want in cases:
+        for got in _both_oai(g, u):
+            assert got == pytest.approx(want, rel=2e-6, abs=1e-12), (g, u, got, want)
+    # the one-sided clamp, side by side: a two-sided clamp of the gate would make these two equal
+    lo8, lo7 = _both_oai(-8.0, 0.0)[1], _both_oai(-7.0, 0.0)[1]
+    assert lo7 == pytest.approx(-4.687169668280189e-05, rel=2e-6) and abs(lo8) < 0.25 * abs(lo7)
+    # alpha and limit are arguments, not constants: alpha = 1 gives plain sigmoid, limit = 2 clamps at 2
+    for got in _both_oai(1.0, 0.0, alpha=1.0):
+        assert got == pytest.approx(0.7310585786300049, rel=2e-6)
+    for got in _both_oai(5.0, 9.0, alpha=1.702, limit=2.0):
+        assert got == pytest.approx(2.0 / (1.0 + 0.03324004351101861) * 3.0, rel=2e-6)   # exp(-1.702 * 2) = 0.0332400435110
+
+
+def test_swiglu_c_and_numpy_forms_agree():
+    g, u = O.normal(71, 4000, 0, 6), O.normal(72, 4000, 0, 6)
+    assert np.allclose(O.swiglu(g, u), O.swiglu_np(g, u), rtol=3e-7, atol=0)
+    c = np.float32([O._swiglu_oai(float(a), float(b), 1.702, 7.0) for a, b in zip(g, u)])
+    assert np.allclose(c, O.swiglu_oai_np(g, u), rtol=2e-6, atol=0)   # alpha is a float in C, a double in numpy
+    assert (np.abs(g) > 7).sum() > 100 and (g < -7).sum() > 30 and (np.abs(u) > 7).sum() > 100   # both clamps exercised
+
+
+# ---------------------------------------------------------------- q8_1s chain (stored half sums)
+def _q8s_rows(x):
+    """fp32 rows [T, K] -> (block_q8_1s stream, block_q8_1x stream) of the same quants."""
+    return (np.concatenate([O.quantize_q8_1s(r) for r in x]), np.concatenate([O.quantize_q8_1(r) for r in x]))
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0, O.MXFP4, O.Q4_0))
+def test_q8schain_equals_q8chain_on_quantizer_output(fmt):
+    """The quantizer stores s0 + s1 = d * sum(q) up to fp32 rounding, so both chains give the same sums to ~1e-6."""
+    K, N, T = 512, 24, 3
+    x = O.round_fp16(O.normal(500 + fmt, (T, K)))
+    W = O.quantize(fmt, O.normal(510 + fmt, (N, K), 0, 0.02))
+    xs, xx = _q8s_rows(x)
+    a, b = O.gemv_q8schain(fmt, W, xs, K, N), O.gemv_q8chain(fmt, W, xx, K, N)
+    rms = np.sqrt(np.mean(b * b))
+    assert np.abs(a - b).max() <= 2e-6 * rms, (fmt, np.abs(a - b).max() / rms)
+
+
+def test_q8schain_uses_the_stored_sums():
+    """Doctored sums that no quantizer would write show which field the min term reads."""
+    K, N = 256, 1
+    # Q4_K: every scale 0, every min 1, d = dmin = 1  ->  weight = -1 everywhere, y = -(sum over blocks of s0 + s1)
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[2:4] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[4 + 4:4 + 8] = 1                 # mins of sub-blocks 0..3 (low 6 bits of bytes 4..7)
+    blk[4 + 8:4 + 12] = 1 << 4           # mins of sub-blocks 4..7 (high nibbles of bytes 8..11)
+    assert np.array_equal(O.dequant(O.Q4_K, blk), np.full(256, -1.0, np.float32))
+    xs = np.zeros((8, 48), np.uint8)
+    hdr = np.zeros((8, 4), np.float32)
+    hdr[:, 0] = 0.5                                         # d8 (irrelevant: the scales are 0)
+    hdr[:, 1] = np.arange(8) + 1.0                          # s0 = 1..8
+    hdr[:, 2] = 100.0 * (np.arange(8) + 1.0)                # s1 = 100..800
+    hdr[:, 3] = 1e9                                         # pad: never read
+    xs[:, :16] = hdr.view(np.uint8)
+    xs[:, 16:] = 3                                          # quants: multiplied by scale 0
+    assert O.gemv_q8schain(O.Q4_K, blk, xs.ravel(), K, N)[0, 0] == -(36.0 + 3600.0)
+    # Q6_K: d = 1, every scale 1, all codes 0 (value -32)  ->  y = sum over 16-groups of (d8 * 0 - 32 * s_half)
+    b6 = np.zeros(210, np.uint8)
+    b6[192:208] = 1
+    b6[208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    assert np.array_equal(O.dequant(O.Q6_K, b6), np.full(256, -32.0, np.float32))
+    assert O.gemv_q8schain(O.Q6_K, b6, xs.ravel(), K, N)[0, 0] == -32.0 * (36.0 + 3600.0)
+    # per-group scale indexing: scale 2 on the second half of block 3 only
+    b6[192 + 3 * 2 + 1] = 2
+    assert O.gemv_q8schain(O.Q6_K, b6, xs.ravel(), K, N)[0, 0] == -32.0 * (36.0 + 3600.0 + 400.0)
+    # and the integer part: one quant 1 facing code 0 (u = 0): nothing; code 5 in element 0 of block 0: d8 * 5 * q
+    b6[0] = 5
+    xs[0, 16] = 7
+    assert O.gemv_q8schain(O.Q6_K, b6, xs.ravel(), K, N)[0, 0] == -32.0 * (36.0 + 3600.0 + 400.0) + 0.5 * 5 * 7
