@@ -40,12 +40,17 @@ enum {
     MX_ERR_UNSUPPORTED = 5, /* valid arguments, combination not built */
     MX_ERR_IO = 6,          /* a file could not be opened or mapped (see mx_gguf_last_error) */
     MX_ERR_FORMAT = 7,      /* a file is not what its format prescribes (see mx_gguf_last_error) */
-    MX_ERR_NOT_FOUND = 8    /* no tensor / key of that name */
+    MX_ERR_NOT_FOUND = 8,   /* no tensor / key of that name */
+    MX_ERR_WORKSPACE = 9    /* the workspace passed to a *_ws entry point is smaller than the launch needs */
 };
 
 const char* mx_status_string(int status);
 int mx_last_hip_error(void);  /* hipError_t of the last MX_ERR_LAUNCH on this thread */
 int mx_version(void);
+/* Optional set-up for the current device: resolves the addresses of the library's per-device scratch arrays (see the
+ * batched GEMVs and mx_gemm_* below) so that the first split-K launch does it no more.  Callers that record HIP
+ * graphs call it once per device before capturing; everyone else may leave it to the first launch.  */
+int mx_init(void);
 
 /* Measurement aid, no counterpart in the reference: reads n_bytes (a multiple of 16, 16-byte aligned) once with the
  * launch geometry of the decode GEMV and no arithmetic, so that a GEMV launch can be priced against a pure read of
@@ -143,10 +148,16 @@ int mx_gemv_mxfp4_soa_q8_x2(mx_stream_t s, const void* x_q8, const uint8_t* gate
  *                        in its SoA form; here the GGUF AoS blocks are batched directly)
  * Q8_0 / MXFP4 batched have no reference counterpart (T >= 2 falls to dequant +
  * GEMM there, src/model/qwen35_dense.cpp:811-831).
- * Batched launches with K >= 8192 and N <= 16384 split K over workgroups and keep their partial sums in
- * a 2 MB per-device scratch array owned by the library (nothing is allocated): two such calls that
- * overlap on one device (different streams) would race on it, exactly as calls sharing the reference's
- * static per-device scratch buffers would (src/model/dense_dispatch.hpp:547-560).  */
+ *
+ * Library-owned scratch (no counterpart in the reference's signatures; it is what lets callers that cannot
+ * allocate -- code under HIP graph capture, serving loops, harnesses that forbid hipMalloc -- use these entry
+ * points as they are): batched launches with T >= 2 and K >= 8192 whose row groups alone would leave CUs idle
+ * split K over workgroups and keep slices x T x N fp32 partial sums in a 2 MB file-scope device array (one copy
+ * per device, resolved with hipGetSymbolAddress on first use or by mx_init, never allocated or freed).  Limit:
+ * slices * min(T, 8) * N <= 524288 floats (e.g. T = 8, N = 16384); a launch beyond it runs unsplit.  Every call
+ * on a device shares that device's array: two such calls that overlap on one device (different streams, graph
+ * branches) race on it, exactly as calls sharing the reference's static per-device scratch buffers would
+ * (src/model/dense_dispatch.hpp:547-560).  Callers that overlap launches use the *_ws forms below.  */
 int mx_gemv_q4_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 /* gemv_q4_K_q8s_batched  include/ie/ops.hpp (gemv_q4_K_q8s_batched), src/ops/gemv_q8dot.cpp:483-597: the
  * activation rows are block_q8_1s (48 B, stored half sums s0/s1; 16-byte aligned) from
@@ -159,6 +170,19 @@ int mx_gemv_q6_K_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint
 int mx_gemv_q8_0_q8_batched(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W,
                                 uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* Caller-workspace forms of the batched GEMVs (no counterpart in the reference): identical results, but the split-K
+ * partial sums go to `ws` (16-byte aligned device memory of at least mx_gemv_batched_ws_bytes(K, N, T) bytes, which
+ * is 0 for shapes that never split), so launches on different streams can overlap.  A workspace that is too small
+ * is MX_ERR_WORKSPACE; nothing is launched.  */
+int mx_gemv_batched_ws_bytes(uint32_t K, uint32_t N, uint32_t T, uint64_t* bytes);
+int mx_gemv_q4_K_q8_batched_ws(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T,
+                               void* ws, uint64_t ws_bytes);
+int mx_gemv_q6_K_q8_batched_ws(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T,
+                               void* ws, uint64_t ws_bytes);
+int mx_gemv_q8_0_q8_batched_ws(mx_stream_t s, const void* x_q8, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T,
+                               void* ws, uint64_t ws_bytes);
+int mx_gemv_q8_0_soa_q8_batched_ws(mx_stream_t s, const void* x_q8, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y,
+                                   uint32_t K, uint32_t N, uint32_t T, void* ws, uint64_t ws_bytes);
 /* Fused gate + up for the other int-dot formats: y_a = W_a . x, y_b = W_b . x in one launch, both matrices [N, K].
  * No counterpart of these names in the reference, which fuses gate/up this way for MXFP4 (gemv_mxfp4_soa_q8_x2,
  * include/ie/ops.hpp:503-513) and for Q4_K with fp16 activations (gemv_q4_K_dual_ffn, src/ops/gemv_q4k.cpp:603-612).
@@ -278,9 +302,11 @@ int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uin
  * as dequant_q8_0_soa_to_Bt + gemm_fp16, src/model/qwen35_dense.cpp:811-831).
  * A launch whose 128-token tiles would cover at most half of the CUs (a short batch against a narrow
  * matrix) and whose K is at least 2048 is cut into 2..8 K slices; their fp32 partial sums go through a
- * 16 MB per-device scratch array owned by the library (nothing is allocated) and are added in slice
+ * 16 MB per-device scratch array owned by the library (a file-scope device array resolved with hipGetSymbolAddress,
+ * never allocated; slices * M * N <= 4 Mi floats, fewer slices beyond that) and are added in slice
  * order by a second small launch: two such calls that overlap on one device race on it, as the
- * reference's static per-device scratch buffers would (src/model/dense_dispatch.hpp:547-560).  */
+ * reference's static per-device scratch buffers would (src/model/dense_dispatch.hpp:547-560).  The *_ws forms
+ * below keep the partial sums in the caller's workspace instead.  */
 int mx_gemm_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M,
                      uint32_t K, uint32_t N);
@@ -290,6 +316,19 @@ int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const
  * K % 256 == 0 (Q6_K), K % 128 == 0 (Q8_0); W is the GGUF block stream, 2-byte aligned.  */
 int mx_gemm_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
 int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+/* Caller-workspace forms (no counterpart in the reference): same results; K-sliced launches keep their partial sums
+ * in `ws` (16-byte aligned device memory), so launches on different streams can overlap.  mx_gemm_ws_bytes gives the
+ * size that allows every slice the launch would like (0: the shape is never sliced); a smaller workspace, NULL / 0
+ * included, is legal and means fewer slices or none.  */
+int mx_gemm_ws_bytes(uint32_t M, uint32_t K, uint32_t N, uint64_t* bytes);
+int mx_gemm_q4_K_ws(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, void* ws,
+                    uint64_t ws_bytes);
+int mx_gemm_q6_K_ws(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, void* ws,
+                    uint64_t ws_bytes);
+int mx_gemm_q8_0_ws(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, void* ws,
+                    uint64_t ws_bytes);
+int mx_gemm_q8_0_soa_ws(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M,
+                        uint32_t K, uint32_t N, void* ws, uint64_t ws_bytes);
 /* Q4_0 weights through the same kernel: gemm_q4_0 / gemm_q4_0_xmx  include/ie/ops.hpp:530-534, src/ops/gemv_q4_0.cpp,
  * src/ops/gemm_q4k_xmx.cpp:418-522; K % 128 == 0, W 2-byte aligned.  */
 int mx_gemm_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);

@@ -414,25 +414,34 @@ struct GemmArgs {
     float* y_acc;                     //   and the fp32 [T, N] buffer w * acc is atomically added into (Y unused)
     uint32_t M, K, N, E;
     uint32_t tiles_m, tiles_n;        // dense tile grid; grouped: tiles_m is an upper bound
-    uint32_t k_split;                 // dense only: K slices per output tile (above 1: fp32 partial sums go to g_gemm_splitk_acc)
+    uint32_t k_split;                 // dense only: K slices per output tile (above 1: fp32 partial sums go to split_acc)
+    float* split_acc;                 // [k_split][M][N] partial sums of a K-sliced launch
 };
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
 
 // Dense launches with too few output tiles for the chip (a short batch against a narrow matrix) cut K into up to
-// eight slices: every slice writes its fp32 partial sums to its own plane of this per-device scratch, and a last
-// launch adds the planes in slice order and rounds to fp16 (so the result does not depend on which slice finished
-// first).  Launches that overlap on one device would race on it, as with the reference's static per-device scratch
-// buffers (src/model/dense_dispatch.hpp:547-560).
-constexpr uint32_t kGemmSplitElems = 4u << 20;   // slices * M * N <= 4 Mi partial sums (16 MB)
+// eight slices: every slice writes its fp32 partial sums to its own plane of a scratch buffer, and a last launch adds
+// the planes in slice order and rounds to fp16 (so the result does not depend on which slice finished first).  The
+// scratch is a caller's workspace (the *_ws entry points) or the file-scope device array below, which the library
+// owns (no entry point allocates): one copy per device, keeping the last call's contents; every element the last
+// launch reads was written by the slices in front of it.  Launches that overlap on one device would race on it, as
+// with the reference's static per-device scratch buffers (src/model/dense_dispatch.hpp:547-560).
+constexpr uint64_t kGemmSplitElems = 4ull << 20;   // slices * M * N <= 4 Mi partial sums (16 MB)
 constexpr uint32_t kGemmSplitMax = 8;
-__device__ float g_gemm_splitk_acc[kGemmSplitElems];
+static __device__ __align__(256) float g_gemm_splitk_acc[kGemmSplitElems];
+static std::atomic<void*> g_gemm_splitk_addr[kMaxDevices];
 
-__global__ __launch_bounds__(256) void gemm_splitk_store_kernel(half_t* y, uint32_t n, uint32_t k_split) {
+int gemm_init_device() {
+    void* p = nullptr;
+    return scratch_address(HIP_SYMBOL(g_gemm_splitk_acc), g_gemm_splitk_addr, &p);
+}
+
+__global__ __launch_bounds__(256) void gemm_splitk_store_kernel(half_t* y, const float* acc, uint32_t n, uint32_t k_split) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    float v = g_gemm_splitk_acc[i];
-    for (uint32_t k = 1; k < k_split; ++k) v += g_gemm_splitk_acc[(size_t)k * n + i];
+    float v = acc[i];
+    for (uint32_t k = 1; k < k_split; ++k) v += acc[(size_t)k * n + i];
     y[i] = (half_t)v;
 }
 
@@ -684,7 +693,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
                     if (MODE == GEMM_MOE_DOWN && g.y_acc)
                         __hip_atomic_fetch_add(g.y_acc + (size_t)g.row_token[row] * g.N + n, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     else if (MODE == GEMM_DENSE && g.k_split > 1)
-                        g_gemm_splitk_acc[((size_t)ks * g.M + row) * g.N + n] = o;
+                        g.split_acc[((size_t)ks * g.M + row) * g.N + n] = o;
                     else
                         g.Y[(size_t)row * g.N + n] = (half_t)o;
                 }
@@ -826,19 +835,21 @@ static int gemm_cu_count() {
 // (twice the workgroups; measured: 64 tiles -> +20 %, 224 tiles -> -9 %); everything else runs
 // 128-token tiles.
 template <class QF, int MODE>
-static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
+static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound,
+                       const SplitWs* caller_ws = nullptr) {
     if constexpr (MODE == GEMM_DENSE) {
         const uint64_t cus = (uint64_t)gemm_cu_count();
         const uint64_t tiles128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 255) / 256);
         const uint64_t tiles64 = (uint64_t)((g.M + 63) / 64) * ((g.N + 255) / 256);
         const uint64_t mn = (uint64_t)g.M * g.N, n_chunks = g.K / kBK;
+        const uint64_t cap = caller_ws ? caller_ws->elems : kGemmSplitElems;   // partial sums the scratch holds
         // K slices a tiling could take: until every CU has a workgroup, each slice at least 8 chunks deep, the partial
         // sums within the scratch
         auto slices = [&](uint64_t tiles) {
             uint64_t k = tiles ? cus / tiles : 1;
             if (k > kGemmSplitMax) k = kGemmSplitMax;
             if (k > n_chunks / 8) k = n_chunks / 8;
-            if (k * mn > kGemmSplitElems) k = kGemmSplitElems / mn;
+            if (k * mn > cap) k = cap / mn;
             return k < 1 ? (uint64_t)1 : k;
         };
         bool ni2 = false;
@@ -858,9 +869,16 @@ static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typenam
         if (k_split >= 2) {
             const uint32_t per = (uint32_t)((n_chunks + k_split - 1) / k_split);
             g.k_split = (uint32_t)((n_chunks + per - 1) / per);   // no empty slice
+            if (caller_ws) {
+                g.split_acc = caller_ws->ptr;
+            } else {
+                void* p = nullptr;
+                if (int rc = scratch_address(HIP_SYMBOL(g_gemm_splitk_acc), g_gemm_splitk_addr, &p)) return rc;
+                g.split_acc = static_cast<float*>(p);
+            }
             const int rc = ni2 ? launch_gemm_ni<QF, MODE, 2>(s, b0, b1, g, rows_bound) : launch_gemm_ni<QF, MODE, 4>(s, b0, b1, g, rows_bound);
             if (rc != MX_OK) return rc;
-            hipLaunchKernelGGL(gemm_splitk_store_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, as_stream(s), g.Y, (uint32_t)mn, g.k_split);
+            hipLaunchKernelGGL(gemm_splitk_store_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, as_stream(s), g.Y, g.split_acc, (uint32_t)mn, g.k_split);
             return launch_status();
         }
         if (ni2) return launch_gemm_ni<QF, MODE, 2>(s, b0, b1, g, rows_bound);
@@ -896,6 +914,36 @@ static int moe_gemm_aos(mx_stream_t s, const uint16_t* rows, const void* W0, con
     return launch_gemm<QF, MODE>(s, b0, b1, g, total_rows);
 }
 
+// Dense entry points.  ws = NULL: K-sliced launches keep their partial sums in the library's per-device scratch.
+template <class QF>
+static int gemm_dense_aos(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, uint32_t k_align,
+                          uint32_t w_align, uint32_t row_bytes, const SplitWs* ws) {
+    if (int rc = check_gemm(A, W, y, M, K, N, k_align, w_align)) return rc;
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
+    typename QF::Bank b{static_cast<const uint8_t*>(W), 0, row_bytes};
+    return launch_gemm<QF, GEMM_DENSE>(s, b, b, g, M, ws);
+}
+static int gemm_dense_q8_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K,
+                             uint32_t N, const SplitWs* ws) {
+    if (int rc = check_gemm(A, qs_W, y, M, K, N, 128)) return rc;
+    MX_REQUIRE_PTR(d_W);
+    MX_REQUIRE_ALIGN(d_W, 4);
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
+    GemmQ8Soa::Bank b{qs_W, d_W, 0, 0, K};
+    return launch_gemm<GemmQ8Soa, GEMM_DENSE>(s, b, b, g, M, ws);
+}
+// A caller's workspace: any size is accepted, the number of K slices adapts to what it holds (none below 2 M N floats).
+static int gemm_ws(void* ws, uint64_t ws_bytes, SplitWs* out) {
+    if (ws_bytes) {
+        MX_REQUIRE_PTR(ws);
+        MX_REQUIRE_ALIGN(ws, 16);
+    }
+    *out = SplitWs{static_cast<float*>(ws), ws_bytes / 4, true};
+    return MX_OK;
+}
+
 }  // namespace mxq
 
 using namespace mxq;
@@ -903,45 +951,50 @@ using namespace mxq;
 extern "C" {
 
 int mx_gemm_q4_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
-    if (int rc = check_gemm(A, W, y, M, K, N, 256)) return rc;
-    GemmArgs g{};
-    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
-    GemmQ4K::Bank b{static_cast<const uint8_t*>(W), 0, K / 256 * (uint32_t)kQ4KBytes};
-    return launch_gemm<GemmQ4K, GEMM_DENSE>(s, b, b, g, M);
+    return gemm_dense_aos<GemmQ4K>(s, A, W, y, M, K, N, 256, 16, K / 256 * (uint32_t)kQ4KBytes, nullptr);
 }
-
 int mx_gemm_q6_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
-    if (int rc = check_gemm(A, W, y, M, K, N, 256, 2)) return rc;
-    GemmArgs g{};
-    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
-    GemmQ6K::Bank b{static_cast<const uint8_t*>(W), 0, K / 256 * (uint32_t)kQ6KBytes};
-    return launch_gemm<GemmQ6K, GEMM_DENSE>(s, b, b, g, M);
+    return gemm_dense_aos<GemmQ6K>(s, A, W, y, M, K, N, 256, 2, K / 256 * (uint32_t)kQ6KBytes, nullptr);
 }
-
 int mx_gemm_q8_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
-    if (int rc = check_gemm(A, W, y, M, K, N, 128, 2)) return rc;
-    GemmArgs g{};
-    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
-    GemmQ8Aos::Bank b{static_cast<const uint8_t*>(W), 0, K / 32 * (uint32_t)kQ8_0Bytes};
-    return launch_gemm<GemmQ8Aos, GEMM_DENSE>(s, b, b, g, M);
+    return gemm_dense_aos<GemmQ8Aos>(s, A, W, y, M, K, N, 128, 2, K / 32 * (uint32_t)kQ8_0Bytes, nullptr);
 }
-
 int mx_gemm_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
-    if (int rc = check_gemm(A, W, y, M, K, N, 128, 2)) return rc;
-    GemmArgs g{};
-    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
-    GemmQ40::Bank b{static_cast<const uint8_t*>(W), 0, K / 32 * 18u};
-    return launch_gemm<GemmQ40, GEMM_DENSE>(s, b, b, g, M);
+    return gemm_dense_aos<GemmQ40>(s, A, W, y, M, K, N, 128, 2, K / 32 * 18u, nullptr);
+}
+int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    return gemm_dense_q8_soa(s, A, qs_W, d_W, y, M, K, N, nullptr);
 }
 
-int mx_gemm_q8_0_soa(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
-    if (int rc = check_gemm(A, qs_W, y, M, K, N, 128)) return rc;
-    MX_REQUIRE_PTR(d_W);
-    MX_REQUIRE_ALIGN(d_W, 4);
-    GemmArgs g{};
-    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
-    GemmQ8Soa::Bank b{qs_W, d_W, 0, 0, K};
-    return launch_gemm<GemmQ8Soa, GEMM_DENSE>(s, b, b, g, M);
+// ---- caller-workspace forms: K-sliced launches keep their partial sums in `ws`, so calls on different streams can overlap
+int mx_gemm_ws_bytes(uint32_t M, uint32_t K, uint32_t N, uint64_t* bytes) {
+    MX_REQUIRE_PTR(bytes);
+    MX_REQUIRE_SHAPE(M > 0 && K > 0 && N > 0);
+    // K is sliced only when the 128-token tiles cover at most half of the CUs; then up to kGemmSplitMax planes of M x N floats
+    const uint64_t tiles128 = (uint64_t)((M + 127) / 128) * ((N + 255) / 256);
+    *bytes = (2 * tiles128 <= (uint64_t)gemm_cu_count() && K / kBK >= 16) ? (uint64_t)kGemmSplitMax * M * N * sizeof(float) : 0;
+    return MX_OK;
+}
+int mx_gemm_q4_K_ws(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, void* ws, uint64_t ws_bytes) {
+    SplitWs w;
+    if (int rc = gemm_ws(ws, ws_bytes, &w)) return rc;
+    return gemm_dense_aos<GemmQ4K>(s, A, W, y, M, K, N, 256, 16, K / 256 * (uint32_t)kQ4KBytes, &w);
+}
+int mx_gemm_q6_K_ws(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, void* ws, uint64_t ws_bytes) {
+    SplitWs w;
+    if (int rc = gemm_ws(ws, ws_bytes, &w)) return rc;
+    return gemm_dense_aos<GemmQ6K>(s, A, W, y, M, K, N, 256, 2, K / 256 * (uint32_t)kQ6KBytes, &w);
+}
+int mx_gemm_q8_0_ws(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, void* ws, uint64_t ws_bytes) {
+    SplitWs w;
+    if (int rc = gemm_ws(ws, ws_bytes, &w)) return rc;
+    return gemm_dense_aos<GemmQ8Aos>(s, A, W, y, M, K, N, 128, 2, K / 32 * (uint32_t)kQ8_0Bytes, &w);
+}
+int mx_gemm_q8_0_soa_ws(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N,
+                        void* ws, uint64_t ws_bytes) {
+    SplitWs w;
+    if (int rc = gemm_ws(ws, ws_bytes, &w)) return rc;
+    return gemm_dense_q8_soa(s, A, qs_W, d_W, y, M, K, N, &w);
 }
 
 int mx_moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,

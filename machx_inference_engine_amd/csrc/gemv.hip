@@ -261,20 +261,38 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, O
     }
 }
 
-// Batched launches with long rows and few of them (T >= 2, K >= 8192, N <= 16384: the down projections in
-// a speculative-verify batch): the row-group grid alone leaves CUs idle and every workgroup restages
-// several activation tiles.  Here the grid is (row groups, K slices): a workgroup stages one slice once and
-// writes its partial sums to a per-device scratch plane; a second, tiny launch adds the slices in slice
-// order and writes y.  (A single launch with a last-arriver reduction needs device-scope fences, which on
-// this part write back the XCD's L2: measured five times slower than the two launches.)
-// The scratch is a file-scope device array: launches that overlap on one device would race on it (as the
-// reference's static per-device scratch buffers do, src/model/dense_dispatch.hpp:547-560).
-constexpr uint32_t kSplitMaxN = 16384, kSplitMaxT = 8, kSplitMaxSlices = 4;
-__device__ float g_splitk_part[kSplitMaxSlices][kSplitMaxT][kSplitMaxN];
+// Batched launches with long rows and few of them (T >= 2, K >= 8192: the down projections in a speculative-verify
+// batch): the row-group grid alone leaves CUs idle and every workgroup restages several activation tiles.  Here
+// the grid is (row groups, K slices): a workgroup stages one slice once and writes its partial sums to a scratch
+// plane, part[(slice * T + t) * N + row]; a second, tiny launch adds the slices in slice order and writes y.  (A
+// single launch with a last-arriver reduction needs device-scope fences, which on this part write back the XCD's
+// L2: measured five times slower than the two launches.)
+// The scratch is either a workspace the caller passes (the *_ws entry points) or the file-scope device array below,
+// which the library owns: no entry point allocates.  The array exists once per device and keeps the last call's
+// contents; every element a reduction reads was written by the split launch in front of it, so nothing needs
+// clearing, but two calls that overlap on one device (different streams, graph branches) would race on it, as calls
+// sharing the reference's static per-device scratch buffers do (src/model/dense_dispatch.hpp:547-560).
+constexpr uint32_t kSplitMaxSlices = 4;
+constexpr uint64_t kSplitElems = 4ull * 8 * 16384;   // 2 MB: four slices of eight tokens of 16384 rows
+static __device__ __align__(256) float g_splitk_part[kSplitElems];
+static std::atomic<void*> g_splitk_addr[kMaxDevices];
+
+int gemv_init_device() {
+    void* p = nullptr;
+    return scratch_address(HIP_SYMBOL(g_splitk_part), g_splitk_addr, &p);
+}
+
+// the library-owned scratch of the current device as a SplitWs
+static int static_split_ws(SplitWs* ws) {
+    void* p = nullptr;
+    if (int rc = scratch_address(HIP_SYMBOL(g_splitk_part), g_splitk_addr, &p)) return rc;
+    *ws = SplitWs{static_cast<float*>(p), kSplitElems, false};
+    return MX_OK;
+}
 
 template <class F, int T, int R, int G>
-__global__ __launch_bounds__(kGemvThreads) void gemv_q8_splitk_kernel(typename F::W w, const uint8_t* xq8, uint32_t K, uint32_t N, uint32_t KS,
-                                                                       uint32_t T_real, uint32_t q8_split) {
+__global__ __launch_bounds__(kGemvThreads) void gemv_q8_splitk_kernel(typename F::W w, const uint8_t* xq8, float* part, uint32_t K, uint32_t N,
+                                                                       uint32_t KS, uint32_t T_real, uint32_t q8_split) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int GROUPS = 64 / G;
     constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
@@ -301,16 +319,17 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_splitk_kernel(typename F
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const float v = group_sum<G>(acc[r][t]);
-            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N) g_splitk_part[ks][t][row0 + r] = v;
+            if (lane == (uint32_t)group_sum_lane<G>(lane) && row0 + r < N && (uint32_t)t < T_real)
+                part[((size_t)ks * T_real + t) * N + row0 + r] = v;
         }
 }
 
 template <class OutT>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(OutT* y, const float* bias, uint32_t N, uint32_t T_real, uint32_t n_split) {
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(OutT* y, const float* bias, const float* part, uint32_t N, uint32_t T_real, uint32_t n_split) {
     const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
     if (row >= N || t >= T_real) return;
     float v = 0.f;
-    for (uint32_t k = 0; k < n_split; ++k) v += g_splitk_part[k][t][row];
+    for (uint32_t k = 0; k < n_split; ++k) v += part[((size_t)k * T_real + t) * N + row];
     if (bias) v += bias[row];
     store_out(y + (size_t)t * N + row, v);
 }
@@ -502,7 +521,7 @@ static uint32_t pick_group(uint32_t units) {
 
 template <class F, int T, int G, class OutT>
 static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8,
-                        uint32_t K, uint32_t N, uint32_t T_real, bool split) {
+                        uint32_t K, uint32_t N, uint32_t T_real, bool split, const SplitWs& ws) {
     // GGUF Q8_0 blocks are 17 dword loads per unit: one unit in flight (measured at T = 1 against two: K = 4096,
     // N = 14336 18.1 -> 15.8 us; K = 14336, N = 4096 18.1 -> 16.6 us)
     constexpr int R = GemvShape<T, F::SUM_GRAN>::R, U = std::is_same<F, FmtQ8Aos>::value ? 1 : GemvShape<T, F::SUM_GRAN>::U;
@@ -526,17 +545,22 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     }
     if constexpr (T >= 2) {
         const uint32_t cus = (uint32_t)cu_count();
-        if (nseg == 1 && K >= 8192 && N <= kSplitMaxN && (n_tiles > 1 || n_rg < 2u * cus)) {
+        if (nseg == 1 && K >= 8192 && (n_tiles > 1 || n_rg < 2u * cus)) {
             uint32_t n_split = (4u * cus + n_rg - 1) / n_rg;   // about four workgroups per CU
             if (n_split < n_tiles) n_split = n_tiles;
             if (n_split > kSplitMaxSlices) n_split = kSplitMaxSlices;
             const uint32_t KS = (K256 + n_split - 1) / n_split * 256;
             n_split = (K + KS - 1) / KS;
             if (n_split >= 2 && KS <= KT_max) {
-                hipLaunchKernelGGL((gemv_q8_splitk_kernel<F, T, R, G>), dim3(n_rg, n_split), dim3(kGemvThreads), act_tile_bytes(T, KS, F::SUM_GRAN), st,
-                                   s0.w, xq8, K, N, KS, T_real, split ? 1u : 0u);
-                hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((N + 255) / 256, T_real), dim3(256), 0, st, s0.y, s0.bias, N, T_real, n_split);
-                return launch_status();
+                const bool fits = ws.ptr && (uint64_t)n_split * T_real * N <= ws.elems;
+                if (!fits && ws.caller) return MX_ERR_WORKSPACE;   // a caller's workspace is never silently bypassed
+                if (fits) {
+                    hipLaunchKernelGGL((gemv_q8_splitk_kernel<F, T, R, G>), dim3(n_rg, n_split), dim3(kGemvThreads), act_tile_bytes(T, KS, F::SUM_GRAN),
+                                       st, s0.w, xq8, ws.ptr, K, N, KS, T_real, split ? 1u : 0u);
+                    hipLaunchKernelGGL((splitk_reduce_kernel<OutT>), dim3((N + 255) / 256, T_real), dim3(256), 0, st, s0.y, s0.bias, ws.ptr, N, T_real,
+                                       n_split);
+                    return launch_status();
+                }
             }
         }
     }
@@ -561,16 +585,16 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
 
 template <class F, int G, class OutT>
 static int launch_q8_g(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg<F, OutT>& s1, int nseg, const uint8_t* xq8, uint32_t K,
-                       uint32_t N, uint32_t T, bool split) {
+                       uint32_t N, uint32_t T, bool split, const SplitWs& ws) {
     switch (T) {
-        case 1: return launch_q8_tg<F, 1, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
-        case 2: return launch_q8_tg<F, 2, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
-        case 3: return launch_q8_tg<F, 3, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
-        case 4: return launch_q8_tg<F, 4, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
+        case 1: return launch_q8_tg<F, 1, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split, ws);
+        case 2: return launch_q8_tg<F, 2, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split, ws);
+        case 3: return launch_q8_tg<F, 3, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split, ws);
+        case 4: return launch_q8_tg<F, 4, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split, ws);
         case 5:
-        case 6: return launch_q8_tg<F, 6, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
+        case 6: return launch_q8_tg<F, 6, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split, ws);
         case 7:
-        case 8: return launch_q8_tg<F, 8, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split);
+        case 8: return launch_q8_tg<F, 8, G, OutT>(st, s0, s1, nseg, xq8, K, N, T, split, ws);
     }
     return MX_ERR_SHAPE;
 }
@@ -578,18 +602,22 @@ static int launch_q8_g(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg
 // T up to 16: passes of at most 8 tokens.
 template <class F, class OutT>
 static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, int nseg, const void* xq8, uint32_t K, uint32_t N, uint32_t T,
-                     bool split = false) {
+                     bool split = false, const SplitWs* caller_ws = nullptr) {
     const uint8_t* x = static_cast<const uint8_t*>(xq8);
     const uint32_t G = pick_group((K + 63) / 64);
+    SplitWs ws{nullptr, 0, false};
+    if (caller_ws) ws = *caller_ws;
+    else if (T >= 2 && nseg == 1 && K >= 8192)   // the only launches that may split K
+        if (int rc = static_split_ws(&ws)) return rc;
     for (uint32_t t0 = 0; t0 < T; t0 += 8) {
         const uint32_t tn = (T - t0 < 8) ? T - t0 : 8;
         GemvSeg<F, OutT> a = s0, b = s1;
         a.y = s0.y + (size_t)t0 * N;
         if (nseg > 1) b.y = s1.y + (size_t)t0 * N;
         const uint8_t* xt = x + (size_t)t0 * (K / 32) * (split ? kQ81sBytes : kQ81xBytes);
-        const int rc = (G == 16)   ? launch_q8_g<F, 16, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split)
-                       : (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split)
-                                   : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split);
+        const int rc = (G == 16)   ? launch_q8_g<F, 16, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split, ws)
+                       : (G == 32) ? launch_q8_g<F, 32, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split, ws)
+                                   : launch_q8_g<F, 64, OutT>(as_stream(s), a, b, nseg, xt, K, N, tn, split, ws);
         if (rc != MX_OK) return rc;
     }
     return MX_OK;
@@ -604,7 +632,8 @@ static int check_common(const void* x, const void* y, uint32_t K, uint32_t N, ui
 }
 
 template <class OutT>
-static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, OutT* y, uint32_t K, uint32_t N, uint32_t T, bool split = false) {
+static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, OutT* y, uint32_t K, uint32_t N, uint32_t T, bool split = false,
+                       const SplitWs* ws = nullptr) {
     const uint32_t k_align = fmt == 0 ? 32 : 256;
     if (int rc = check_common(xq8, y, K, N, T, k_align)) return rc;
     MX_REQUIRE_PTR(W);
@@ -613,14 +642,14 @@ static int gemv_aos_q8(int fmt, mx_stream_t s, const void* xq8, const void* W, O
     const uint8_t* base = static_cast<const uint8_t*>(W);
     if (fmt == 1) {
         GemvSeg<FmtQ4K, OutT> g{{base, K / 256 * (uint32_t)kQ4KBytes}, y, nullptr};
-        return launch_q8<FmtQ4K, OutT>(s, g, g, 1, xq8, K, N, T, split);
+        return launch_q8<FmtQ4K, OutT>(s, g, g, 1, xq8, K, N, T, split, ws);
     }
     if (fmt == 2) {
         GemvSeg<FmtQ6K, OutT> g{{base, K / 256 * (uint32_t)kQ6KBytes}, y, nullptr};
-        return launch_q8<FmtQ6K, OutT>(s, g, g, 1, xq8, K, N, T, split);
+        return launch_q8<FmtQ6K, OutT>(s, g, g, 1, xq8, K, N, T, split, ws);
     }
     GemvSeg<FmtQ8Aos, OutT> g{{base, K / 32 * (uint32_t)kQ8_0Bytes}, y, nullptr};
-    return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T, split);
+    return launch_q8<FmtQ8Aos, OutT>(s, g, g, 1, xq8, K, N, T, split, ws);
 }
 
 template <class F, class ActT, class OutT, int EPI = FACT_STORE>
@@ -798,8 +827,8 @@ int mx_gemv_q8_0_q8_f32(mx_stream_t s, const void* x, const void* W, float* y, u
     return gemv_aos_q8<float>(0, s, x, W, y, K, N, 1);
 }
 
-int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K,
-                                uint32_t N, uint32_t T) {
+static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K, uint32_t N,
+                                 uint32_t T, const SplitWs* ws) {
     if (int rc = check_common(x, y, K, N, T, 32)) return rc;
     MX_REQUIRE_PTR(qs_W);
     MX_REQUIRE_PTR(d_W);
@@ -807,7 +836,54 @@ int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x, const int8_t* qs_W
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
     GemvSeg<FmtQ8Soa, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
-    return launch_q8<FmtQ8Soa, half_t>(s, g, g, 1, x, K, N, T);
+    return launch_q8<FmtQ8Soa, half_t>(s, g, g, 1, x, K, N, T, false, ws);
+}
+int mx_gemv_q8_0_soa_q8_batched(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K,
+                                uint32_t N, uint32_t T) {
+    return gemv_q8_0_soa_batched(s, x, qs_W, d_W, y, K, N, T, nullptr);
+}
+
+// ---- caller-workspace forms of the batched GEMVs: the split-K partial sums go to `ws` instead of the library's
+// per-device scratch, so calls on different streams can overlap.  ws_bytes below mx_gemv_batched_ws_bytes(K, N, T)
+// is MX_ERR_WORKSPACE; a shape that never splits K (the query returns 0) ignores the workspace.
+static int check_ws(const void* ws, uint64_t ws_bytes, uint32_t K, uint32_t N, uint32_t T, SplitWs* out) {
+    uint64_t need = 0;
+    if (int rc = mx_gemv_batched_ws_bytes(K, N, T, &need)) return rc;
+    if (need) {
+        MX_REQUIRE_PTR(ws);
+        MX_REQUIRE_ALIGN(ws, 16);
+        if (ws_bytes < need) return MX_ERR_WORKSPACE;
+    }
+    *out = SplitWs{static_cast<float*>(const_cast<void*>(ws)), ws_bytes / 4, true};
+    return MX_OK;
+}
+int mx_gemv_batched_ws_bytes(uint32_t K, uint32_t N, uint32_t T, uint64_t* bytes) {
+    MX_REQUIRE_PTR(bytes);
+    MX_REQUIRE_SHAPE(K > 0 && N > 0 && T >= 1 && T <= 16);
+    // an upper bound over every format and device: up to kSplitMaxSlices slices of a pass of at most 8 tokens
+    *bytes = (T >= 2 && K >= 8192) ? (uint64_t)kSplitMaxSlices * (T < 8 ? T : 8) * N * sizeof(float) : 0;
+    return MX_OK;
+}
+int mx_gemv_q8_0_soa_q8_batched_ws(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K, uint32_t N,
+                                   uint32_t T, void* ws, uint64_t ws_bytes) {
+    SplitWs w;
+    if (int rc = check_ws(ws, ws_bytes, K, N, T, &w)) return rc;
+    return gemv_q8_0_soa_batched(s, x, qs_W, d_W, y, K, N, T, &w);
+}
+static int gemv_aos_batched_ws(int fmt, mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T, void* ws,
+                               uint64_t ws_bytes) {
+    SplitWs w;
+    if (int rc = check_ws(ws, ws_bytes, K, N, T, &w)) return rc;
+    return gemv_aos_q8<half_t>(fmt, s, x, W, reinterpret_cast<half_t*>(y), K, N, T, false, &w);
+}
+int mx_gemv_q4_K_q8_batched_ws(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T, void* ws, uint64_t ws_bytes) {
+    return gemv_aos_batched_ws(1, s, x, W, y, K, N, T, ws, ws_bytes);
+}
+int mx_gemv_q6_K_q8_batched_ws(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T, void* ws, uint64_t ws_bytes) {
+    return gemv_aos_batched_ws(2, s, x, W, y, K, N, T, ws, ws_bytes);
+}
+int mx_gemv_q8_0_q8_batched_ws(mx_stream_t s, const void* x, const void* W, uint16_t* y, uint32_t K, uint32_t N, uint32_t T, void* ws, uint64_t ws_bytes) {
+    return gemv_aos_batched_ws(0, s, x, W, y, K, N, T, ws, ws_bytes);
 }
 int mx_gemv_q8_0_soa_q8(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K, uint32_t N) {
     return mx_gemv_q8_0_soa_q8_batched(s, x, qs_W, d_W, y, K, N, 1);

@@ -18,12 +18,18 @@ const char* mx_status_string(int status) {
         case MX_ERR_IO: return "file could not be opened or mapped";
         case MX_ERR_FORMAT: return "file violates its format";
         case MX_ERR_NOT_FOUND: return "no entry of that name";
+        case MX_ERR_WORKSPACE: return "workspace smaller than this launch needs (see the *_ws_bytes query)";
     }
     return "unknown status";
 }
 
 int mx_last_hip_error(void) { return mxq::g_last_hip_error; }
 
-int mx_version(void) { return 100; }
+int mx_version(void) { return 110; }
+
+int mx_init(void) {
+    if (int rc = mxq::gemv_init_device()) return rc;
+    return mxq::gemm_init_device();
+}
 
 }  // extern "C"

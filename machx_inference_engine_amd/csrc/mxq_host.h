@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mxq.h"
 
 namespace mxq {
@@ -23,6 +25,43 @@ inline int launch_status() {
 }
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// Partial-sum scratch of a split-K launch: either the library's own file-scope device array (resolved per device,
+// see scratch_address) or a workspace the caller passed to a *_ws entry point.
+struct SplitWs {
+    float* ptr;        // device address
+    uint64_t elems;    // capacity in floats
+    bool caller;       // caller-owned: a launch that does not fit is an error instead of falling back to the unsplit kernel
+};
+
+// Device address of a file-scope __device__ array.  In host code the array's name is only a stand-in for the symbol:
+// every device holds its own copy at its own address, which hipGetSymbolAddress returns for the CURRENT device.  The
+// address is resolved once per device and kept in `slot` (one per array, indexed by device ordinal).
+constexpr int kMaxDevices = 64;
+template <class Sym>
+inline int scratch_address(const Sym& symbol, std::atomic<void*> (&slot)[kMaxDevices], void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        g_last_hip_error = (int)(e != hipSuccess ? e : hipErrorInvalidDevice);
+        return MX_ERR_LAUNCH;
+    }
+    void* p = slot[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, symbol);
+        if (e != hipSuccess || !p) {
+            g_last_hip_error = (int)(e != hipSuccess ? e : hipErrorInvalidSymbol);
+            return MX_ERR_LAUNCH;
+        }
+        slot[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return MX_OK;
+}
+
+// per-device set-up of the translation units that own scratch arrays (mx_init)
+int gemv_init_device();
+int gemm_init_device();
 
 }  // namespace mxq
 

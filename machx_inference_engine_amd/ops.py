@@ -161,6 +161,48 @@ def gemv_q8_0_soa_q8_batched(x_q8, qs_W, d_W, K, N, T, y=None):
     return _gemv_q8("mx_gemv_q8_0_soa_q8_batched", x_q8, (_u8(qs_W), _ptr(d_W)), K, N, T, y)
 
 
+def init():
+    """Resolve the library's per-device scratch addresses for the current device (optional; see mx_init)."""
+    rc = lib.mx_init()
+    if rc != 0:
+        raise MxError("mx_init", rc)
+
+
+def gemv_batched_ws_bytes(K, N, T):
+    import ctypes
+    n = ctypes.c_uint64(0)
+    rc = lib.mx_gemv_batched_ws_bytes(K, N, T, ctypes.addressof(n))
+    if rc != 0:
+        raise MxError("mx_gemv_batched_ws_bytes", rc)
+    return n.value
+
+
+def gemm_ws_bytes(M, K, N):
+    import ctypes
+    n = ctypes.c_uint64(0)
+    rc = lib.mx_gemm_ws_bytes(M, K, N, ctypes.addressof(n))
+    if rc != 0:
+        raise MxError("mx_gemm_ws_bytes", rc)
+    return n.value
+
+
+def gemv_q8_batched_ws(fmt, x_q8, wargs, K, N, T, ws, y=None):
+    """Caller-workspace batched GEMV: fmt in ('q4_K', 'q6_K', 'q8_0', 'q8_0_soa'); wargs = weight tensors in C-ABI order;
+    ws = a device tensor of at least gemv_batched_ws_bytes(K, N, T) bytes (or None when that is 0)."""
+    y = _out(y, (T, N), torch.float16, x_q8)
+    _call("mx_gemv_%s_q8_batched_ws" % fmt, _u8(x_q8), *[_ptr(w) for w in wargs], _ptr(y), K, N, T, _ptr(ws) if ws is not None else None,
+          ws.numel() * ws.element_size() if ws is not None else 0)
+    return y
+
+
+def gemm_ws(fmt, A, wargs, M, K, N, ws, y=None):
+    """Caller-workspace dense quant-GEMM: fmt in ('q4_K', 'q6_K', 'q8_0', 'q8_0_soa')."""
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_%s_ws" % fmt, _f16(A), *[_ptr(w) for w in wargs], _ptr(y), M, K, N, _ptr(ws) if ws is not None else None,
+          ws.numel() * ws.element_size() if ws is not None else 0)
+    return y
+
+
 def gemv_mxfp4_soa_q8_batched(x_q8, qs_plane, e_plane, K, N, T, y=None):
     return _gemv_q8("mx_gemv_mxfp4_soa_q8_batched", x_q8, (_u8(qs_plane), _u8(e_plane)), K, N, T, y)
 

@@ -61,3 +61,26 @@ def test_argument_validation_without_gpu(lib):
     assert l.mx_repack_mxfp4_to_soa(blk.ctypes.data, 3, qs.ctypes.data, e.ctypes.data) == OK
     assert e.tolist() == [0, 17, 34] and qs[:16].tolist() == list(range(1, 17))
     assert l.mx_repack_mxfp4_to_soa(None, 3, qs.ctypes.data, e.ctypes.data) == NULL
+
+
+def test_workspace_forms_validate_before_any_hip_call(lib):
+    """The *_ws entry points: size query, NULL / misaligned / too-small workspace."""
+    l, _ = lib
+    OK, NULL, SHAPE, ALIGN, WORKSPACE = 0, 1, 2, 3, 9
+    p16 = 0x1000
+    n = C.c_uint64(7)
+    assert l.mx_gemv_batched_ws_bytes(14336, 4096, 8, C.addressof(n)) == OK and n.value == 4 * 8 * 4096 * 4
+    assert l.mx_gemv_batched_ws_bytes(14336, 4096, 16, C.addressof(n)) == OK and n.value == 4 * 8 * 4096 * 4   # passes of 8 tokens
+    assert l.mx_gemv_batched_ws_bytes(4096, 14336, 8, C.addressof(n)) == OK and n.value == 0                    # short rows never split
+    assert l.mx_gemv_batched_ws_bytes(14336, 4096, 1, C.addressof(n)) == OK and n.value == 0
+    assert l.mx_gemv_batched_ws_bytes(14336, 4096, 8, None) == NULL
+    assert l.mx_gemv_batched_ws_bytes(14336, 4096, 17, C.addressof(n)) == SHAPE
+    need = 4 * 8 * 4096 * 4
+    assert l.mx_gemv_q8_0_soa_q8_batched_ws(None, p16, p16, p16, p16, 14336, 4096, 8, None, need) == NULL
+    assert l.mx_gemv_q8_0_soa_q8_batched_ws(None, p16, p16, p16, p16, 14336, 4096, 8, 0x1004, need) == ALIGN
+    assert l.mx_gemv_q8_0_soa_q8_batched_ws(None, p16, p16, p16, p16, 14336, 4096, 8, p16, need - 4) == WORKSPACE
+    assert l.mx_gemv_q6_K_q8_batched_ws(None, p16, p16, p16, 14336, 4096, 8, p16, 16) == WORKSPACE
+    assert l.mx_status_string(WORKSPACE).startswith(b"workspace")
+    assert l.mx_gemm_ws_bytes(128, 14336, 4096, None) == NULL
+    assert l.mx_gemm_q4_K_ws(None, p16, p16, p16, 128, 14336, 4096, None, 64) == NULL
+    assert l.mx_gemm_q4_K_ws(None, p16, p16, p16, 128, 14336, 4096, 0x1004, 64) == ALIGN
