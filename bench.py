@@ -13,8 +13,11 @@ before the timed region.
 
 Prints ONE JSON line: the metric is achieved HBM GB/s on algorithmic bytes
 (weights once + q8 activations + fp16 outputs).  `roofline` prices the dominant
-kernel against the 8 TB/s HBM peak; `cpu_baseline` times the reference's CPU
-path (dequant to fp32 + scalar fp32 dot, restated in oracle/) on the host cores.
+GEMV kernel against the 8 TB/s HBM peak, `roofline_gemm` the prefill quant-GEMM at
+T = 2048 (BASELINE config 3) against the 2.5 PFLOP/s dense fp16 MFMA peak;
+`cpu_baseline` times the reference's CPU path (dequant to fp32 + scalar fp32 dot,
+restated in oracle/) on the host cores.  Every weight is a seeded N(0, 0.02) tensor
+quantized in HBM (machx_inference_engine_amd.synth), every activation N(0, 1).
 """
 import argparse
 import json
@@ -47,6 +50,9 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="distinct weight sets rotated through (331.7 MB each)")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: a few launches of the dominant kernels and of a plain copy of known size, no timing")
+    ap.add_argument("--shape", default=None, metavar="KIND:T:K:N",
+                    help="profiling aid: only launches of one kernel at one shape (KIND in gemm_q4_K, gemv_q8_0_soa, gemv_q6_K, gemv_q4_K), "
+                         "so that a rocprofv3 run holds exactly one (kernel, shape) pair; prints its HIP-event average")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures one GPU only (the path is data-parallel over output rows / experts, "
@@ -63,6 +69,58 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
 
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    MFMA_PEAK = 2500.0   # dense fp16 MFMA, TFLOP/s
+
+    def kernel_avg_us(fn, n_launch):
+        """Average duration of one call of fn(i): HIP events around 5 replays of a graph of n_launch calls, on the stream
+        the kernels are launched on (torch's current stream)."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn(0)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for i in range(n_launch):
+                fn(i)
+        gr.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (5 * n_launch) * 1e3
+
+    if args.shape:
+        kind, T, K, N = args.shape.split(":")
+        T, K, N = int(T), int(K), int(N)
+        if kind == "gemm_q4_K":
+            wq = synth.normal_weights("q4_K", N, K, seed=900, device=dev)
+            a16 = torch.randn((T, K), device=dev, generator=g).half()
+            yg = torch.empty((T, N), dtype=torch.float16, device=dev)
+            us = kernel_avg_us(lambda i: ops.gemm_q4_K(a16, wq, T, K, N, yg), 8)
+            print(json.dumps({"shape": args.shape, "avg_launch_us": round(us, 2), "TFLOPs": round(2.0 * T * N * K / us / 1e6, 1),
+                              "frac_mfma": round(2.0 * T * N * K / us / 1e6 / MFMA_PEAK, 4), "launches": 49}))
+        else:
+            fmt = kind[len("gemv_"):]
+            base = fmt.replace("_soa", "")
+            n_w = max(2, int(1.2e9 // (N * synth.row_bytes(base, K))))      # > 1 GB of weights in rotation
+            wl = [synth.normal_weights(base, N, K, seed=70 + i, device=dev) for i in range(n_w)]
+            if fmt.endswith("_soa"):
+                wl = [synth.split_q8_0(w) for w in wl]
+            xsq = ops.quantize_q8_1(torch.randn((T, K), device=dev, generator=g).half())
+            yt = torch.empty((T, N), dtype=torch.float16, device=dev)
+            if fmt.endswith("_soa"):
+                fn = lambda i: ops.gemv_q8_0_soa_q8_batched(xsq, wl[i % n_w][0], wl[i % n_w][1], K, N, T, yt)
+            else:
+                fn = lambda i: getattr(ops, "gemv_%s_q8_batched" % fmt)(xsq, wl[i % n_w], K, N, T, yt)
+            us = kernel_avg_us(fn, 2 * n_w)
+            b = gemv_bytes(synth.row_bytes(base, K), K, N, T)
+            print(json.dumps({"shape": args.shape, "avg_launch_us": round(us, 2), "GBps": round(b / us / 1e3, 1),
+                              "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4), "launches": 12 * n_w + 1}))
+        return
+
     # ---------------------------------------------------------------- inputs, resident in HBM
     fmts = ("q6_K", "q8_0")
     shapes = {"gate": (H, FF), "up": (H, FF), "down": (FF, H)}   # (K, N)
@@ -71,10 +129,8 @@ def main():
         ws = {}
         for fi, fmt in enumerate(fmts):
             for ni, (name, (K, N)) in enumerate(shapes.items()):
-                ws[(fmt, name)] = synth.random_weights(fmt, N, K, seed=1000 * s + 10 * fi + ni, device=dev)
+                ws[(fmt, name)] = synth.normal_weights(fmt, N, K, seed=1000 * s + 10 * fi + ni, device=dev)
         sets.append(ws)
-    g = torch.Generator(device=dev)
-    g.manual_seed(7)
     x = torch.randn((1, H), device=dev, generator=g).half()
     h = torch.randn((1, FF), device=dev, generator=g).half()
     xq, hq = ops.quantize_q8_1(x), ops.quantize_q8_1(h)
@@ -121,7 +177,7 @@ def main():
             dst.copy_(src)
         for i in range(8):
             step(sets[i % len(sets)])
-        wq = synth.random_weights("q4_K", FF, H, seed=900, device=dev)
+        wq = synth.normal_weights("q4_K", FF, H, seed=900, device=dev)
         a16 = torch.randn((2048, H), device=dev, generator=g).half()
         for _ in range(4):
             ops.gemm_q4_K(a16, wq, 2048, H, FF)
@@ -160,23 +216,6 @@ def main():
 
     # ---------------------------------------------------------------- roofline of the dominant kernel (HIP events)
     # Dominant by time and bytes: the Q8_0 gate/up GEMV (K=4096, N=14336), 62,390,272 weight bytes per launch.
-    def kernel_avg_us(fn, n_launch):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        fn(0)
-        torch.cuda.synchronize()
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(gr):
-            for i in range(n_launch):
-                fn(i)
-        gr.replay()
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(5):
-            gr.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / (5 * n_launch) * 1e3
-
     if args.unfused:
         mats = [ws[("q8_0_soa", n)] for ws in sets for n in ("gate", "up")]
         dom_us = kernel_avg_us(lambda i: ops.gemv_q8_0_soa_q8(xq, mats[i % len(mats)][0], mats[i % len(mats)][1], H, FF, y_ff[("q8_0", "gate")]),
@@ -202,13 +241,30 @@ def main():
                 # not part of the fraction above: what a read-only kernel reaches on the same bytes on this device
                 "stream_read_same_bytes": {"avg_launch_us": round(read_us, 3), "GBps": round(n_read / read_us / 1e3, 1)}}
 
+    # ---------------------------------------------------------------- the GEMM half of the metric: quant-GEMM at T = 2048
+    # BASELINE config 3, Q4_K 14336 x 4096 (N(0, 0.02) weights encoded in HBM) x fp16 activations N(0, 1) [2048 x 4096]
+    Tg, Kg, Ng = 2048, H, FF
+    wq = synth.normal_weights("q4_K", Ng, Kg, seed=900, device=dev)
+    a16 = torch.randn((Tg, Kg), device=dev, generator=g).half()
+    yg = torch.empty((Tg, Ng), dtype=torch.float16, device=dev)
+    gemm_us = kernel_avg_us(lambda i: ops.gemm_q4_K(a16, wq, Tg, Kg, Ng, yg), 8)
+    gemm_flop = 2.0 * Tg * Ng * Kg
+    gemm_tf = gemm_flop / gemm_us / 1e6
+    roofline_gemm = {"bound": "mfma", "kernel": "gemm_kernel<GemmQ4K, dense, 128-token tiles> T=2048 K=4096 N=14336 (v_mfma_f32_32x32x16_f16)",
+                     "achieved": round(gemm_tf, 1), "peak": MFMA_PEAK, "unit": "TFLOP/s", "frac": round(gemm_tf / MFMA_PEAK, 4),
+                     "flop_per_launch": gemm_flop, "avg_launch_us": round(gemm_us, 2),
+                     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt);
+                     # algorithmic bytes: W 33,030,144 + A 16,777,216 + Y 58,720,256
+                     "traffic": 254400000 + 58900000, "algorithmic_bytes": Ng * synth.row_bytes("q4_K", Kg) + Tg * Kg * 2 + Tg * Ng * 2}
+    del wq, a16, yg
+
     out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8 dot, fp32 fold", "data": "synthetic",
            "config": {"workload": "configs[1]: decode GEMV gate/up 4096->14336 + down 14336->4096, Q6_K and Q8_0, T=1, "
                                   "%s, %d rotating weight sets" % ("6 launches/step" if args.unfused else "gate+up fused: 4 launches/step", len(sets)),
                       "bytes_per_step": bytes_per_step, "hip_graph": bool(graphs), "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
-           "roofline": roofline}
+           "roofline": roofline, "roofline_gemm": roofline_gemm}
 
     # ---------------------------------------------------------------- detail: the other batch sizes and formats
     if not args.no_detail:
@@ -220,7 +276,7 @@ def main():
                         ("q4_K", ops.gemv_q4_K_q8_batched)):
             for name, (K, N) in (("gate_up", (H, FF)), ("down", (FF, H))):
                 if fmt == "q4_K":
-                    ws_l = [synth.random_weights(fmt, N, K, seed=77 + i, device=dev) for i in range(12)]
+                    ws_l = [synth.normal_weights(fmt, N, K, seed=77 + i, device=dev) for i in range(12)]
                 else:
                     # every matrix of every set, whatever its shape: the buffers are whole blocks and the same size for
                     # (K, N) and (N, K), and a dozen of them (0.6-0.75 GB) cannot stay in the 256 MB Infinity Cache
@@ -260,7 +316,7 @@ def main():
             us_c, us_f = kernel_avg_us(chain, 2 * len(sets)), kernel_avg_us(fused, 2 * len(sets))
             detail["ffn_decode_%s_T1" % fmt] = {"chain_4_launches_us": round(us_c, 2), "fused_2_launches_us": round(us_f, 2)}
         # BASELINE config 1: Q4_K 4096x4096, fp32 activations, fp32 out (9.4 MB: cache resident unless rotated)
-        w1 = [synth.random_weights("q4_K", 4096, 4096, seed=500 + i, device=dev) for i in range(40)]
+        w1 = [synth.normal_weights("q4_K", 4096, 4096, seed=500 + i, device=dev) for i in range(40)]
         a32 = torch.randn(4096, device=dev, generator=g)
         y32 = torch.empty(4096, dtype=torch.float32, device=dev)
         us = kernel_avg_us(lambda i: ops.gemv_q4_K(a32, w1[i % len(w1)], 4096, 4096, y32), 2 * len(w1))
@@ -273,16 +329,15 @@ def main():
         del w1
         # lm_head-sized decode GEMV (the largest single GEMV of a decode step): Q6_K, 4096 -> 151936, 510 MB
         NV = 151936
-        wl = [synth.random_weights("q6_K", NV, H, seed=700 + i, device=dev) for i in range(2)]
+        wl = [synth.normal_weights("q6_K", NV, H, seed=700 + i, device=dev) for i in range(2)]
         yv = torch.empty(NV, dtype=torch.float16, device=dev)
         us = kernel_avg_us(lambda i: ops.gemv_q6_K_q8(xq, wl[i % 2], H, NV, yv), 4)
         b = gemv_bytes(synth.row_bytes("q6_K", H), H, NV, 1)
         detail["lm_head_q6_K_K4096_N151936_T1"] = {"us": round(us, 1), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
         del wl, yv
         # BASELINE config 3: prefill quant-GEMM, Q4_K, fp16 MFMA (peak 2.5 PFLOP/s dense fp16)
-        MFMA_PEAK = 2500.0
         for (K, N) in ((H, FF), (FF, H)):
-            wq = synth.random_weights("q4_K", N, K, seed=900, device=dev)
+            wq = synth.normal_weights("q4_K", N, K, seed=900, device=dev)
             for T in (512, 2048, 4096):
                 a16 = torch.randn((T, K), device=dev, generator=g).half()
                 yg = torch.empty((T, N), dtype=torch.float16, device=dev)
@@ -308,9 +363,9 @@ def main():
         nrep = 6   # rotate expert banks so a decode step cannot live in the Infinity Cache
         banks = []
         for i in range(nrep):
-            gq, ge = synth.split_mxfp4(synth.random_weights("mxfp4", E4 * H4, H4, seed=3000 + i, device=dev))
-            uq, ue = synth.split_mxfp4(synth.random_weights("mxfp4", E4 * H4, H4, seed=3100 + i, device=dev))
-            dq, de = synth.split_mxfp4(synth.random_weights("mxfp4", E4 * H4, H4, seed=3200 + i, device=dev))
+            gq, ge = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3000 + i, device=dev))
+            uq, ue = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3100 + i, device=dev))
+            dq, de = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3200 + i, device=dev))
             banks.append((gq, ge, uq, ue, dq, de))
         qs_st, e_st = H4 * H4 // 2, H4 * H4 // 32
         per_expert = 3 * (qs_st + e_st)
@@ -353,9 +408,9 @@ def main():
         del banks
         # BASELINE config 5: Qwen3-MoE style grouped GEMM, E=128 top-8 H=2048 EF=768, 2048 tokens, Zipf(1.1), Q8_0 experts
         E5, K5, H5, EF5, T5 = 128, 8, 2048, 768, 2048
-        gq5, gd5 = synth.split_q8_0(synth.random_weights("q8_0", E5 * EF5, H5, seed=5000, device=dev))
-        uq5, ud5 = synth.split_q8_0(synth.random_weights("q8_0", E5 * EF5, H5, seed=5001, device=dev))
-        dq5, dd5 = synth.split_q8_0(synth.random_weights("q8_0", E5 * H5, EF5, seed=5002, device=dev))
+        gq5, gd5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * EF5, H5, seed=5000, device=dev))
+        uq5, ud5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * EF5, H5, seed=5001, device=dev))
+        dq5, dd5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * H5, EF5, seed=5002, device=dev))
         pz = np.arange(1, E5 + 1, dtype=np.float64) ** -1.1
         pz = pz[rng.permutation(E5)]
         pz /= pz.sum()
