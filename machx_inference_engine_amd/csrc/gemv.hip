@@ -2,6 +2,7 @@
 // Q4_K / Q6_K / Q8_0 / MXFP4 weights: int-dot on q8 activations and the
 // float-activation variants.  Kernel structure: mxq_gemv_core.h.
 #include "mxq_gemv_core.h"
+#include "mxq_mmq.h"
 #include <stdlib.h>
 
 #include <type_traits>
@@ -599,6 +600,81 @@ static int launch_q8_g(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSeg
     return MX_ERR_SHAPE;
 }
 
+// ---------------------------------------------------------------- batches on the matrix cores (mxq_mmq.h)
+// Formats with an int8 operand producer run every batch of two and more rows there: the weight stream is the same,
+// the per-token dot products become one matrix instruction per block and 32 rows.
+template <class F> struct MmqOf { using type = void; };
+template <> struct MmqOf<FmtQ8Soa> { using type = MmqQ8Soa; };
+template <> struct MmqOf<FmtQ8Aos> { using type = MmqQ8Aos; };
+template <> struct MmqOf<FmtQ4K> { using type = MmqQ4K; };
+template <> struct MmqOf<FmtQ6K> { using type = MmqQ6K; };
+template <> struct MmqOf<FmtMxfp4Soa> { using type = MmqMxfp4Soa; };
+
+static typename FmtQ8Soa::Bank mmq_bank(const FmtQ8Soa::W& w) { return {w.qs, w.d, 0, 0, w.K}; }
+static typename FmtQ4K::Bank mmq_bank(const FmtQ4K::W& w) { return {w.base, 0, w.row_bytes}; }
+static MmqQ8Aos::Bank mmq_bank(const FmtQ8Aos::W& w) { return {w.base, 0, w.row_bytes}; }
+static typename FmtQ6K::Bank mmq_bank(const FmtQ6K::W& w) { return {w.base, 0, w.row_bytes}; }
+static typename FmtMxfp4Soa::Bank mmq_bank(const FmtMxfp4Soa::W& w) { return {w.qs, w.e, 0, 0, w.K}; }
+
+constexpr uint32_t kMmqLdsBudget = 48 * 1024;
+constexpr uint32_t kMmqMaxRanges = 16;   // K ranges across workgroups of one dense launch
+
+// staged k range per pass: the largest multiple of `gran` elements whose LDS image fits the budget
+static uint32_t mmq_pass_range(uint32_t T, int TV, bool has_min, uint32_t gran) {
+    const uint32_t per256 = T * 256u + 8u * (uint32_t)(2 * TV) * 4u * (has_min ? 2u : 1u);
+    const uint32_t n256 = (kMmqLdsBudget - 32u * T) / per256;
+    const uint32_t kr = n256 * 256u / gran * gran;
+    return kr ? kr : gran;
+}
+
+// K ranges across workgroups of a dense launch when the row blocks alone leave CUs idle: about two workgroups per CU,
+// every wave keeping at least two groups
+static uint32_t mmq_dense_ranges(uint32_t K, uint32_t N, uint32_t WR, uint32_t WK) {
+    const uint32_t cus = (uint32_t)cu_count();
+    const uint32_t n_groups = (K / 32u + 7u) / 8u, rgs = (N + 32u * WR - 1u) / (32u * WR);
+    uint32_t Z = 1;
+    if (2u * rgs < 3u * cus) Z = (2u * cus + rgs - 1u) / rgs;
+    if (Z > n_groups / (2u * WK)) Z = n_groups / (2u * WK);
+    if (Z > kMmqMaxRanges) Z = kMmqMaxRanges;
+    return Z < 1 ? 1 : Z;
+}
+
+template <class P, int TV, int WR, int WK>
+static int launch_mmq_dense_cfg(hipStream_t st, const typename P::Bank& bank, const uint8_t* xq8, half_t* y, uint32_t K, uint32_t N, uint32_t T,
+                                bool split, const SplitWs& ws) {
+    const uint32_t nb = K / 32u, n_groups = (nb + 7u) / 8u;
+    const uint32_t rgs = (N + 32u * WR - 1u) / (32u * WR);
+    uint32_t Z = mmq_dense_ranges(K, N, WR, WK);   // the partial sums have to fit the scratch
+    if (Z > 1 && (!ws.ptr || (uint64_t)Z * T * N > ws.elems)) {
+        if (ws.caller) return MX_ERR_WORKSPACE;
+        while (Z > 1 && (uint64_t)Z * T * N > ws.elems) --Z;
+    }
+    const uint32_t gz = (n_groups + Z - 1u) / Z;
+    Z = (n_groups + gz - 1u) / gz;
+    uint32_t kr = mmq_pass_range(T, TV, P::HAS_MIN, 256u * WK);
+    const uint32_t need = (gz + WK - 1u) / WK * WK * 256u;
+    if (kr > need) kr = need;
+    MmqArgs<P> a{};
+    a.bank0 = bank; a.bank1 = bank; a.xq8 = xq8; a.out = y; a.part = Z > 1 ? ws.ptr : nullptr;
+    a.M = T; a.K = K; a.N = N; a.E = 1; a.q8_split = split ? 1u : 0u; a.kr = kr;
+    uint32_t lds = mmq_lds_bytes(T, kr, TV, P::HAS_MIN);
+    const uint32_t red = (uint32_t)(WR * WK) * TV * 64u * 4u;
+    if (lds < red) lds = red;
+    hipLaunchKernelGGL((mmq_kernel<P, TV, 1, WR, WK, MMQ_STORE>), dim3(rgs, 1, Z), dim3(64 * WR * WK), lds, st, a);
+    if (Z > 1) {
+        const uint32_t mn = T * N;
+        hipLaunchKernelGGL(mmq_reduce_kernel, dim3((mn + 255u) / 256u), dim3(256), 0, st, y, ws.ptr, mn, Z);
+    }
+    return launch_status();
+}
+
+template <class P>
+static int launch_mmq_dense(hipStream_t st, const typename P::Bank& bank, const uint8_t* xq8, half_t* y, uint32_t K, uint32_t N, uint32_t T, bool split,
+                            const SplitWs& ws) {
+    if (T <= 8) return launch_mmq_dense_cfg<P, 4, 1, 4>(st, bank, xq8, y, K, N, T, split, ws);
+    return launch_mmq_dense_cfg<P, 8, 2, 2>(st, bank, xq8, y, K, N, T, split, ws);
+}
+
 // T up to 16: passes of at most 8 tokens.
 template <class F, class OutT>
 static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, int nseg, const void* xq8, uint32_t K, uint32_t N, uint32_t T,
@@ -607,8 +683,14 @@ static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, in
     const uint32_t G = pick_group((K + 63) / 64);
     SplitWs ws{nullptr, 0, false};
     if (caller_ws) ws = *caller_ws;
-    else if (T >= 2 && nseg == 1 && K >= 8192)   // the only launches that may split K
+    else if (T >= 2 && nseg == 1)   // the only launches that may split K
         if (int rc = static_split_ws(&ws)) return rc;
+    using P = typename MmqOf<F>::type;
+    if constexpr (!std::is_void<P>::value && std::is_same<OutT, half_t>::value) {
+        // measured crossover against the vector-ALU batch kernels (4096 -> 14336, us): Q8_0 planes T = 4: 15.4 vs 16.1,
+        // T = 8: 20.4 vs 17.6; Q6_K T = 8: 26.2 vs 22.0; batches of 9 .. 16 take one pass here instead of two there
+        if (T >= 5 && nseg == 1 && !s0.bias) return launch_mmq_dense<P>(as_stream(s), mmq_bank(s0.w), x, s0.y, K, N, T, split, ws);
+    }
     for (uint32_t t0 = 0; t0 < T; t0 += 8) {
         const uint32_t tn = (T - t0 < 8) ? T - t0 : 8;
         GemvSeg<F, OutT> a = s0, b = s1;
@@ -860,8 +942,13 @@ static int check_ws(const void* ws, uint64_t ws_bytes, uint32_t K, uint32_t N, u
 int mx_gemv_batched_ws_bytes(uint32_t K, uint32_t N, uint32_t T, uint64_t* bytes) {
     MX_REQUIRE_PTR(bytes);
     MX_REQUIRE_SHAPE(K > 0 && N > 0 && T >= 1 && T <= 16);
-    // an upper bound over every format and device: up to kSplitMaxSlices slices of a pass of at most 8 tokens
-    *bytes = (T >= 2 && K >= 8192) ? (uint64_t)kSplitMaxSlices * (T < 8 ? T : 8) * N * sizeof(float) : 0;
+    // the K ranges the launch would like on this device (none: the row blocks fill the chip), T x N partial sums each
+    // batches of 5 and more run on the matrix cores (K ranges as the row blocks need them); smaller ones split K >= 8192 over up
+    // to kSplitMaxSlices slices
+    uint32_t Z = 1;
+    if (T >= 5) Z = T <= 8 ? mmq_dense_ranges(K, N, 1, 4) : mmq_dense_ranges(K, N, 2, 2);
+    else if (T >= 2 && K >= 8192) Z = kSplitMaxSlices;
+    *bytes = Z > 1 ? (uint64_t)Z * T * N * sizeof(float) : 0;
     return MX_OK;
 }
 int mx_gemv_q8_0_soa_q8_batched_ws(mx_stream_t s, const void* x, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t K, uint32_t N,

@@ -15,6 +15,9 @@
 // function in the epilogue.
 #include "mxq_gemv_core.h"
 #include "mxq_host.h"
+#include "mxq_mmq.h"
+
+#include <type_traits>
 
 namespace mxq {
 
@@ -330,8 +333,46 @@ static int launch_moe(mx_stream_t s, const typename F::Bank& b0, const typename 
 #undef MX_MOE_G
 }
 
+// ---------------------------------------------------------------- expert-grouped rows on the matrix cores (mxq_mmq.h)
+// grid (blocks of 32 WR weight rows, experts): a workgroup walks its expert's rows in passes of 2 TV tokens; its slice of
+// the expert's weights (32 WR rows) is re-read from L2 by every pass after the first.
+constexpr uint32_t kMmqMoeLdsBudget = 48 * 1024;
+
+template <class P, int TV, int NW, int WR, int WK, int EPI>
+static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, const typename P::Bank& b1, const MoeArgs& m, uint32_t E) {
+    MmqArgs<P> a{};
+    a.bank0 = b0; a.bank1 = b1; a.xq8 = m.xq8; a.expert_offsets = m.expert_offsets; a.out = m.out; a.bias0 = m.bias0; a.bias1 = m.bias1;
+    a.route_w = m.route_w; a.alpha = m.alpha; a.limit = m.limit; a.M = 0; a.K = m.K; a.N = m.N; a.E = E; a.q8_split = m.q8_split;
+    a.act_f16 = m.act_f16;
+    constexpr uint32_t TT = 2 * TV, gran = 256u * WK;
+    const uint32_t per256 = TT * 256u + 8u * TT * 4u * (P::HAS_MIN ? 2u : 1u);
+    uint32_t kr = (kMmqMoeLdsBudget - 32u * TT) / per256 * 256u / gran * gran;
+    if (!kr) kr = gran;
+    const uint32_t need = ((m.K + 255u) / 256u + WK - 1u) / WK * WK * 256u;
+    if (kr > need) kr = need;
+    a.kr = kr;
+    uint32_t lds = mmq_lds_bytes(TT, kr, TV, P::HAS_MIN);
+    const uint32_t red = (uint32_t)(NW * WR * WK) * TV * 64u * 4u;
+    if (lds < red) lds = red;
+    const uint32_t rgs = (m.N + 32u * WR - 1u) / (32u * WR);
+    if (E > 65535u) return MX_ERR_SHAPE;
+    hipLaunchKernelGGL((mmq_kernel<P, TV, NW, WR, WK, EPI>), dim3(rgs, E, 1), dim3(64 * NW * WR * WK), lds, st, a);
+    return launch_status();
+}
+
+// avg_rows = expected rows per expert (0: unknown)
+template <class P, int NW, int EPI>
+static int launch_mmq_grouped(mx_stream_t s, const typename P::Bank& b0, const typename P::Bank& b1, const MoeArgs& m, uint32_t E, uint32_t avg_rows) {
+    hipStream_t st = as_stream(s);
+    if (avg_rows && avg_rows <= 8) return launch_mmq_grouped_cfg<P, 4, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E);
+    if (avg_rows && avg_rows <= 16) return launch_mmq_grouped_cfg<P, 8, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E);
+    return launch_mmq_grouped_cfg<P, 16, NW, (NW == 1 ? 4 : 2), 1, EPI>(st, b0, b1, m, E);
+}
+
 // rows per token tile in grouped mode: expected rows per expert, rounded up to 4 or 8
 static uint32_t grouped_tt(uint64_t total_rows, uint32_t E) { return (total_rows <= 4ull * E) ? 4 : 8; }
+// expected rows per expert for the matrix-core launch (0: the signature carries no row count)
+static uint32_t avg_rows(uint32_t total_rows, uint32_t E) { return total_rows == 0xFFFFFFFFu ? 0u : (total_rows + E - 1u) / E; }
 
 template <class F, int MODE>
 static int launch_moe_fact(mx_stream_t s, const typename F::Bank& b0, const typename F::Bank& b1, MoeFactArgs a, uint32_t n_seg) {
@@ -397,6 +438,11 @@ static int moe_grouped_kquant(mx_stream_t s, const void* act_q8, bool split, con
     a.xq8 = static_cast<const uint8_t*>(act_q8); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out);
     a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = split ? 1u : 0u;
     const typename F::Bank b0 = F::bank(W0, expert_stride_bytes, K, N), b1 = F::bank(W1, expert_stride_bytes, K, N);
+    constexpr int MEPI = EPI == EPI_SILU ? MMQ_SILU : MMQ_DOWN_BIAS;
+    if constexpr (std::is_same<F, FmtQ4K>::value) return launch_mmq_grouped<MmqQ4K, NW, MEPI>(s, b0, b1, a, E, avg_rows(total_rows, E));
+    if constexpr (std::is_same<F, FmtQ6K>::value) return launch_mmq_grouped<MmqQ6K, NW, MEPI>(s, b0, b1, a, E, avg_rows(total_rows, E));
+    if constexpr (std::is_same<F, FmtQ4KStr>::value) return launch_mmq_grouped<MmqQ4KStr, NW, MEPI>(s, b0, b1, a, E, avg_rows(total_rows, E));
+    if constexpr (std::is_same<F, FmtQ6KStr>::value) return launch_mmq_grouped<MmqQ6KStr, NW, MEPI>(s, b0, b1, a, E, avg_rows(total_rows, E));
     return launch_moe<F, NW, EPI>(s, b0, b1, a, E, grouped_tt(total_rows, E));
 }
 
@@ -493,7 +539,7 @@ static int moe_grouped_gate_up_silu_q8_gemv(mx_stream_t s, const void* xq8_packe
     a.xq8 = static_cast<const uint8_t*>(xq8_packed); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(h_packed);
     a.act_div = 1; a.K = H; a.N = E_ffn; a.n_experts = E;
     FmtQ8Soa::Bank bg{g_qs, g_d, qs_stride, d_stride, H}, bu{u_qs, u_d, qs_stride, d_stride, H};
-    return launch_moe<FmtQ8Soa, 2, EPI_SILU>(s, bg, bu, a, E, grouped_tt(total_rows, E));
+    return launch_mmq_grouped<MmqQ8Soa, 2, MMQ_SILU>(s, bg, bu, a, E, avg_rows(total_rows, E));
 }
 static int moe_grouped_down_q8_gemv(mx_stream_t s, const void* hq8_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
                            uint64_t d_stride, const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E,
@@ -506,7 +552,7 @@ static int moe_grouped_down_q8_gemv(mx_stream_t s, const void* hq8_packed, const
     a.xq8 = static_cast<const uint8_t*>(hq8_packed); a.expert_offsets = expert_offsets; a.route_w = reinterpret_cast<const half_t*>(sorted_w);
     a.out = reinterpret_cast<half_t*>(out_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = E;
     FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
-    return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, E, grouped_tt(total_rows, E));
+    return launch_mmq_grouped<MmqQ8Soa, 1, MMQ_DOWN_WEIGHTED>(s, b, b, a, E, avg_rows(total_rows, E));
 }
 
 int mx_moe_prefill_gate_up_silu_q8(mx_stream_t s, const void* xq8_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
@@ -534,6 +580,7 @@ static int moe_mxfp4_gate_up(mx_stream_t s, const void* x_q8, const uint8_t* g_q
     a.xq8 = static_cast<const uint8_t*>(x_q8); a.topk_idx = topk_idx; a.expert_offsets = expert_offsets; a.bias0 = gate_bias; a.bias1 = up_bias;
     a.out = reinterpret_cast<half_t*>(h_out); a.alpha = alpha; a.limit = limit; a.act_div = act_div; a.K = H; a.N = E_ffn; a.n_experts = n_experts;
     FmtMxfp4Soa::Bank bg{g_qs, g_e, qs_stride, e_stride, H}, bu{u_qs, u_e, qs_stride, e_stride, H};
+    if (expert_offsets) return launch_mmq_grouped<MmqMxfp4Soa, 2, MMQ_OAI>(s, bg, bu, a, n_seg, tt);   // grouped: tt = expected rows per expert
     return launch_moe<FmtMxfp4Soa, 2, EPI_OAI>(s, bg, bu, a, n_seg, tt);
 }
 int mx_moe_gate_up_oai_mxfp4(mx_stream_t s, const void* x_q8, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
@@ -550,7 +597,7 @@ int mx_moe_grouped_gate_up_oai_mxfp4(mx_stream_t s, const void* xq8_packed, cons
                                      uint32_t total_rows, float alpha, float limit) {
     MX_REQUIRE_PTR(expert_offsets);
     return moe_mxfp4_gate_up(s, xq8_packed, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, nullptr, expert_offsets, h_packed, E, 1,
-                             H, E_ffn, E, alpha, limit, grouped_tt(total_rows, E));
+                             H, E_ffn, E, alpha, limit, avg_rows(total_rows, E));
 }
 static int moe_mxfp4_down(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
                           const float* down_bias, const int32_t* topk_idx, const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t n_seg,
@@ -565,6 +612,7 @@ static int moe_mxfp4_down(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, 
     a.out = reinterpret_cast<half_t*>(out_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
     if (act_is_f16) a.act_f16 = static_cast<const half_t*>(h_q8);
     FmtMxfp4Soa::Bank b{d_qs, d_e, qs_stride, e_stride, E_ffn};
+    if (expert_offsets) return launch_mmq_grouped<MmqMxfp4Soa, 1, MMQ_DOWN_BIAS>(s, b, b, a, n_seg, tt);   // grouped: tt = expected rows per expert
     return launch_moe<FmtMxfp4Soa, 1, EPI_DOWN_BIAS>(s, b, b, a, n_seg, tt);
 }
 int mx_moe_down_mxfp4(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
@@ -578,7 +626,7 @@ int mx_moe_grouped_down_mxfp4(mx_stream_t s, const void* hq8_packed, const uint8
                               uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
     MX_REQUIRE_PTR(expert_offsets);
     return moe_mxfp4_down(s, hq8_packed, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
-                          grouped_tt(total_rows, E));
+                          avg_rows(total_rows, E));
 }
 
 // The down projections taking h as fp16 and quantizing it while staging (same q8 values as mx_quantize_q8_1(h)): no quantize launch.
@@ -593,7 +641,7 @@ int mx_moe_grouped_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_packed_f16, c
                                   uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
     MX_REQUIRE_PTR(expert_offsets);
     return moe_mxfp4_down(s, h_packed_f16, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
-                          grouped_tt(total_rows, E), true);
+                          avg_rows(total_rows, E), true);
 }
 int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
                        const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {

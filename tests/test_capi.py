@@ -69,9 +69,9 @@ def test_workspace_forms_validate_before_any_hip_call(lib):
     OK, NULL, SHAPE, ALIGN, WORKSPACE = 0, 1, 2, 3, 9
     p16 = 0x1000
     n = C.c_uint64(7)
+    # without a GPU the library assumes 256 CUs: 128 blocks of 32 rows want 4 K ranges of T x N partial sums
     assert l.mx_gemv_batched_ws_bytes(14336, 4096, 8, C.addressof(n)) == OK and n.value == 4 * 8 * 4096 * 4
-    assert l.mx_gemv_batched_ws_bytes(14336, 4096, 16, C.addressof(n)) == OK and n.value == 4 * 8 * 4096 * 4   # passes of 8 tokens
-    assert l.mx_gemv_batched_ws_bytes(4096, 14336, 8, C.addressof(n)) == OK and n.value == 0                    # short rows never split
+    assert l.mx_gemv_batched_ws_bytes(4096, 151936, 8, C.addressof(n)) == OK and n.value == 0                   # enough row blocks: K is never split
     assert l.mx_gemv_batched_ws_bytes(14336, 4096, 1, C.addressof(n)) == OK and n.value == 0
     assert l.mx_gemv_batched_ws_bytes(14336, 4096, 8, None) == NULL
     assert l.mx_gemv_batched_ws_bytes(14336, 4096, 17, C.addressof(n)) == SHAPE

@@ -27,7 +27,7 @@ def test_split_k_gemv_static_scratch_equals_workspace_form(mx):
     rb = K // 32 * 40
     for (N, T) in ((N1, T1), (N2, T2)):
         need = ops.gemv_batched_ws_bytes(K, N, T)
-        assert need == 4 * T * N * 4
+        assert need >= 2 * T * N * 4            # these shapes split K over at least two ranges
         ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
         y_static = ops.gemv_q8_0_soa_q8_batched(xq[:T * rb], qs[:N * K], d[:N * (K // 32)], K, N, T)
         y_ws = ops.gemv_q8_batched_ws("q8_0_soa", xq[:T * rb], (qs[:N * K], d[:N * (K // 32)]), K, N, T, ws)
