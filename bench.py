@@ -50,6 +50,9 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="distinct weight sets rotated through (331.7 MB each)")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: a few launches of the dominant kernels and of a plain copy of known size, no timing")
+    ap.add_argument("--legs", default="all",
+                    help="comma-separated detail legs to run (batched, ffn, c1, lm_head, c3, c4, c5); with a list the headline legs are skipped "
+                         "and only the detail table is printed (development aid)")
     ap.add_argument("--shape", default=None, metavar="KIND:T:K:N",
                     help="profiling aid: only launches of one kernel at one shape (KIND in gemm_q4_K, gemv_q8_0_soa, gemv_q6_K, gemv_q4_K), "
                          "so that a rocprofv3 run holds exactly one (kernel, shape) pair; prints its HIP-event average")
@@ -120,6 +123,11 @@ def main():
             print(json.dumps({"shape": args.shape, "avg_launch_us": round(us, 2), "GBps": round(b / us / 1e3, 1),
                               "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4), "launches": 12 * n_w + 1}))
         return
+
+    legs = None if args.legs == "all" else set(args.legs.split(","))
+    if legs is not None:
+        args.no_cpu, args.sets, args.steps, args.warmup = True, 1, 8, 2
+    want = lambda name: legs is None or name in legs
 
     # ---------------------------------------------------------------- inputs, resident in HBM
     fmts = ("q6_K", "q8_0")
@@ -268,169 +276,192 @@ def main():
 
     # ---------------------------------------------------------------- detail: the other batch sizes and formats
     if not args.no_detail:
-        detail = {}
-        def soa_batched(xsq_, w, K, N, T, yt_):
-            return ops.gemv_q8_0_soa_q8_batched(xsq_, w[0], w[1], K, N, T, yt_)
-
-        for fmt, fn in (("q6_K", ops.gemv_q6_K_q8_batched), ("q8_0_soa", soa_batched), ("q8_0", ops.gemv_q8_0_q8_batched),
-                        ("q4_K", ops.gemv_q4_K_q8_batched)):
-            for name, (K, N) in (("gate_up", (H, FF)), ("down", (FF, H))):
-                if fmt == "q4_K":
-                    ws_l = [synth.normal_weights(fmt, N, K, seed=77 + i, device=dev) for i in range(12)]
-                else:
-                    # every matrix of every set, whatever its shape: the buffers are whole blocks and the same size for
-                    # (K, N) and (N, K), and a dozen of them (0.6-0.75 GB) cannot stay in the 256 MB Infinity Cache
-                    ws_l = [ws[(fmt, n)] for ws in sets for n in ("gate", "up", "down")]
-                for T in (1, 2, 4, 8):
-                    xs = torch.randn((T, K), device=dev, generator=g).half()
-                    xsq = ops.quantize_q8_1(xs)
-                    yt = torch.empty((T, N), dtype=torch.float16, device=dev)
-                    us = kernel_avg_us(lambda i: fn(xsq, ws_l[i % len(ws_l)], K, N, T, yt), 3 * len(ws_l))
-                    b = gemv_bytes(synth.row_bytes(fmt.replace("_soa", ""), K), K, N, T)
-                    detail["%s_%s_T%d" % (fmt, name, T)] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1),
-                                                            "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
-                    if T == 1 and name == "gate_up":
-                        # the same launch on one matrix over and over: served from the 256 MB Infinity Cache, not from HBM
-                        us_c = kernel_avg_us(lambda i: fn(xsq, ws_l[0], K, N, T, yt), 24)
-                        detail["%s_%s_T1_cache_resident" % (fmt, name)] = {"us": round(us_c, 2), "GBps": round(b / us_c / 1e3, 1)}
-                del ws_l
-        # one decode FFN (fp16 x in, fp16 y out) as the reference's launch chain and as the two fused launches
-        xf = torch.randn(H, device=dev, generator=g).half()
-        xq_b = torch.empty(H // 32 * 40, dtype=torch.uint8, device=dev)
-        hq_b = torch.empty(FF // 32 * 40, dtype=torch.uint8, device=dev)
-        g_b, u_b, h_b = (torch.empty(FF, dtype=torch.float16, device=dev) for _ in range(3))
-        y_b = torch.empty(H, dtype=torch.float16, device=dev)
-        for fmt, key in (("q8_0_soa", "q8_0_soa"), ("q6_K", "q6_K")):
-            def chain(i):
-                ws = sets[i % len(sets)]
-                ops.quantize_q8_1(xf, xq_b)
-                ops.gemv_q8_x2(fmt, xq_b, ws[(key, "gate")], ws[(key, "up")], H, FF, g_b, u_b)
-                ops.swiglu_q8(g_b, u_b, out=(h_b, hq_b))
-                gemv(key.replace("_soa", ""), hq_b, ws, "down", FF, H, y_b)
-
-            def fused(i):
-                ws = sets[i % len(sets)]
-                ops.gemv_x2_silu(fmt, xf, ws[(key, "gate")], ws[(key, "up")], H, FF, h_b)
-                ops.gemv_f16q8(fmt, h_b, ws[(key, "down")], FF, H, y_b)
-
-            us_c, us_f = kernel_avg_us(chain, 2 * len(sets)), kernel_avg_us(fused, 2 * len(sets))
-            detail["ffn_decode_%s_T1" % fmt] = {"chain_4_launches_us": round(us_c, 2), "fused_2_launches_us": round(us_f, 2)}
-        # BASELINE config 1: Q4_K 4096x4096, fp32 activations, fp32 out (9.4 MB: cache resident unless rotated)
-        w1 = [synth.normal_weights("q4_K", 4096, 4096, seed=500 + i, device=dev) for i in range(40)]
-        a32 = torch.randn(4096, device=dev, generator=g)
-        y32 = torch.empty(4096, dtype=torch.float32, device=dev)
-        us = kernel_avg_us(lambda i: ops.gemv_q4_K(a32, w1[i % len(w1)], 4096, 4096, y32), 2 * len(w1))
-        b = 4096 * synth.row_bytes("q4_K", 4096) + 2 * 4096 * 4
-        detail["config1_q4_K_4096x4096_f32"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
-        aq = ops.quantize_q8_1(a32)
-        y16 = torch.empty(4096, dtype=torch.float16, device=dev)
-        us = kernel_avg_us(lambda i: ops.gemv_q4_K_q8(aq, w1[i % len(w1)], 4096, 4096, y16), 2 * len(w1))
-        detail["config1_q4_K_4096x4096_q8"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
-        del w1
-        # lm_head-sized decode GEMV (the largest single GEMV of a decode step): Q6_K, 4096 -> 151936, 510 MB
-        NV = 151936
-        wl = [synth.normal_weights("q6_K", NV, H, seed=700 + i, device=dev) for i in range(2)]
-        yv = torch.empty(NV, dtype=torch.float16, device=dev)
-        us = kernel_avg_us(lambda i: ops.gemv_q6_K_q8(xq, wl[i % 2], H, NV, yv), 4)
-        b = gemv_bytes(synth.row_bytes("q6_K", H), H, NV, 1)
-        detail["lm_head_q6_K_K4096_N151936_T1"] = {"us": round(us, 1), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
-        del wl, yv
-        # BASELINE config 3: prefill quant-GEMM, Q4_K, fp16 MFMA (peak 2.5 PFLOP/s dense fp16)
-        for (K, N) in ((H, FF), (FF, H)):
-            wq = synth.normal_weights("q4_K", N, K, seed=900, device=dev)
-            for T in (512, 2048, 4096):
-                a16 = torch.randn((T, K), device=dev, generator=g).half()
-                yg = torch.empty((T, N), dtype=torch.float16, device=dev)
-                us = kernel_avg_us(lambda i: ops.gemm_q4_K(a16, wq, T, K, N, yg), 4)
-                tf = 2.0 * T * N * K / us / 1e6
-                ent = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
-                if T >= 2048:
-                    # the same product the reference's way on this box: dequantize W to an fp16 [K, N] matrix, then the
-                    # vendor library's fp16 GEMM (rocBLAS here, oneDNN there); and that GEMM alone
-                    bt = ops.dequant_to_Bt("q4_K", wq, K, N)
-                    us_g = kernel_avg_us(lambda i: ops.gemm_fp16(a16, bt, T, N, K, torch.float16, yg), 4)
-                    us_2 = kernel_avg_us(lambda i: (ops.dequant_to_Bt("q4_K", wq, K, N, bt), ops.gemm_fp16(a16, bt, T, N, K, torch.float16, yg)), 4)
-                    ent["vendor_fp16_gemm_us"] = round(us_g, 1)
-                    ent["vendor_fp16_gemm_TFLOPs"] = round(2.0 * T * N * K / us_g / 1e6, 1)
-                    ent["dequant_plus_vendor_gemm_us"] = round(us_2, 1)
-                    del bt
-                detail["config3_gemm_q4_K_T%d_K%d_N%d" % (T, K, N)] = ent
-                del a16, yg
-            del wq
-        # BASELINE config 4: MXFP4 MoE decode at gpt-oss-20b shape (E=32, top-4, H=EF=2880), T=1 and T=32
         import numpy as np
-        E4, K4, H4 = 32, 4, 2880
-        nrep = 6   # rotate expert banks so a decode step cannot live in the Infinity Cache
-        banks = []
-        for i in range(nrep):
-            gq, ge = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3000 + i, device=dev))
-            uq, ue = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3100 + i, device=dev))
-            dq, de = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3200 + i, device=dev))
-            banks.append((gq, ge, uq, ue, dq, de))
-        qs_st, e_st = H4 * H4 // 2, H4 * H4 // 32
-        per_expert = 3 * (qs_st + e_st)
         rng = np.random.default_rng(4)
-        for T in (1, 32):
-            logits = rng.standard_normal((T, E4)).astype(np.float32)
-            ids = np.sort(np.argsort(-logits, axis=1)[:, :K4], axis=1).astype(np.int32)
-            wts = np.full((T, K4), 0.25, np.float32)
-            off, si, wp, t2p = ops.build_moe_packing(ids, wts, E4)
-            n_distinct = int((np.diff(off.astype(np.int64)) > 0).sum())
-            xt = torch.randn((T, H4), device=dev, generator=g).half()
-            TK = T * K4
-            offd, sid = torch.from_numpy(off).to(dev), torch.from_numpy(si).to(dev)
-            idsd = torch.from_numpy(ids.ravel().copy()).to(dev)
-            hbuf = torch.empty((TK, H4), dtype=torch.float16, device=dev)
-            obuf = torch.empty((TK, H4), dtype=torch.float16, device=dev)
-            xq8 = ops.quantize_q8_1(xt)
-            xpq = ops.quantize_q8_1(ops.moe_gather_rows(xt, sid, TK, H4))
-            hq8 = ops.quantize_q8_1(hbuf)
+        detail = {}
+        if want('batched'):
+            def soa_batched(xsq_, w, K, N, T, yt_):
+                return ops.gemv_q8_0_soa_q8_batched(xsq_, w[0], w[1], K, N, T, yt_)
 
-            def layer(i):
-                b = banks[i % nrep]
-                if T == 1:    # device-side expert ids, one launch per stage
-                    ops.moe_gate_up_oai_mxfp4(xq8, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, idsd, T, K4, H4, H4, E4, h_out=hbuf)
-                    if args.unfused:
+            for fmt, fn in (("q6_K", ops.gemv_q6_K_q8_batched), ("q8_0_soa", soa_batched), ("q8_0", ops.gemv_q8_0_q8_batched),
+                            ("q4_K", ops.gemv_q4_K_q8_batched)):
+                for name, (K, N) in (("gate_up", (H, FF)), ("down", (FF, H))):
+                    if fmt == "q4_K":
+                        ws_l = [synth.normal_weights(fmt, N, K, seed=77 + i, device=dev) for i in range(12)]
+                    else:
+                        # every matrix of every set, whatever its shape: the buffers are whole blocks and the same size for
+                        # (K, N) and (N, K), and a dozen of them (0.6-0.75 GB) cannot stay in the 256 MB Infinity Cache
+                        ws_l = [ws[(fmt, n)] for ws in sets for n in ("gate", "up", "down")]
+                    for T in (1, 2, 4, 8):
+                        xs = torch.randn((T, K), device=dev, generator=g).half()
+                        xsq = ops.quantize_q8_1(xs)
+                        yt = torch.empty((T, N), dtype=torch.float16, device=dev)
+                        us = kernel_avg_us(lambda i: fn(xsq, ws_l[i % len(ws_l)], K, N, T, yt), 3 * len(ws_l))
+                        b = gemv_bytes(synth.row_bytes(fmt.replace("_soa", ""), K), K, N, T)
+                        detail["%s_%s_T%d" % (fmt, name, T)] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1),
+                                                                "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+                        if T == 1 and name == "gate_up":
+                            # the same launch on one matrix over and over: served from the 256 MB Infinity Cache, not from HBM
+                            us_c = kernel_avg_us(lambda i: fn(xsq, ws_l[0], K, N, T, yt), 24)
+                            detail["%s_%s_T1_cache_resident" % (fmt, name)] = {"us": round(us_c, 2), "GBps": round(b / us_c / 1e3, 1)}
+                    del ws_l
+        if want('ffn'):
+            # one decode FFN (fp16 x in, fp16 y out) as the reference's launch chain and as the two fused launches
+            xf = torch.randn(H, device=dev, generator=g).half()
+            xq_b = torch.empty(H // 32 * 40, dtype=torch.uint8, device=dev)
+            hq_b = torch.empty(FF // 32 * 40, dtype=torch.uint8, device=dev)
+            g_b, u_b, h_b = (torch.empty(FF, dtype=torch.float16, device=dev) for _ in range(3))
+            y_b = torch.empty(H, dtype=torch.float16, device=dev)
+            for fmt, key in (("q8_0_soa", "q8_0_soa"), ("q6_K", "q6_K")):
+                def chain(i):
+                    ws = sets[i % len(sets)]
+                    ops.quantize_q8_1(xf, xq_b)
+                    ops.gemv_q8_x2(fmt, xq_b, ws[(key, "gate")], ws[(key, "up")], H, FF, g_b, u_b)
+                    ops.swiglu_q8(g_b, u_b, out=(h_b, hq_b))
+                    gemv(key.replace("_soa", ""), hq_b, ws, "down", FF, H, y_b)
+
+                def fused(i):
+                    ws = sets[i % len(sets)]
+                    ops.gemv_x2_silu(fmt, xf, ws[(key, "gate")], ws[(key, "up")], H, FF, h_b)
+                    ops.gemv_f16q8(fmt, h_b, ws[(key, "down")], FF, H, y_b)
+
+                us_c, us_f = kernel_avg_us(chain, 2 * len(sets)), kernel_avg_us(fused, 2 * len(sets))
+                detail["ffn_decode_%s_T1" % fmt] = {"chain_4_launches_us": round(us_c, 2), "fused_2_launches_us": round(us_f, 2)}
+        if want('c1'):
+            # BASELINE config 1: Q4_K 4096x4096, fp32 activations, fp32 out (9.4 MB: cache resident unless rotated)
+            w1 = [synth.normal_weights("q4_K", 4096, 4096, seed=500 + i, device=dev) for i in range(40)]
+            a32 = torch.randn(4096, device=dev, generator=g)
+            y32 = torch.empty(4096, dtype=torch.float32, device=dev)
+            us = kernel_avg_us(lambda i: ops.gemv_q4_K(a32, w1[i % len(w1)], 4096, 4096, y32), 2 * len(w1))
+            b = 4096 * synth.row_bytes("q4_K", 4096) + 2 * 4096 * 4
+            detail["config1_q4_K_4096x4096_f32"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+            aq = ops.quantize_q8_1(a32)
+            y16 = torch.empty(4096, dtype=torch.float16, device=dev)
+            us = kernel_avg_us(lambda i: ops.gemv_q4_K_q8(aq, w1[i % len(w1)], 4096, 4096, y16), 2 * len(w1))
+            detail["config1_q4_K_4096x4096_q8"] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+            del w1
+        if want('lm_head'):
+            # lm_head-sized decode GEMV (the largest single GEMV of a decode step): Q6_K, 4096 -> 151936, 510 MB
+            NV = 151936
+            wl = [synth.normal_weights("q6_K", NV, H, seed=700 + i, device=dev) for i in range(2)]
+            yv = torch.empty(NV, dtype=torch.float16, device=dev)
+            us = kernel_avg_us(lambda i: ops.gemv_q6_K_q8(xq, wl[i % 2], H, NV, yv), 4)
+            b = gemv_bytes(synth.row_bytes("q6_K", H), H, NV, 1)
+            detail["lm_head_q6_K_K4096_N151936_T1"] = {"us": round(us, 1), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+            del wl, yv
+        if want('c3'):
+            # BASELINE config 3: prefill quant-GEMM, Q4_K, fp16 MFMA (peak 2.5 PFLOP/s dense fp16)
+            for (K, N) in ((H, FF), (FF, H)):
+                wq = synth.normal_weights("q4_K", N, K, seed=900, device=dev)
+                for T in (512, 2048, 4096):
+                    a16 = torch.randn((T, K), device=dev, generator=g).half()
+                    yg = torch.empty((T, N), dtype=torch.float16, device=dev)
+                    us = kernel_avg_us(lambda i: ops.gemm_q4_K(a16, wq, T, K, N, yg), 4)
+                    tf = 2.0 * T * N * K / us / 1e6
+                    ent = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
+                    if T >= 2048:
+                        # the same product the reference's way on this box: dequantize W to an fp16 [K, N] matrix, then the
+                        # vendor library's fp16 GEMM (rocBLAS here, oneDNN there); and that GEMM alone
+                        bt = ops.dequant_to_Bt("q4_K", wq, K, N)
+                        us_g = kernel_avg_us(lambda i: ops.gemm_fp16(a16, bt, T, N, K, torch.float16, yg), 4)
+                        us_2 = kernel_avg_us(lambda i: (ops.dequant_to_Bt("q4_K", wq, K, N, bt), ops.gemm_fp16(a16, bt, T, N, K, torch.float16, yg)), 4)
+                        ent["vendor_fp16_gemm_us"] = round(us_g, 1)
+                        ent["vendor_fp16_gemm_TFLOPs"] = round(2.0 * T * N * K / us_g / 1e6, 1)
+                        ent["dequant_plus_vendor_gemm_us"] = round(us_2, 1)
+                        del bt
+                    detail["config3_gemm_q4_K_T%d_K%d_N%d" % (T, K, N)] = ent
+                    del a16, yg
+                del wq
+        if want('c4'):
+            # BASELINE config 4: MXFP4 MoE decode at gpt-oss-20b shape (E=32, top-4, H=EF=2880), T=1 and T=32
+            E4, K4, H4 = 32, 4, 2880
+            nrep = 6   # rotate expert banks so a decode step cannot live in the Infinity Cache
+            banks = []
+            for i in range(nrep):
+                gq, ge = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3000 + i, device=dev))
+                uq, ue = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3100 + i, device=dev))
+                dq, de = synth.split_mxfp4(synth.normal_weights("mxfp4", E4 * H4, H4, seed=3200 + i, device=dev))
+                banks.append((gq, ge, uq, ue, dq, de))
+            qs_st, e_st = H4 * H4 // 2, H4 * H4 // 32
+            per_expert = 3 * (qs_st + e_st)
+            for T in (1, 32):
+                logits = rng.standard_normal((T, E4)).astype(np.float32)
+                ids = np.sort(np.argsort(-logits, axis=1)[:, :K4], axis=1).astype(np.int32)
+                wts = np.full((T, K4), 0.25, np.float32)
+                off, si, wp, t2p = ops.build_moe_packing(ids, wts, E4)
+                n_distinct = int((np.diff(off.astype(np.int64)) > 0).sum())
+                xt = torch.randn((T, H4), device=dev, generator=g).half()
+                TK = T * K4
+                offd, sid = torch.from_numpy(off).to(dev), torch.from_numpy(si).to(dev)
+                idsd = torch.from_numpy(ids.ravel().copy()).to(dev)
+                hbuf = torch.empty((TK, H4), dtype=torch.float16, device=dev)
+                obuf = torch.empty((TK, H4), dtype=torch.float16, device=dev)
+                xq8 = ops.quantize_q8_1(xt)
+                xpq = ops.quantize_q8_1(ops.moe_gather_rows(xt, sid, TK, H4))
+                hq8 = ops.quantize_q8_1(hbuf)
+
+                def layer(i):
+                    b = banks[i % nrep]
+                    if T == 1:    # device-side expert ids, one launch per stage
+                        ops.moe_gate_up_oai_mxfp4(xq8, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, idsd, T, K4, H4, H4, E4, h_out=hbuf)
+                        if args.unfused:
+                            ops.quantize_q8_1(hbuf, hq8)
+                            ops.moe_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
+                        else:     # h quantized while the down launch stages it: same bits, one launch fewer
+                            ops.moe_down_mxfp4_f16(hbuf, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
+                    else:         # expert-grouped rows, each routed expert streamed once
+                        ops.moe_grouped_gate_up_oai_mxfp4(xpq, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, offd, TK, E4, H4, H4, h_packed=hbuf)
+                        # with 128 rows every workgroup would requantize all of them: the separate quantize launch is cheaper here
                         ops.quantize_q8_1(hbuf, hq8)
-                        ops.moe_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
-                    else:     # h quantized while the down launch stages it: same bits, one launch fewer
-                        ops.moe_down_mxfp4_f16(hbuf, b[4], b[5], qs_st, e_st, None, idsd, T, K4, H4, H4, E4, out_packed=obuf)
-                else:         # expert-grouped rows, each routed expert streamed once
-                    ops.moe_grouped_gate_up_oai_mxfp4(xpq, b[0], b[1], b[2], b[3], qs_st, e_st, None, None, offd, TK, E4, H4, H4, h_packed=hbuf)
-                    # with 128 rows every workgroup would requantize all of them: the separate quantize launch is cheaper here
-                    ops.quantize_q8_1(hbuf, hq8)
-                    ops.moe_grouped_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, offd, TK, E4, H4, H4, out_packed=obuf)
+                        ops.moe_grouped_down_mxfp4(hq8, b[4], b[5], qs_st, e_st, None, offd, TK, E4, H4, H4, out_packed=obuf)
 
-            us = kernel_avg_us(layer, 2 * nrep)
-            bts = n_distinct * per_expert
-            detail["config4_moe_mxfp4_T%d" % T] = {"us": round(us, 1), "distinct_experts": n_distinct, "GBps": round(bts / us / 1e3, 1),
-                                                   "frac_hbm": round(bts / us / 1e3 / HBM_PEAK_GBS, 4)}
-        del banks
-        # BASELINE config 5: Qwen3-MoE style grouped GEMM, E=128 top-8 H=2048 EF=768, 2048 tokens, Zipf(1.1), Q8_0 experts
-        E5, K5, H5, EF5, T5 = 128, 8, 2048, 768, 2048
-        gq5, gd5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * EF5, H5, seed=5000, device=dev))
-        uq5, ud5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * EF5, H5, seed=5001, device=dev))
-        dq5, dd5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * H5, EF5, seed=5002, device=dev))
-        pz = np.arange(1, E5 + 1, dtype=np.float64) ** -1.1
-        pz = pz[rng.permutation(E5)]
-        pz /= pz.sum()
-        ids5 = np.stack([np.sort(rng.choice(E5, size=K5, replace=False, p=pz)) for _ in range(T5)]).astype(np.int32)
-        w5 = np.full(ids5.shape, 1.0 / K5, np.float32)
-        off5, si5, wp5, t2p5 = ops.build_moe_packing(ids5, w5, E5)
-        TK5 = T5 * K5
-        x5 = torch.randn((T5, H5), device=dev, generator=g).half()
-        off5d, wp5d = torch.from_numpy(off5).to(dev), torch.from_numpy(wp5).to(dev).half()
-        xp5 = ops.moe_gather_rows(x5[:, :].contiguous(), torch.from_numpy(si5).to(dev), TK5, H5) if TK5 <= 65535 else None
-        h5 = torch.empty((TK5, EF5), dtype=torch.float16, device=dev)
-        o5 = torch.empty((TK5, H5), dtype=torch.float16, device=dev)
+                us = kernel_avg_us(layer, 2 * nrep)
+                bts = n_distinct * per_expert
+                detail["config4_moe_mxfp4_T%d" % T] = {"us": round(us, 1), "distinct_experts": n_distinct, "GBps": round(bts / us / 1e3, 1),
+                                                       "frac_hbm": round(bts / us / 1e3 / HBM_PEAK_GBS, 4)}
+            del banks
+        if want('c5'):
+            # BASELINE config 5: Qwen3-MoE style grouped GEMM, E=128 top-8 H=2048 EF=768, 2048 tokens, Zipf(1.1), Q8_0 experts
+            E5, K5, H5, EF5, T5 = 128, 8, 2048, 768, 2048
+            gq5, gd5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * EF5, H5, seed=5000, device=dev))
+            uq5, ud5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * EF5, H5, seed=5001, device=dev))
+            dq5, dd5 = synth.split_q8_0(synth.normal_weights("q8_0", E5 * H5, EF5, seed=5002, device=dev))
+            pz = np.arange(1, E5 + 1, dtype=np.float64) ** -1.1
+            pz = pz[rng.permutation(E5)]
+            pz /= pz.sum()
+            ids5 = np.stack([np.sort(rng.choice(E5, size=K5, replace=False, p=pz)) for _ in range(T5)]).astype(np.int32)
+            w5 = np.full(ids5.shape, 1.0 / K5, np.float32)
+            off5, si5, wp5, t2p5 = ops.build_moe_packing(ids5, w5, E5)
+            TK5 = T5 * K5
+            x5 = torch.randn((T5, H5), device=dev, generator=g).half()
+            off5d, wp5d = torch.from_numpy(off5).to(dev), torch.from_numpy(wp5).to(dev).half()
+            xp5 = ops.moe_gather_rows(x5[:, :].contiguous(), torch.from_numpy(si5).to(dev), TK5, H5) if TK5 <= 65535 else None
+            h5 = torch.empty((TK5, EF5), dtype=torch.float16, device=dev)
+            o5 = torch.empty((TK5, H5), dtype=torch.float16, device=dev)
 
-        def layer5(i):
-            ops.moe_gemm_gate_up_silu_q8(xp5, gq5, gd5, uq5, ud5, EF5 * H5, EF5 * H5 // 32, off5d, TK5, E5, H5, EF5, h5)
-            ops.moe_gemm_down_q8(h5, dq5, dd5, H5 * EF5, H5 * EF5 // 32, off5d, wp5d, TK5, E5, H5, EF5, o5)
+            def layer5(i):
+                ops.moe_gemm_gate_up_silu_q8(xp5, gq5, gd5, uq5, ud5, EF5 * H5, EF5 * H5 // 32, off5d, TK5, E5, H5, EF5, h5)
+                ops.moe_gemm_down_q8(h5, dq5, dd5, H5 * EF5, H5 * EF5 // 32, off5d, wp5d, TK5, E5, H5, EF5, o5)
 
-        us = kernel_avg_us(layer5, 3)
-        tf = 2.0 * TK5 * H5 * EF5 * 3 / us / 1e6
-        detail["config5_moe_grouped_gemm_q8_0"] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4)}
+            us = kernel_avg_us(layer5, 3)
+            tf = 2.0 * TK5 * H5 * EF5 * 3 / us / 1e6
+            detail["config5_moe_grouped_gemm_q8_0"] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4),
+                                                       "route": "fp16 rows, fp16 MFMA (mx_moe_gemm_*)"}
+            # the same layer through the reference's own signatures: q8 rows (quantize_q8_1) -> moe_prefill_gate_up_silu_q8 ->
+            # quantize_q8_1 -> moe_prefill_down_q8, int8 MFMA with the per-block fp32 fold (peak 5 POP/s dense int8)
+            xq5 = torch.empty(TK5 * (H5 // 32) * 40, dtype=torch.uint8, device=dev)
+            hq5 = torch.empty(TK5 * (EF5 // 32) * 40, dtype=torch.uint8, device=dev)
+
+            def layer5_q8(i):
+                ops.quantize_q8_1(xp5, xq5)
+                ops.moe_prefill_gate_up_silu_q8(xq5, gq5, gd5, uq5, ud5, EF5 * H5, EF5 * H5 // 32, off5d, TK5, E5, H5, EF5, h5)
+                ops.quantize_q8_1(h5, hq5)
+                ops.moe_prefill_down_q8(hq5, dq5, dd5, H5 * EF5, H5 * EF5 // 32, off5d, wp5d, TK5, E5, H5, EF5, o5)
+
+            us8 = kernel_avg_us(layer5_q8, 3)
+            to8 = 2.0 * TK5 * H5 * EF5 * 3 / us8 / 1e6
+            detail["config5_moe_grouped_q8_rows"] = {"us": round(us8, 1), "TOPs": round(to8, 1), "frac_int8_mfma": round(to8 / 5000.0, 4),
+                                                     "route": "q8 rows through the reference's signatures, int8 MFMA + fp32 fold (incl. the two quantize launches)"}
         out["detail"] = detail
 
     # ---------------------------------------------------------------- CPU baseline (reported only)

@@ -689,7 +689,9 @@ static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, in
     if constexpr (!std::is_void<P>::value && std::is_same<OutT, half_t>::value) {
         // measured crossover against the vector-ALU batch kernels (4096 -> 14336, us): Q8_0 planes T = 4: 15.4 vs 16.1,
         // T = 8: 20.4 vs 17.6; Q6_K T = 8: 26.2 vs 22.0; batches of 9 .. 16 take one pass here instead of two there
-        if (T >= 5 && nseg == 1 && !s0.bias) return launch_mmq_dense<P>(as_stream(s), mmq_bank(s0.w), x, s0.y, K, N, T, split, ws);
+        // (GGUF Q8_0 blocks: the 2-byte aligned block walk loses below a full second pass, 24.4 vs 30.9 us at T = 8)
+        constexpr uint32_t kMmqFromT = std::is_same<F, FmtQ8Aos>::value ? 9u : 5u;
+        if (T >= kMmqFromT && nseg == 1 && !s0.bias) return launch_mmq_dense<P>(as_stream(s), mmq_bank(s0.w), x, s0.y, K, N, T, split, ws);
     }
     for (uint32_t t0 = 0; t0 < T; t0 += 8) {
         const uint32_t tn = (T - t0 < 8) ? T - t0 : 8;

@@ -336,17 +336,18 @@ static int launch_moe(mx_stream_t s, const typename F::Bank& b0, const typename 
 // ---------------------------------------------------------------- expert-grouped rows on the matrix cores (mxq_mmq.h)
 // grid (blocks of 32 WR weight rows, experts): a workgroup walks its expert's rows in passes of 2 TV tokens; its slice of
 // the expert's weights (32 WR rows) is re-read from L2 by every pass after the first.
-constexpr uint32_t kMmqMoeLdsBudget = 48 * 1024;
+constexpr uint32_t kMmqMoeLdsBudget = 48 * 1024, kMmqMoeLdsBudgetBig = 78 * 1024;   // the larger one for 32-token passes (opt-in above 64 KB)
 
 template <class P, int TV, int NW, int WR, int WK, int EPI>
-static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, const typename P::Bank& b1, const MoeArgs& m, uint32_t E) {
+static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, const typename P::Bank& b1, const MoeArgs& m, uint32_t E, uint32_t avg) {
     MmqArgs<P> a{};
     a.bank0 = b0; a.bank1 = b1; a.xq8 = m.xq8; a.expert_offsets = m.expert_offsets; a.out = m.out; a.bias0 = m.bias0; a.bias1 = m.bias1;
     a.route_w = m.route_w; a.alpha = m.alpha; a.limit = m.limit; a.M = 0; a.K = m.K; a.N = m.N; a.E = E; a.q8_split = m.q8_split;
     a.act_f16 = m.act_f16;
     constexpr uint32_t TT = 2 * TV, gran = 256u * WK;
     const uint32_t per256 = TT * 256u + 8u * TT * 4u * (P::HAS_MIN ? 2u : 1u);
-    uint32_t kr = (kMmqMoeLdsBudget - 32u * TT) / per256 * 256u / gran * gran;
+    const uint32_t budget = TV == 16 ? kMmqMoeLdsBudgetBig : kMmqMoeLdsBudget;
+    uint32_t kr = (budget - 32u * TT) / per256 * 256u / gran * gran;
     if (!kr) kr = gran;
     const uint32_t need = ((m.K + 255u) / 256u + WK - 1u) / WK * WK * 256u;
     if (kr > need) kr = need;
@@ -356,7 +357,26 @@ static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, co
     if (lds < red) lds = red;
     const uint32_t rgs = (m.N + 32u * WR - 1u) / (32u * WR);
     if (E > 65535u) return MX_ERR_SHAPE;
-    hipLaunchKernelGGL((mmq_kernel<P, TV, NW, WR, WK, EPI>), dim3(rgs, E, 1), dim3(64 * NW * WR * WK), lds, st, a);
+    if (lds > 64u * 1024u) {
+        static bool attr_set = false;   // LDS above the 64 KB default limit: opt in once per kernel
+        if (!attr_set) {
+            const hipError_t er = hipFuncSetAttribute(reinterpret_cast<const void*>(&mmq_kernel<P, TV, NW, WR, WK, EPI>),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMmqMoeLdsBudgetBig);
+            if (er != hipSuccess) {
+                g_last_hip_error = (int)er;
+                return MX_ERR_LAUNCH;
+            }
+            attr_set = true;
+        }
+    }
+    // token tiles of an expert are dealt over gridDim.z workgroups: the expert sizes live on the device and are skewed (a few
+    // experts hold most rows), so the split is sized for experts several times the average; workgroups without a tile leave at once
+    uint32_t zt = 1;
+    if (avg == 0 || avg > TT) {
+        zt = avg ? (4u * avg + TT - 1u) / TT : 8u;
+        if (zt > 32u) zt = 32u;
+    }
+    hipLaunchKernelGGL((mmq_kernel<P, TV, NW, WR, WK, EPI>), dim3(rgs, E, zt), dim3(64 * NW * WR * WK), lds, st, a);
     return launch_status();
 }
 
@@ -364,9 +384,9 @@ static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, co
 template <class P, int NW, int EPI>
 static int launch_mmq_grouped(mx_stream_t s, const typename P::Bank& b0, const typename P::Bank& b1, const MoeArgs& m, uint32_t E, uint32_t avg_rows) {
     hipStream_t st = as_stream(s);
-    if (avg_rows && avg_rows <= 8) return launch_mmq_grouped_cfg<P, 4, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E);
-    if (avg_rows && avg_rows <= 16) return launch_mmq_grouped_cfg<P, 8, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E);
-    return launch_mmq_grouped_cfg<P, 16, NW, (NW == 1 ? 4 : 2), 1, EPI>(st, b0, b1, m, E);
+    if (avg_rows && avg_rows <= 8) return launch_mmq_grouped_cfg<P, 4, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E, avg_rows);
+    if (avg_rows && avg_rows <= 16) return launch_mmq_grouped_cfg<P, 8, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E, avg_rows);
+    return launch_mmq_grouped_cfg<P, 16, NW, (NW == 1 ? 4 : 2), 1, EPI>(st, b0, b1, m, E, avg_rows);
 }
 
 // rows per token tile in grouped mode: expected rows per expert, rounded up to 4 or 8

@@ -633,14 +633,18 @@ __global__ __launch_bounds__(64 * NW * WR * WK, 2) void mmq_kernel(MmqArgs<P> a)
     const uint32_t nb = a.K / 32u, n_groups = (nb + 7u) / 8u;
     const uint32_t n0 = (blockIdx.x * WR + wr) * 32u;
     const uint32_t n = n0 + j < a.N ? n0 + j : a.N - 1u;
-    // K range of this workgroup (dense launches may split K over gridDim.z), walked in passes of kr elements
-    const uint32_t gz = (n_groups + gridDim.z - 1u) / gridDim.z;
-    const uint32_t G0 = blockIdx.z * gz, G1 = G0 + gz < n_groups ? G0 + gz : n_groups;
+    // gridDim.z: dense launches split K into ranges (partial sums to `part`); grouped launches deal the token tiles of an
+    // expert round-robin, so that an expert with many rows is spread over many workgroups
+    const bool grouped = a.expert_offsets != nullptr;
+    const uint32_t kz = grouped ? 1u : gridDim.z, kzi = grouped ? 0u : blockIdx.z;
+    const uint32_t gz = (n_groups + kz - 1u) / kz;
+    const uint32_t G0 = kzi * gz, G1 = G0 + gz < n_groups ? G0 + gz : n_groups;
+    const uint32_t t_step = grouped ? gridDim.z * 2u * TV : 2u * TV, t_first = grouped ? blockIdx.z * 2u * TV : 0u;
     const uint32_t gp = a.kr / 256u;                     // groups per pass (multiple of WK)
     const size_t q8_row_bytes = (size_t)nb * (a.q8_split ? kQ81sBytes : kQ81xBytes);
     float* red = reinterpret_cast<float*>(lds);          // [NWAVES][TV][64] partial sums, after the last pass (reuses the plane)
 
-    for (uint32_t t0 = r_begin; t0 < r_end; t0 += TT) {
+    for (uint32_t t0 = r_begin + t_first; t0 < r_end; t0 += t_step) {
         const uint32_t nt = r_end - t0 < TT ? r_end - t0 : TT;
         auto xrow = [&](uint32_t t) { return a.xq8 + (size_t)(t0 + t) * q8_row_bytes; };
         float acc[TV];
@@ -681,7 +685,7 @@ __global__ __launch_bounds__(64 * NW * WR * WK, 2) void mmq_kernel(MmqArgs<P> a)
                 if (t >= nt || n0 + j >= a.N) continue;
                 const uint32_t row = t0 + t, col = n0 + j;
                 if (a.part) {
-                    a.part[((size_t)blockIdx.z * a.M + row) * a.N + col] = s0;
+                    a.part[((size_t)kzi * a.M + row) * a.N + col] = s0;
                     continue;
                 }
                 float o;

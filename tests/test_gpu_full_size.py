@@ -147,3 +147,23 @@ def test_config5_grouped_gemm_full_size(mx):
     y_ref = op_h[t2p_r].reshape(T, Kt, Hm).sum(axis=1)
     check(host(y).astype(np.float32), y_ref, "C5 reduce_sum")
     assert np.isfinite(hp_h).all() and np.isfinite(op_h).all()
+    # ---- the same layer through the reference's own q8 signatures (include/ie/moe_q8.hpp:51-72): block_q8_1x rows in,
+    # int-dot on the matrix cores, against the q8-chain oracle
+    xq = ops.quantize_q8_1(xp)
+    hq8 = ops.moe_prefill_gate_up_silu_q8(xq, gq, gd, uq, ud, EF * Hm, EF * Hm // 32, off, TK, E, Hm, EF)
+    hqq = ops.quantize_q8_1(hq8)
+    oq8 = ops.moe_prefill_down_q8(hqq, dq, dd, Hm * EF, Hm * EF // 32, off, wp, TK, E, Hm, EF)
+    xq_h, hq_h = host(xq).reshape(TK, -1), host(hqq).reshape(TK, -1)
+    hq8_h, oq8_h = host(hq8).astype(np.float32), host(oq8).astype(np.float32)
+    assert np.array_equal(hq_h.ravel(), O.quantize_q8_1(hq8_h))
+    for e in experts:
+        if counts[e] == 0:
+            continue
+        rr = off_r[e] + np.unique(np.concatenate([[0, counts[e] - 1], rng.integers(0, counts[e], 3)]))
+        g = O.gemv_q8chain(O.Q8_0, g_h[e], xq_h[rr], Hm, EF)
+        u = O.gemv_q8chain(O.Q8_0, u_h[e], xq_h[rr], Hm, EF)
+        check(hq8_h[rr], O.swiglu_np(g.astype(np.float32), u.astype(np.float32)), "C5 q8 rows, gate_up expert %d (%d rows)" % (e, counts[e]))
+        o = O.gemv_q8chain(O.Q8_0, d_h[e], hq_h[rr], EF, Hm) * wp_r[rr][:, None]
+        check(oq8_h[rr], o, "C5 q8 rows, down expert %d" % e)
+    # rows of experts nobody sampled: finite, and every row written (the buffers come from torch.empty)
+    assert np.isfinite(hq8_h).all() and np.isfinite(oq8_h).all()
