@@ -433,6 +433,43 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
         }
     }
     bool staged = false;
+    // One K tile that one staging round covers (16 floats per thread): request the activation chunk, then the first row
+    // group's weight units, and only then touch the activations.  Loads return in order, so the wait for the chunk
+    // leaves the younger weight requests in flight while the row is written to LDS.
+    typename F::Raw pre[R];
+    const bool lead = n_tiles == 1 && K <= 16u * kGemvThreads && blockIdx.x < n_rg;
+    const bool pre_live = lead && gl < (K + 63) / 64 && (K & 63u) == 0;
+    if (lead) {
+        float v[16];
+        const uint32_t i = threadIdx.x;
+        const bool live = i < (K + 63) / 64 * 4;
+        if (live && i * 16 < K) {
+            load16(A + i * 16, v);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) v[j] = 0.f;
+        }
+        if (pre_live) {
+            const uint32_t prow0 = blockIdx.x * ROWS_PER_WG + (wave * GROUPS + grp) * (PAIR ? 1 : R);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t row = PAIR ? prow0 : prow0 + r;
+                const typename F::Cursor c = F::cursor((PAIR && r) ? w1 : w, row < N ? row : N - 1, gl);
+                pre[r] = load_unit<F, G>(c, 0, false);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (live) {
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) sum += v[j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) reinterpret_cast<float4*>(xa)[fact_slot(i * 4 + j)] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
+            s16[i] = sum;
+        }
+        __syncthreads();
+        staged = true;
+    }
     for (uint32_t rg = blockIdx.x; rg < n_rg; rg += n_wg) {
         const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * (PAIR ? 1 : R);
         float acc[R];
@@ -458,7 +495,10 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fact_kernel(typename F::W w
                 const uint32_t ul = it * G + gl, e0 = F::elem_off(ul);
                 typename F::Raw raw[R];
 #pragma unroll
-                for (int r = 0; r < R; ++r) raw[r] = load_unit<F, G>(cu[r], it, half_tail && ul == n_units - 1);
+                for (int r = 0; r < R; ++r) {
+                    if (pre_live && it == 0 && rg == blockIdx.x) raw[r] = pre[r];
+                    else raw[r] = load_unit<F, G>(cu[r], it, half_tail && ul == n_units - 1);
+                }
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     acc[r] += fact_unit<F>(raw[r], cu[r], xa, s16, e0);

@@ -281,6 +281,10 @@ __device__ __forceinline__ void load16(const float* p, float (&v)[16]) {
         for (int j = 0; j < 16; ++j) v[j] = p[j];
     }
 }
+// The staged row is kept in 16-byte slots, slot q stored at q ^ ((q >> 4) & 15).  A lane's unit is 64 consecutive
+// floats, so without the permutation the 64 lanes of a ds_read_b128 all fall on the same four banks (lane stride 256 B);
+// with it the 16 lanes served together read 16 different slots (Q4_K-style units) or 8 (Q6_K's interleaved units).
+__device__ __forceinline__ uint32_t fact_slot(uint32_t q) { return q ^ ((q >> 4) & 15u); }
 template <class ActT>
 __device__ __forceinline__ void stage_fact(float* xa, float* s16, const ActT* A, uint32_t kt) {
     for (uint32_t i = threadIdx.x; i < (kt + 63) / 64 * 4; i += blockDim.x) {
@@ -295,7 +299,7 @@ __device__ __forceinline__ void stage_fact(float* xa, float* s16, const ActT* A,
 #pragma unroll
         for (int j = 0; j < 16; ++j) s += v[j];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) reinterpret_cast<float4*>(xa + i * 16)[j] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
+        for (int j = 0; j < 4; ++j) reinterpret_cast<float4*>(xa)[fact_slot(i * 4 + j)] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
         s16[i] = s;
     }
 }
@@ -311,7 +315,7 @@ __device__ __forceinline__ float fact_unit(const typename F::Raw& raw, const typ
         float dq = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float4 x = *reinterpret_cast<const float4*>(xa + eg + 4 * i);
+            const float4 x = reinterpret_cast<const float4*>(xa)[fact_slot((eg >> 2) + i)];
             dq += x.x * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 0) + x.y * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 1) +
                   x.z * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 2) + x.w * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 3);
         }
