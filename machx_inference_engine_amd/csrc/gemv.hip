@@ -697,9 +697,9 @@ static int launch_mmq_dense_cfg(hipStream_t st, const typename P::Bank& bank, co
     MmqArgs<P> a{};
     a.bank0 = bank; a.bank1 = bank; a.xq8 = xq8; a.out = y; a.part = Z > 1 ? ws.ptr : nullptr;
     a.M = T; a.K = K; a.N = N; a.E = 1; a.q8_split = split ? 1u : 0u; a.kr = kr;
-    uint32_t lds = mmq_lds_bytes(T, kr, TV, P::HAS_MIN);
     const uint32_t red = (uint32_t)(WR * WK) * TV * 64u * 4u;
-    if (lds < red) lds = red;
+    a.red_off = (mmq_lds_bytes(T, kr, TV, P::HAS_MIN) + 15u) & ~15u;
+    const uint32_t lds = a.red_off + red;
     hipLaunchKernelGGL((mmq_kernel<P, TV, 1, WR, WK, MMQ_STORE>), dim3(rgs, 1, Z), dim3(64 * WR * WK), lds, st, a);
     if (Z > 1) {
         const uint32_t mn = T * N;

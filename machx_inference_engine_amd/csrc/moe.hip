@@ -340,21 +340,22 @@ constexpr uint32_t kMmqMoeLdsBudget = 48 * 1024, kMmqMoeLdsBudgetBig = 78 * 1024
 
 template <class P, int TV, int NW, int WR, int WK, int EPI>
 static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, const typename P::Bank& b1, const MoeArgs& m, uint32_t E, uint32_t avg) {
+    constexpr bool NATIVE = mmq_native<P>::value;
     MmqArgs<P> a{};
     a.bank0 = b0; a.bank1 = b1; a.xq8 = m.xq8; a.expert_offsets = m.expert_offsets; a.out = m.out; a.bias0 = m.bias0; a.bias1 = m.bias1;
     a.route_w = m.route_w; a.alpha = m.alpha; a.limit = m.limit; a.M = 0; a.K = m.K; a.N = m.N; a.E = E; a.q8_split = m.q8_split;
     a.act_f16 = m.act_f16;
     constexpr uint32_t TT = 2 * TV, gran = 256u * WK;
-    const uint32_t per256 = TT * 256u + 8u * TT * 4u * (P::HAS_MIN ? 2u : 1u);
-    const uint32_t budget = TV == 16 ? kMmqMoeLdsBudgetBig : kMmqMoeLdsBudget;
+    constexpr uint32_t red = (uint32_t)(NW * WR * WK) * TV * 64u * 4u;
+    const uint32_t per256 = TT * (NATIVE ? 512u : 256u) + 8u * TT * 4u * (P::HAS_MIN ? 2u : 1u);
+    const uint32_t budget = ((TV == 16 || (NATIVE && TV == 8)) ? kMmqMoeLdsBudgetBig : (NATIVE ? 64u * 1024u : kMmqMoeLdsBudget)) - red;
     uint32_t kr = (budget - 32u * TT) / per256 * 256u / gran * gran;
     if (!kr) kr = gran;
     const uint32_t need = ((m.K + 255u) / 256u + WK - 1u) / WK * WK * 256u;
     if (kr > need) kr = need;
     a.kr = kr;
-    uint32_t lds = mmq_lds_bytes(TT, kr, TV, P::HAS_MIN);
-    const uint32_t red = (uint32_t)(NW * WR * WK) * TV * 64u * 4u;
-    if (lds < red) lds = red;
+    a.red_off = (mmq_lds_bytes(TT, kr, TV, P::HAS_MIN, NATIVE) + 15u) & ~15u;
+    const uint32_t lds = a.red_off + red;
     const uint32_t rgs = (m.N + 32u * WR - 1u) / (32u * WR);
     if (E > 65535u) return MX_ERR_SHAPE;
     if (lds > 64u * 1024u) {
@@ -371,12 +372,20 @@ static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, co
     }
     // token tiles of an expert are dealt over gridDim.z workgroups: the expert sizes live on the device and are skewed (a few
     // experts hold most rows), so the split is sized for experts several times the average; workgroups without a tile leave at once
-    uint32_t zt = 1;
+    uint32_t zt = 2;   // even with small experts a few hold more rows than one tile: their second tile gets a workgroup of its own
     if (avg == 0 || avg > TT) {
         zt = avg ? (4u * avg + TT - 1u) / TT : 8u;
         if (zt > 32u) zt = 32u;
     }
-    hipLaunchKernelGGL((mmq_kernel<P, TV, NW, WR, WK, EPI>), dim3(rgs, E, zt), dim3(64 * NW * WR * WK), lds, st, a);
+    // workgroups per expert along the weight rows: when the staged image covers K, about two resident workgroups per CU in
+    // all, each streaming several row blocks against its one image; otherwise one workgroup per row block
+    uint32_t gx = rgs;
+    if (kr >= need && avg && avg <= TT) {   // known, small experts only: with skewed or unknown sizes the row blocks stay spread
+        const uint64_t slots = 2ull * (uint64_t)cu_count_moe();
+        const uint32_t per = (uint32_t)(((uint64_t)rgs * E + slots - 1u) / slots);   // nearly every expert has one tile
+        if (per > 1u) gx = (rgs + per - 1u) / per;
+    }
+    hipLaunchKernelGGL((mmq_kernel<P, TV, NW, WR, WK, EPI>), dim3(gx, E, zt), dim3(64 * NW * WR * WK), lds, st, a);
     return launch_status();
 }
 
@@ -386,7 +395,8 @@ static int launch_mmq_grouped(mx_stream_t s, const typename P::Bank& b0, const t
     hipStream_t st = as_stream(s);
     if (avg_rows && avg_rows <= 8) return launch_mmq_grouped_cfg<P, 4, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E, avg_rows);
     if (avg_rows && avg_rows <= 16) return launch_mmq_grouped_cfg<P, 8, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E, avg_rows);
-    return launch_mmq_grouped_cfg<P, 16, NW, (NW == 1 ? 4 : 2), 1, EPI>(st, b0, b1, m, E, avg_rows);
+    if constexpr (mmq_native<P>::value) return launch_mmq_grouped_cfg<P, 8, NW, 1, 4 / NW, EPI>(st, b0, b1, m, E, avg_rows);   // passes of at most 16 tokens
+    else return launch_mmq_grouped_cfg<P, 16, NW, (NW == 1 ? 4 : 2), 1, EPI>(st, b0, b1, m, E, avg_rows);
 }
 
 // rows per token tile in grouped mode: expected rows per expert, rounded up to 4 or 8
@@ -600,7 +610,8 @@ static int moe_mxfp4_gate_up(mx_stream_t s, const void* x_q8, const uint8_t* g_q
     a.xq8 = static_cast<const uint8_t*>(x_q8); a.topk_idx = topk_idx; a.expert_offsets = expert_offsets; a.bias0 = gate_bias; a.bias1 = up_bias;
     a.out = reinterpret_cast<half_t*>(h_out); a.alpha = alpha; a.limit = limit; a.act_div = act_div; a.K = H; a.N = E_ffn; a.n_experts = n_experts;
     FmtMxfp4Soa::Bank bg{g_qs, g_e, qs_stride, e_stride, H}, bu{u_qs, u_e, qs_stride, e_stride, H};
-    if (expert_offsets) return launch_mmq_grouped<MmqMxfp4Soa, 2, MMQ_OAI>(s, bg, bu, a, n_seg, tt);   // grouped: tt = expected rows per expert
+    if (expert_offsets && H >= 256) return launch_mmq_grouped<MmqMxfp4Native, 2, MMQ_OAI>(s, bg, bu, a, n_seg, tt);   // grouped: tt = expected rows per expert
+    if (expert_offsets) return launch_mmq_grouped<MmqMxfp4Soa, 2, MMQ_OAI>(s, bg, bu, a, n_seg, tt);
     return launch_moe<FmtMxfp4Soa, 2, EPI_OAI>(s, bg, bu, a, n_seg, tt);
 }
 int mx_moe_gate_up_oai_mxfp4(mx_stream_t s, const void* x_q8, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
@@ -632,7 +643,8 @@ static int moe_mxfp4_down(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, 
     a.out = reinterpret_cast<half_t*>(out_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
     if (act_is_f16) a.act_f16 = static_cast<const half_t*>(h_q8);
     FmtMxfp4Soa::Bank b{d_qs, d_e, qs_stride, e_stride, E_ffn};
-    if (expert_offsets) return launch_mmq_grouped<MmqMxfp4Soa, 1, MMQ_DOWN_BIAS>(s, b, b, a, n_seg, tt);   // grouped: tt = expected rows per expert
+    if (expert_offsets && E_ffn >= 256) return launch_mmq_grouped<MmqMxfp4Native, 1, MMQ_DOWN_BIAS>(s, b, b, a, n_seg, tt);   // grouped: tt = expected rows per expert
+    if (expert_offsets) return launch_mmq_grouped<MmqMxfp4Soa, 1, MMQ_DOWN_BIAS>(s, b, b, a, n_seg, tt);
     return launch_moe<FmtMxfp4Soa, 1, EPI_DOWN_BIAS>(s, b, b, a, n_seg, tt);
 }
 int mx_moe_down_mxfp4(mx_stream_t s, const void* h_q8, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,

@@ -38,6 +38,13 @@ struct ActTile {
     uint32_t KT;
 };
 
+// Where 16-quant chunk q of a staged row lives.  A lane reads the chunks facing its 64-element unit, so lanes sit 64 B
+// apart (units of consecutive elements) and the 16 lanes one ds_read_b128 pass serves would share four bank groups; the
+// XOR spreads them over all sixteen.  Units of consecutive elements (every format but Q6_K) permute the four chunks inside
+// a unit; Q6_K's units interleave two 128-element halves (K is a multiple of 256 there), so the bits one up are used.
+template <int SUM_GRAN>
+__device__ __forceinline__ uint32_t act_slot(uint32_t q) { return q ^ (((q >> 4) & 3u) << (SUM_GRAN == 16 ? 1 : 0)); }
+
 // Stage T q8_1 rows, elements [k0, k0+kt), into LDS.  `xrow(t)` -> pointer to
 // the first block of activation row t.  All threads of the block call this.
 // split = false: block_q8_1x {d, s, qs[32]} (40 B); the per-16 sums of SUM_GRAN 16 are
@@ -68,7 +75,7 @@ __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t 
                 ds = *reinterpret_cast<const float2*>(blk);
             }
         }
-        qs[(size_t)t * (KT_alloc / 16) + hb] = make_uint4(q0.x, q0.y, q1.x, q1.y);
+        qs[(size_t)t * (KT_alloc / 16) + act_slot<SUM_GRAN>(hb)] = make_uint4(q0.x, q0.y, q1.x, q1.y);
         if (SUM_GRAN == 16) {
             float sh = s_half;
             if (!split) {
@@ -136,7 +143,7 @@ __device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint3
         }
         const int s32 = s16 + __shfl_xor(s16, 1);
         if (!in) continue;
-        qs[(size_t)t * (KT_alloc / 16) + hb] = make_uint4(q[0], q[1], q[2], q[3]);
+        qs[(size_t)t * (KT_alloc / 16) + act_slot<SUM_GRAN>(hb)] = make_uint4(q[0], q[1], q[2], q[3]);
         if (SUM_GRAN == 16) {
             reinterpret_cast<float2*>(hdr)[(size_t)t * (KT_alloc / 16) + hb] = make_float2(d, d * (float)s16);
         } else if ((hb & 1u) == 0) {
@@ -169,7 +176,7 @@ __device__ __forceinline__ void gemv_step(const typename F::Raw (&raw)[R], const
     for (int t = 0; t < T; ++t) {
         uint4 x[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) x[g] = act.qs[(size_t)t * (act.KT / 16) + ((e0 + g * F::GROUP_OFF) >> 4)];
+        for (int g = 0; g < 4; ++g) x[g] = act.qs[(size_t)t * (act.KT / 16) + act_slot<F::SUM_GRAN>((e0 + g * F::GROUP_OFF) >> 4)];
         if (F::PAIRED) {
             // groups (0,1) and (2,3): one activation block and one weight scale each
             float d0, d1, s0 = 0.f, s1 = 0.f;

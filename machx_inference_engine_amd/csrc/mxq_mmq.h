@@ -24,12 +24,20 @@
 // few rows) meet in a scratch plane that a second launch reduces.
 #pragma once
 
+#include <type_traits>
+
 #include "mxq_formats.h"
 
 namespace mxq {
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef int v8i_t __attribute__((ext_vector_type(8)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
+typedef float v16f_t __attribute__((ext_vector_type(16)));
+
+// producers that feed the scaled FP8 x FP4 matrix instruction declare NATIVE_FP4
+template <class P, class = void> struct mmq_native : std::false_type {};
+template <class P> struct mmq_native<P, std::void_t<decltype(P::NATIVE_FP4)>> : std::true_type {};
 
 __device__ __forceinline__ v4i_t as_v4i(const uint4& u) {
     v4i_t r;
@@ -211,6 +219,62 @@ struct MmqMxfp4Soa {
     }
 };
 
+// MXFP4 planes fed to the matrix cores as they lie in memory: v_mfma_scale_f32_32x32x64_f8f6f4 takes E2M1 codes and one
+// E8M0 scale per lane and 32 k-values, which is exactly a block of this format (include/ie/quant_blocks.hpp:46-54), so
+// there is no code -> integer conversion at all.  The q8 activation codes go in as two FP8 (E4M3) operands, q = 16 hi + lo
+// with hi = q >> 4 in -8..7 and lo = q & 15, both exact in E4M3; the hi instruction runs with the scale 2^4 and both
+// accumulate into the same registers, so the instruction pair returns 2^(e-127) * sum_k e2m1(w_k) * q_k exactly (every
+// partial sum is a small multiple of 2^(e-128)), the same number as weight-scale x integer dot of the vector kernels.
+// What the fold still does per block is the multiplication by the activation block scale d_x, which is not a power of two.
+//
+// Operand geometry (measured on gfx950 with one-hot operands): the instruction sums K = 64 in four groups of 16; an FP4
+// lane (column j, half h) holds groups 2h and 2h+1 as 32 consecutive nibbles (low nibble first), an FP8 lane (row i, half
+// h) holds group h in bytes 0..15 and group 2 + h in bytes 16..31.  So lane half h of the weight operand carries the whole
+// block 2 s + h of pair s, and the token rows are arranged so that the two blocks of a pair land in different result rows:
+// rows 0..15 = up to 16 tokens against block 2 s (bytes 16..31 of their operand are zero), rows 16..31 = the same tokens
+// against block 2 s + 1 (bytes 0..15 zero).  Result registers v < 8 of lane (j, h) are then tokens 8 (v / 4) + 4 h + v % 4
+// for block 2 s and registers 8 + v the same tokens for block 2 s + 1.
+struct MmqMxfp4Native {
+    using W = FmtMxfp4Soa::W;
+    using Bank = FmtMxfp4Soa::Bank;
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return FmtMxfp4Soa::expert(b, e); }
+    static constexpr bool NATIVE_FP4 = true;
+    static constexpr int SUBS = 1;
+    static constexpr bool HAS_MIN = false;
+    static constexpr uint32_t K_ALIGN = 32;
+    struct Raw {
+        uint4 q[4];       // blocks h, 2 + h, 4 + h, 6 + h of the group
+        uint32_t e[2];    // the eight exponents of the group; lane half h uses bytes h and 2 + h of e[s / 2]
+    };
+    // Nothing is computed on the loaded words here (that would make the request wait for them).  A partial last group
+    // (block count not a multiple of 8) re-reads the row's last block for its dead blocks and takes the eight exponent
+    // bytes that end at the row end; the staged activations of dead blocks are zero, so whatever they hold adds nothing.
+    // live = false: every lane reads the same valid bytes (the loads of a pipeline slot past the end of the walk).
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t g, uint32_t h, uint32_t nb, bool live = true) {
+        const uint8_t* row = w.qs + (size_t)n * (w.K >> 1);
+        const uint32_t last = nb - 1u, e_at = 8u * g + 8u <= nb ? 8u * g : nb - 8u;
+        const uint8_t* e = live ? w.e + (size_t)n * nb + e_at : w.e;
+        Raw r;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const uint32_t b = 8u * g + 2u * s + h;
+            r.q[s] = *reinterpret_cast<const uint4*>(live ? row + (size_t)(b < last ? b : last) * 16u : w.qs);
+        }
+        const uint2 ee = load_u2_a1(e);
+        r.e[0] = ee.x;
+        r.e[1] = ee.y;
+        return r;
+    }
+    // exponent byte of pair S for lane half h (block 2 S + h of group g), moved to byte 0
+    template <int S>
+    __device__ static __forceinline__ int scale_word(const Raw& r, uint32_t g, uint32_t h, uint32_t nb) {
+        const uint32_t skew = 8u * g + 8u <= nb ? 0u : 8u * g + 8u - nb;   // bytes the partial group's exponent window was moved down
+        const uint64_t all = ((uint64_t)r.e[1] << 32) | r.e[0];
+        const uint32_t at = skew + 2u * S + h;                             // past the window for a dead block: any valid byte will do
+        return (int)(uint32_t)(all >> (8u * (at < 7u ? at : 7u)));
+    }
+};
+
 // Q4_K AoS blocks: group g = block g of the row; sub-block s = nibble (s & 1) of qs[32 (s / 2) + l], l = 0..31
 // (include/ie/dequant_ref.hpp:38-53); lane half h owns l = 16 h .. 16 h + 15.  Codes stay unsigned (0..15); the min
 // term folds on the stored block sum of the activation row.
@@ -359,14 +423,53 @@ struct MmqAct {
     const float* sx;
     uint32_t stride;   // plane row pitch in bytes
 };
-__host__ __device__ constexpr uint32_t mmq_lds_bytes(uint32_t T, uint32_t kr, int TV, bool has_min) {
-    return T * (kr + 32u) + (kr / 32u) * (uint32_t)(2 * TV) * 4u * (has_min ? 2u : 1u);
+__host__ __device__ constexpr uint32_t mmq_row_pitch(uint32_t kr, bool native) { return native ? 2u * kr + 16u : kr + 32u; }
+__host__ __device__ constexpr uint32_t mmq_lds_bytes(uint32_t T, uint32_t kr, int TV, bool has_min, bool native = false) {
+    return T * mmq_row_pitch(kr, native) + (kr / 32u) * (uint32_t)(2 * TV) * 4u * (has_min ? 2u : 1u);
 }
 
-template <int TV, bool HAS_MIN, class RowFn>
+// Four 4-bit values (one per byte) through a 16-entry byte table: two byte permutes over the table halves, a third one
+// takes byte i from the low or the high result.
+__device__ __forceinline__ uint32_t mmq_lut16(uint32_t n, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
+    const uint32_t sel = n & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel), hi = __builtin_amdgcn_perm(t3, t2, sel);
+    return __builtin_amdgcn_perm(hi, lo, ((n >> 1) & 0x04040404u) | 0x03020100u);
+}
+
+// The 32 codes of one activation block into the staged image.  Int8 plane: as they are (32 B at 32 b).  FP8 image of
+// the native FP4 path (64 B at 64 b): [hi chunk 0][hi chunk 1][lo chunk 0][lo chunk 1], hi = q >> 4 and lo = q & 15 as
+// E4M3 bytes (0, 1, .. 15 -> 00 38 40 44 48 4A 4C 4E 50 .. 57; -8 .. -1 -> D0 CE CC CA C8 C4 C0 B8); chunk h holds, at
+// byte p, element ((16 h + p) >> 1) + 16 ((16 h + p) & 1), the order of the nibbles of an MXFP4 block (byte m = elements
+// m and m + 16).
+template <bool NATIVE>
+__device__ __forceinline__ void mmq_store_codes(uint8_t* row, uint32_t b, const uint4& q0, const uint4& q1) {
+    if constexpr (!NATIVE) {
+        uint4* dst = reinterpret_cast<uint4*>(row + 32u * b);
+        dst[0] = q0;
+        dst[1] = q1;
+    } else {
+        const uint32_t w[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        uint32_t hi[8], lo[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            lo[j] = mmq_lut16(w[j] & 0x0F0F0F0Fu, 0x44403800u, 0x4E4C4A48u, 0x53525150u, 0x57565554u);
+            hi[j] = mmq_lut16((w[j] >> 4) & 0x0F0F0F0Fu, 0x44403800u, 0x4E4C4A48u, 0xCACCCED0u, 0xB8C0C4C8u);
+        }
+        // dwords j and j + 4 hold elements 4j.. and 16 + 4j..: interleave them byte by byte
+        auto il0 = [](uint32_t a, uint32_t c) { return __builtin_amdgcn_perm(c, a, 0x05010400u); };
+        auto il1 = [](uint32_t a, uint32_t c) { return __builtin_amdgcn_perm(c, a, 0x07030602u); };
+        uint4* dst = reinterpret_cast<uint4*>(row + 64u * b);
+        dst[0] = make_uint4(il0(hi[0], hi[4]), il1(hi[0], hi[4]), il0(hi[1], hi[5]), il1(hi[1], hi[5]));
+        dst[1] = make_uint4(il0(hi[2], hi[6]), il1(hi[2], hi[6]), il0(hi[3], hi[7]), il1(hi[3], hi[7]));
+        dst[2] = make_uint4(il0(lo[0], lo[4]), il1(lo[0], lo[4]), il0(lo[1], lo[5]), il1(lo[1], lo[5]));
+        dst[3] = make_uint4(il0(lo[2], lo[6]), il1(lo[2], lo[6]), il0(lo[3], lo[7]), il1(lo[3], lo[7]));
+    }
+}
+
+template <int TV, bool HAS_MIN, bool NATIVE, class RowFn>
 __device__ __forceinline__ MmqAct mmq_stage(uint8_t* lds, RowFn xrow, uint32_t T, uint32_t k0, uint32_t kr, uint32_t K, bool split) {
     constexpr uint32_t TP = 2 * TV;
-    const uint32_t stride = kr + 32u, nblk = kr / 32u;
+    const uint32_t stride = mmq_row_pitch(kr, NATIVE), nblk = kr / 32u;
     float* dx = reinterpret_cast<float*>(lds + (size_t)T * stride);
     float* sx = dx + (size_t)nblk * TP;
     const uint32_t bsz = split ? kQ81sBytes : kQ81xBytes, hsz = split ? 16u : 8u;
@@ -407,9 +510,7 @@ __device__ __forceinline__ MmqAct mmq_stage(uint8_t* lds, RowFn xrow, uint32_t T
             const uint32_t i = base + (uint32_t)u * blockDim.x;
             if (i < total) {
                 const uint32_t t = i / nblk, b = i - t * nblk;
-                uint4* dst = reinterpret_cast<uint4*>(lds + (size_t)t * stride + 32u * b);
-                dst[0] = q0[u];
-                dst[1] = q1[u];
+                mmq_store_codes<NATIVE>(lds + (size_t)t * stride, b, q0[u], q1[u]);
                 dx[(size_t)b * TP + t] = d[u];
                 if (HAS_MIN) sx[(size_t)b * TP + t] = sm[u];
             }
@@ -421,10 +522,10 @@ __device__ __forceinline__ MmqAct mmq_stage(uint8_t* lds, RowFn xrow, uint32_t T
 // The same image from fp16 rows, quantized on the way in: d = amax / 127, q = round-half-away(v * 127 / amax),
 // s = d * float(sum q) per 32-element block, exactly quantize_q8_1 (src/ops/gemv_q8dot.cpp:94-124), so the staged
 // image is bit-identical to staging the quantizer's output.  One thread per (token, block).  `hrow(t)` -> row t.
-template <int TV, bool HAS_MIN, class RowFn>
+template <int TV, bool HAS_MIN, bool NATIVE, class RowFn>
 __device__ __forceinline__ MmqAct mmq_stage_f16(uint8_t* lds, RowFn hrow, uint32_t T, uint32_t k0, uint32_t kr, uint32_t K) {
     constexpr uint32_t TP = 2 * TV;
-    const uint32_t stride = kr + 32u, nblk = kr / 32u;
+    const uint32_t stride = mmq_row_pitch(kr, NATIVE), nblk = kr / 32u;
     float* dx = reinterpret_cast<float*>(lds + (size_t)T * stride);
     float* sx = dx + (size_t)nblk * TP;
     const uint32_t total = T * nblk;
@@ -461,9 +562,7 @@ __device__ __forceinline__ MmqAct mmq_stage_f16(uint8_t* lds, RowFn hrow, uint32
             }
             sm = d * (float)sum;
         }
-        uint4* dst = reinterpret_cast<uint4*>(lds + (size_t)t * stride + 32u * b);
-        dst[0] = make_uint4(q[0], q[1], q[2], q[3]);
-        dst[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        mmq_store_codes<NATIVE>(lds + (size_t)t * stride, b, make_uint4(q[0], q[1], q[2], q[3]), make_uint4(q[4], q[5], q[6], q[7]));
         dx[(size_t)b * TP + t] = d;
         if (HAS_MIN) sx[(size_t)b * TP + t] = sm;
     }
@@ -553,7 +652,7 @@ template <class P, int TV>
 struct MmqWalk {
     typename P::Raw raw[2];
     // the first group, requested by the caller before it stages the activations (it does not depend on them)
-    __device__ __forceinline__ void prefetch(const typename P::W& w, uint32_t n, uint32_t g_lo, uint32_t h, uint32_t nb) { raw[0] = P::load(w, n, g_lo, h, nb); }
+    __device__ __forceinline__ void prefetch(const typename P::W& w, uint32_t n, uint32_t g_lo, uint32_t, uint32_t h, uint32_t nb) { raw[0] = P::load(w, n, g_lo, h, nb); }
     // the partial last group of a row (block count not a multiple of 8), outside the pipeline
     __device__ __forceinline__ void tail(const typename P::W& w, uint32_t n, uint32_t g, uint32_t g_base, uint32_t h, uint32_t nb, const MmqAct& act,
                                          uint32_t a_off, float (&acc)[TV]) {
@@ -585,6 +684,101 @@ struct MmqWalk {
     }
 };
 
+// ---------------------------------------------------------------- native FP4: one group = four block pairs
+// `a_off` = row_a * pitch + 64 * (j / 16) + 16 h for token row_a = min(j % 16, live rows - 1): the lane's hi chunk of block
+// 2 s + j / 16 of the pair; the lo chunk lies 32 bytes on.  keep_lo / keep_hi: all ones in the lanes whose data belongs in
+// bytes 0..15 / 16..31 of the operand (j < 16 / j >= 16).
+template <class P, int TV, int S>
+__device__ __forceinline__ void mmq_pair_issue(const typename P::Raw& raw, const MmqAct& act, uint32_t a_off, uint32_t gl, uint32_t g, uint32_t nb,
+                                               uint32_t keep_lo, uint32_t keep_hi, v16f_t& C) {
+    const uint8_t* ap = act.plane + a_off + (8u * gl + 2u * S) * 64u;
+    const uint4 xh = *reinterpret_cast<const uint4*>(ap), xl = *reinterpret_cast<const uint4*>(ap + 32);
+    const v8i_t ah = {(int)(xh.x & keep_lo), (int)(xh.y & keep_lo), (int)(xh.z & keep_lo), (int)(xh.w & keep_lo),
+                      (int)(xh.x & keep_hi), (int)(xh.y & keep_hi), (int)(xh.z & keep_hi), (int)(xh.w & keep_hi)};
+    const v8i_t al = {(int)(xl.x & keep_lo), (int)(xl.y & keep_lo), (int)(xl.z & keep_lo), (int)(xl.w & keep_lo),
+                      (int)(xl.x & keep_hi), (int)(xl.y & keep_hi), (int)(xl.z & keep_hi), (int)(xl.w & keep_hi)};
+    const v8i_t b = {(int)raw.q[S].x, (int)raw.q[S].y, (int)raw.q[S].z, (int)raw.q[S].w, 0, 0, 0, 0};
+    const v16f_t z = {};
+    constexpr int sa = 0x7F83;              // byte 0: 2^4 for the hi operand, byte 1: 2^0 for the lo operand
+    const int sb = P::template scale_word<S>(raw, g, (threadIdx.x >> 5) & 1u, nb);   // the block exponent of this lane half in byte 0
+    C = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, b, z, 0, 4, 0, sa, 0, sb);
+    C = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(al, b, C, 0, 4, 1, sa, 0, sb);
+}
+
+template <class P, int TV, int S>
+__device__ __forceinline__ void mmq_pair(const typename P::Raw& raw, const MmqAct& act, uint32_t a_off, uint32_t gl, uint32_t g, uint32_t nb, uint32_t h,
+                                         uint32_t keep_lo, uint32_t keep_hi, float (&acc)[TV], v16f_t (&C)[2]) {
+    constexpr uint32_t TP = 2 * TV;
+    if constexpr (S < 4) {
+        constexpr int cur = S & 1, nxt = cur ^ 1;
+        if constexpr (S + 1 < 4) mmq_pair_issue<P, TV, S + 1>(raw, act, a_off, gl, g, nb, keep_lo, keep_hi, C[nxt]);
+        float dx0[TV], dx1[TV];
+        mmq_read4<TV>(act.dx + (size_t)(8u * gl + 2u * S) * TP, h, dx0);
+        mmq_read4<TV>(act.dx + (size_t)(8u * gl + 2u * S + 1u) * TP, h, dx1);
+        {
+            // each product is rounded on its own before it is added (the fold of the other kernels: acc += c * (d_x * idot))
+#pragma clang fp contract(off)
+#pragma unroll
+            for (int v = 0; v < TV; ++v) {
+                const float p0 = dx0[v] * C[cur][v];
+                acc[v] += p0;
+            }
+#pragma unroll
+            for (int v = 0; v < TV; ++v) {
+                const float p1 = dx1[v] * C[cur][8 + v];
+                acc[v] += p1;
+            }
+        }
+        mmq_pair<P, TV, S + 1>(raw, act, a_off, gl, g, nb, h, keep_lo, keep_hi, acc, C);
+    }
+}
+
+template <class P, int TV>
+__device__ __forceinline__ void mmq_group_native(const typename P::Raw& raw, const MmqAct& act, uint32_t a_off, uint32_t g, uint32_t g_base, uint32_t nb,
+                                                 uint32_t h, float (&acc)[TV]) {
+    static_assert(TV <= 8, "a pass of the native FP4 path holds at most 16 tokens");
+    const uint32_t keep_lo = (threadIdx.x & 16u) ? 0u : 0xFFFFFFFFu, keep_hi = ~keep_lo;
+    v16f_t C[2];
+    mmq_pair_issue<P, TV, 0>(raw, act, a_off, g - g_base, g, nb, keep_lo, keep_hi, C[0]);
+    mmq_pair<P, TV, 0>(raw, act, a_off, g - g_base, g, nb, h, keep_lo, keep_hi, acc, C);
+}
+
+// The walk of the native path: a group is 18 registers, so three groups are in flight behind the one being multiplied.
+// Slots past the end of the walk load one broadcast address (no load sits under a branch).
+template <class P, int TV>
+struct MmqWalkNative {
+    typename P::Raw raw[4];
+    __device__ __forceinline__ void prefetch(const typename P::W& w, uint32_t n, uint32_t g_lo, uint32_t g_hi, uint32_t h, uint32_t nb) {
+#pragma unroll
+        for (int u = 0; u < 3; ++u) raw[u] = P::load(w, n, g_lo + u, h, nb, g_lo + u < g_hi);
+    }
+    // partial groups run through the pipeline like whole ones
+    __device__ __forceinline__ void tail(const typename P::W&, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, const MmqAct&, uint32_t, float (&)[TV]) {}
+    __device__ __forceinline__ void run(const typename P::W& w, uint32_t n, uint32_t g_lo, uint32_t g_hi, uint32_t g_base, uint32_t h, uint32_t nb,
+                                        const MmqAct& act, uint32_t a_off, float (&acc)[TV]) {
+        for (uint32_t g = g_lo; g < g_hi; g += 4) {
+            raw[3] = P::load(w, n, g + 3, h, nb, g + 3 < g_hi);
+            __builtin_amdgcn_sched_barrier(0);
+            mmq_group_native<P, TV>(raw[0], act, a_off, g, g_base, nb, h, acc);
+            raw[0] = P::load(w, n, g + 4, h, nb, g + 4 < g_hi);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 1 < g_hi) mmq_group_native<P, TV>(raw[1], act, a_off, g + 1, g_base, nb, h, acc);
+            raw[1] = P::load(w, n, g + 5, h, nb, g + 5 < g_hi);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 2 < g_hi) mmq_group_native<P, TV>(raw[2], act, a_off, g + 2, g_base, nb, h, acc);
+            raw[2] = P::load(w, n, g + 6, h, nb, g + 6 < g_hi);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 3 < g_hi) mmq_group_native<P, TV>(raw[3], act, a_off, g + 3, g_base, nb, h, acc);
+        }
+    }
+};
+
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global load of the
+// wave (its fence covers global memory), which would drain the weight words requested ahead of the barrier; here only the
+// LDS counter is waited for, so those loads stay in flight across the barrier.
+__device__ __forceinline__ void mmq_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---------------------------------------------------------------- kernel
 enum { MMQ_STORE = 0, MMQ_SILU = 1, MMQ_OAI = 2, MMQ_DOWN_WEIGHTED = 3, MMQ_DOWN_BIAS = 4 };
 
@@ -603,6 +797,7 @@ struct MmqArgs {
     uint32_t M, K, N, E;
     uint32_t q8_split;
     uint32_t kr;                      // staged k range per pass (multiple of 256 WK)
+    uint32_t red_off;                 // byte offset of the partial-sum exchange area in LDS (behind the staged image)
 };
 
 __device__ __forceinline__ float mmq_silu_mul(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
@@ -611,14 +806,18 @@ __device__ __forceinline__ float mmq_swiglu_oai(float g, float u, float alpha, f
     return (x / (1.f + __expf(alpha * -x))) * (z + 1.f);
 }
 
-// Grid: x = blocks of 32 WR weight rows, y = expert (grouped) or 1, z = K range (dense, with `part`) or 1.
-// Workgroup = NW x WR x WK waves.  A pass covers up to 8 TV / 4 token rows... i.e. 2 TV tokens: T <= 8 (TV = 4),
-// 16 (TV = 8), 32 (TV = 16); an expert with more rows runs several passes over its weights (served from L2: a
-// workgroup's slice of an expert is 32 WR rows).
+// Grid: x = workgroups per expert (each takes the blocks of 32 WR weight rows x, x + gridDim.x, ...), y = expert (grouped)
+// or 1, z = K range (dense, with `part`) or token tile dealing (grouped).  Workgroup = NW x WR x WK waves.  A pass covers
+// up to 2 TV token rows: T <= 8 (TV = 4), 16 (TV = 8), 32 (TV = 16); an expert with more rows runs several passes over
+// its weights.  When one staged image covers the whole K range (the usual case) it is built once per token tile and every
+// row block of the workgroup runs against it; the first weight words of the next row block are requested before the
+// partial sums of the current one meet, so a workgroup with several row blocks streams without gaps.
+// LDS: the staged image, then `red` [waves][TV][64] floats where the partial sums of the WK waves (and the NW matrices) meet.
 template <class P, int TV, int NW, int WR, int WK, int EPI>
 __global__ __launch_bounds__(64 * NW * WR * WK, 2) void mmq_kernel(MmqArgs<P> a) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr uint32_t TT = 2 * TV;   // token rows per pass
+    constexpr bool NATIVE = mmq_native<P>::value;
     const uint32_t lane = threadIdx.x & 63u, j = lane & 31u, h = lane >> 5;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t wk = wave % WK, wr = (wave / WK) % WR, wm = wave / (WK * WR);
@@ -631,8 +830,7 @@ __global__ __launch_bounds__(64 * NW * WR * WK, 2) void mmq_kernel(MmqArgs<P> a)
     }
     const typename P::W w = P::expert((NW == 2 && wm) ? a.bank1 : a.bank0, e);
     const uint32_t nb = a.K / 32u, n_groups = (nb + 7u) / 8u;
-    const uint32_t n0 = (blockIdx.x * WR + wr) * 32u;
-    const uint32_t n = n0 + j < a.N ? n0 + j : a.N - 1u;
+    const uint32_t n_rb = (a.N + 32u * WR - 1u) / (32u * WR);
     // gridDim.z: dense launches split K into ranges (partial sums to `part`); grouped launches deal the token tiles of an
     // expert round-robin, so that an expert with many rows is spread over many workgroups
     const bool grouped = a.expert_offsets != nullptr;
@@ -641,70 +839,112 @@ __global__ __launch_bounds__(64 * NW * WR * WK, 2) void mmq_kernel(MmqArgs<P> a)
     const uint32_t G0 = kzi * gz, G1 = G0 + gz < n_groups ? G0 + gz : n_groups;
     const uint32_t t_step = grouped ? gridDim.z * 2u * TV : 2u * TV, t_first = grouped ? blockIdx.z * 2u * TV : 0u;
     const uint32_t gp = a.kr / 256u;                     // groups per pass (multiple of WK)
+    const bool single = G1 - G0 <= gp;                   // one image covers the K range
     const size_t q8_row_bytes = (size_t)nb * (a.q8_split ? kQ81sBytes : kQ81xBytes);
-    float* red = reinterpret_cast<float*>(lds);          // [NWAVES][TV][64] partial sums, after the last pass (reuses the plane)
+    float* red = reinterpret_cast<float*>(lds + a.red_off);
 
     for (uint32_t t0 = r_begin + t_first; t0 < r_end; t0 += t_step) {
         const uint32_t nt = r_end - t0 < TT ? r_end - t0 : TT;
         auto xrow = [&](uint32_t t) { return a.xq8 + (size_t)(t0 + t) * q8_row_bytes; };
-        float acc[TV];
+        auto hrow = [&](uint32_t t) { return a.act_f16 + (size_t)(t0 + t) * a.K; };
+        // token rows past the tile re-read its last row (their results are dropped)
+        const uint32_t jt = NATIVE ? (j & 15u) : j, row_a = jt < nt ? jt : nt - 1u;
+        typename std::conditional<NATIVE, MmqWalkNative<P, TV>, MmqWalk<P, TV>>::type walk;
+        MmqAct act{};
+        bool staged = false, requested = false;
+        // what the epilogue reads from global memory is requested ahead of the weight walk: a load issued in the epilogue
+        // would have to wait for the whole queue of weight words requested for the next row block before it
+        float rw[TV];
 #pragma unroll
-        for (int v = 0; v < TV; ++v) acc[v] = 0.f;
-        for (uint32_t gb = G0; gb < G1; gb += gp) {
-            const uint32_t ge = gb + gp < G1 ? gb + gp : G1;          // groups [gb, ge) of this pass
-            const uint32_t per = (ge - gb + WK - 1u) / WK;
-            const uint32_t g_lo = gb + wk * per < ge ? gb + wk * per : ge, g_hi = g_lo + per < ge ? g_lo + per : ge;
-            const uint32_t g_full = g_hi < nb / 8u ? g_hi : nb / 8u;   // the pipeline takes whole groups; a partial last group follows it
-            MmqWalk<P, TV> walk;
-            if (g_lo < g_full) walk.prefetch(w, n, g_lo, h, nb);
-            __syncthreads();                                            // the plane of the previous pass is no longer read
-            auto hrow = [&](uint32_t t) { return a.act_f16 + (size_t)(t0 + t) * a.K; };
-            const MmqAct act = a.act_f16 ? mmq_stage_f16<TV, P::HAS_MIN>(lds, hrow, nt, gb * 256u, (ge - gb) * 256u, a.K)
-                                         : mmq_stage<TV, P::HAS_MIN>(lds, xrow, nt, gb * 256u, (ge - gb) * 256u, a.K, a.q8_split != 0);
-            __syncthreads();
-            const uint32_t row_a = j < nt ? j : nt - 1u;                // token rows past the tile re-read its last row (their results are dropped)
-            const uint32_t a_off = row_a * act.stride + 16u * h;
-            if (g_lo < g_full) walk.run(w, n, g_lo, g_full, gb, h, nb, act, a_off, acc);
-            if (g_hi > g_full && g_lo <= g_full) walk.tail(w, n, g_full, gb, h, nb, act, a_off, acc);
+        for (int v = 0; v < TV; ++v) {
+            const uint32_t t = 8u * (v / 4) + 4u * h + (v % 4);
+            rw[v] = (EPI == MMQ_DOWN_WEIGHTED) ? (float)a.route_w[t0 + (t < nt ? t : nt - 1u)] : 0.f;
         }
-        // ---- partial sums of the WK waves (and the NW matrices) meet in LDS
-        __syncthreads();
+        for (uint32_t rb = blockIdx.x; rb < n_rb; rb += gridDim.x) {
+            const uint32_t n0 = (rb * WR + wr) * 32u;
+            const uint32_t n = n0 + j < a.N ? n0 + j : a.N - 1u;
+            // MMQ_OAI: the bias of this wave's matrix joins its partial sum before the exchange (wave wk = 0 of each matrix);
+            // MMQ_DOWN_BIAS: added after the fp16 rounding of the sum, in the epilogue
+            float bias_a = 0.f;
+            if (EPI == MMQ_OAI || EPI == MMQ_DOWN_BIAS) {
+                const float* bp = (NW == 2 && wm) ? a.bias1 : a.bias0;
+                if (bp) bias_a = bp[(size_t)e * a.N + n];
+            }
+            float acc[TV];
 #pragma unroll
-        for (int v = 0; v < TV; ++v) red[((size_t)wave * TV + v) * 64u + lane] = acc[v];
-        __syncthreads();
-        if (wk == 0 && wm == 0) {
+            for (int v = 0; v < TV; ++v) acc[v] = 0.f;
+            for (uint32_t gb = G0; gb < G1; gb += gp) {
+                const uint32_t ge = gb + gp < G1 ? gb + gp : G1;          // groups [gb, ge) of this pass
+                const uint32_t per = (ge - gb + WK - 1u) / WK;
+                const uint32_t g_lo = gb + wk * per < ge ? gb + wk * per : ge, g_hi = g_lo + per < ge ? g_lo + per : ge;
+                // the pipeline takes whole groups and a partial last group follows it, except where the producer loads both alike
+                const uint32_t g_full = (NATIVE || g_hi < nb / 8u) ? g_hi : nb / 8u;
+                if (!requested && g_lo < g_full) walk.prefetch(w, n, g_lo, g_full, h, nb);
+                requested = false;
+                if (!staged) {
+                    mmq_lds_barrier();                                        // the image of the previous pass is no longer read
+                    act = a.act_f16 ? mmq_stage_f16<TV, P::HAS_MIN, NATIVE>(lds, hrow, nt, gb * 256u, (ge - gb) * 256u, a.K)
+                                    : mmq_stage<TV, P::HAS_MIN, NATIVE>(lds, xrow, nt, gb * 256u, (ge - gb) * 256u, a.K, a.q8_split != 0);
+                    mmq_lds_barrier();
+                    staged = single;
+                }
+                const uint32_t a_off = row_a * act.stride + 16u * h + (NATIVE ? 64u * (j >> 4) : 0u);
+                if (g_lo < g_full) walk.run(w, n, g_lo, g_full, gb, h, nb, act, a_off, acc);
+                if (g_hi > g_full && g_lo <= g_full) walk.tail(w, n, g_full, gb, h, nb, act, a_off, acc);
+                // the epilogue's operands are made to arrive here, while nothing else is outstanding: otherwise the wait for
+                // them would sit in the epilogue, behind the weight words requested just below
+                asm volatile("" : "+v"(bias_a));
 #pragma unroll
-            for (int v = 0; v < TV; ++v) {
-                const uint32_t t = 8u * (v / 4) + 4u * h + (v % 4);
-                float s0 = 0.f, s1 = 0.f;
+                for (int v = 0; v < TV; ++v) asm volatile("" : "+v"(rw[v]));
+                if (EPI == MMQ_OAI && ge == G1 && wk == 0) {
 #pragma unroll
-                for (int k = 0; k < WK; ++k) {
-                    s0 += red[((size_t)((0 * WR + wr) * WK + k) * TV + v) * 64u + lane];
-                    if (NW == 2) s1 += red[((size_t)((1 * WR + wr) * WK + k) * TV + v) * 64u + lane];
+                    for (int v = 0; v < TV; ++v) acc[v] += bias_a;
                 }
-                if (t >= nt || n0 + j >= a.N) continue;
-                const uint32_t row = t0 + t, col = n0 + j;
-                if (a.part) {
-                    a.part[((size_t)kzi * a.M + row) * a.N + col] = s0;
-                    continue;
+                if (single && rb + gridDim.x < n_rb && g_lo < g_full) {
+                    // the next row block's first weight words, requested before the partial sums of this one meet
+                    const uint32_t nn0 = ((rb + gridDim.x) * WR + wr) * 32u;
+                    walk.prefetch(w, nn0 + j < a.N ? nn0 + j : a.N - 1u, g_lo, g_full, h, nb);
+                    requested = true;
                 }
-                float o;
-                if (EPI == MMQ_SILU) {
-                    o = mmq_silu_mul(s0, s1);                                          // src/ops/moe_q8.cpp:94-97
-                } else if (EPI == MMQ_OAI) {
-                    // rounding points of the reference chain: half(acc + bias) per projection, then the fp16 activation
-                    const float g = (float)(half_t)(s0 + (a.bias0 ? a.bias0[(size_t)e * a.N + col] : 0.f));
-                    const float u = (float)(half_t)(s1 + (a.bias1 ? a.bias1[(size_t)e * a.N + col] : 0.f));
-                    o = mmq_swiglu_oai(g, u, a.alpha, a.limit);
-                } else if (EPI == MMQ_DOWN_WEIGHTED) {
-                    o = (float)a.route_w[row] * s0;                                   // src/ops/moe_q8.cpp:143-144
-                } else if (EPI == MMQ_DOWN_BIAS) {
-                    o = (float)(half_t)s0;                                            // gemv out, then add_bias (elementwise.cpp:782-793)
-                    if (a.bias0) o += a.bias0[(size_t)e * a.N + col];
-                } else {
-                    o = s0;
+            }
+            // ---- partial sums of the WK waves (and the NW matrices) meet in LDS
+            mmq_lds_barrier();
+#pragma unroll
+            for (int v = 0; v < TV; ++v) red[((size_t)wave * TV + v) * 64u + lane] = acc[v];
+            mmq_lds_barrier();
+            if (wk == 0 && wm == 0) {
+#pragma unroll
+                for (int v = 0; v < TV; ++v) {
+                    const uint32_t t = 8u * (v / 4) + 4u * h + (v % 4);
+                    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                    for (int k = 0; k < WK; ++k) {
+                        s0 += red[((size_t)((0 * WR + wr) * WK + k) * TV + v) * 64u + lane];
+                        if (NW == 2) s1 += red[((size_t)((1 * WR + wr) * WK + k) * TV + v) * 64u + lane];
+                    }
+                    if (t >= nt || n0 + j >= a.N) continue;
+                    const uint32_t row = t0 + t, col = n0 + j;
+                    if (a.part) {
+                        a.part[((size_t)kzi * a.M + row) * a.N + col] = s0;
+                        continue;
+                    }
+                    float o;
+                    if (EPI == MMQ_SILU) {
+                        o = mmq_silu_mul(s0, s1);                                          // src/ops/moe_q8.cpp:94-97
+                    } else if (EPI == MMQ_OAI) {
+                        // rounding points of the reference chain: half(acc + bias) per projection, then the fp16 activation
+                        const float g = (float)(half_t)s0, u = (float)(half_t)s1;   // sums with their biases
+                        o = mmq_swiglu_oai(g, u, a.alpha, a.limit);
+                    } else if (EPI == MMQ_DOWN_WEIGHTED) {
+                        o = rw[v] * s0;                                                   // src/ops/moe_q8.cpp:143-144
+                    } else if (EPI == MMQ_DOWN_BIAS) {
+                        o = (float)(half_t)s0;                                            // gemv out, then add_bias (elementwise.cpp:782-793)
+                        if (a.bias0) o += bias_a;
+                    } else {
+                        o = s0;
+                    }
+                    a.out[(size_t)row * a.N + col] = (half_t)o;
                 }
-                a.out[(size_t)row * a.N + col] = (half_t)o;
             }
         }
     }

@@ -42,14 +42,15 @@ def f16(a):
 
 
 def check_rows(a, b, what):
-    """Two fp16 results of the same arithmetic: equal up to a few fp16 ulps where fp32 noise crosses a
-    rounding boundary (and is then re-quantised downstream)."""
+    """Two fp16 results of the same arithmetic in different fp32 summation orders (vector-ALU decode kernels, matrix-core
+    grouped kernels): equal up to a few fp16 ulps where fp32 noise crosses a rounding boundary (and is then re-quantised
+    downstream: after gate/up, quantize, down and the weighted sum about 3 % of a layer's outputs move by one ulp)."""
     a32, b32 = a.astype(np.float32), b.astype(np.float32)
     rms = float(np.sqrt(np.mean(b32 * b32)))
     frac_equal = float(np.mean(a == b))
     err = float(np.abs(a32 - b32).max() / rms)
     print("%s: %.4f bit-equal, max_abs/rms=%.2e" % (what, frac_equal, err), flush=True)
-    assert frac_equal > 0.98 and err < 1e-2, what
+    assert frac_equal > 0.95 and err < 1e-2, what
 
 
 # Stages that mirror the reference's chain of fp16 roundings (half(acc + bias), then the fp16
@@ -58,18 +59,33 @@ def check_rows(a, b, what):
 CHAIN_GATE = 2e-3
 
 
-def ref_gate_up_oai(Wg, Wu, bg, bu, e, xq_row, K, N):
-    """-> (lo, hi, g16, u16): envelope of half(swiglu_oai(g16, u16)) over the admissible roundings of the two
-    intermediates: the fp32 device sums may sit on the other side of an fp16 rounding boundary than
-    the fp64 oracle sums, and swiglu_oai's (up + 1) factor can amplify that ulp without bound in
-    relative terms, so the stage is checked against the set of results the reference chain can
-    produce when g16 / u16 move by at most one fp16 ulp."""
-    g = f16(O.gemv_q8chain(O.MXFP4, Wg[e], xq_row, K, N)[0] + bg[e]).astype(np.float16)
-    u = f16(O.gemv_q8chain(O.MXFP4, Wu[e], xq_row, K, N)[0] + bu[e]).astype(np.float16)
+def sum_noise(acc, other=0.0):
+    """What the order of an fp32 accumulation can move a sum by: a few fp32 ulps of the partial sums, whose scale is
+    the row's rms and the two addends.  Implementations (the reference's sub-group reductions included) differ by
+    this much before the fp16 rounding, and for an element whose acc + bias nearly cancels that exceeds one fp16 ulp
+    of the small result."""
+    a = np.asarray(acc, np.float64)
+    return 2.0 ** -18 * (np.abs(a) + np.abs(other) + float(np.sqrt(np.mean(a * a))))
+
+
+def f16_candidates(s64, eta):
+    """fp16 values a chain may hold for the fp64 sum s64 known to +-eta: one ulp beyond the rounded ends."""
     inf = np.float16(np.inf)
-    outs = [f16(O.swiglu_oai_np(gg.astype(np.float32), uu.astype(np.float32)))
-            for gg in (np.nextafter(g, -inf), g, np.nextafter(g, inf)) for uu in (np.nextafter(u, -inf), u, np.nextafter(u, inf))]
-    return np.min(outs, axis=0), np.max(outs, axis=0), g.astype(np.float32), u.astype(np.float32)
+    return (np.nextafter(f16(s64 - eta).astype(np.float16), -inf), f16(s64).astype(np.float16), np.nextafter(f16(s64 + eta).astype(np.float16), inf))
+
+
+def ref_gate_up_oai(Wg, Wu, bg, bu, e, xq_row, K, N):
+    """-> (lo, hi, g16, u16, eta_g, eta_u): envelope of half(swiglu_oai(g16, u16)) over the admissible roundings of the
+    two intermediates: the fp32 device sums may sit on the other side of an fp16 rounding boundary than
+    the fp64 oracle sums (by the accumulation-order noise `sum_noise`, then one fp16 ulp), and swiglu_oai's (up + 1)
+    factor can amplify that ulp without bound in relative terms, so the stage is checked against the set of results the
+    reference chain can produce when g16 / u16 move that far."""
+    ag = O.gemv_q8chain(O.MXFP4, Wg[e], xq_row, K, N)[0].astype(np.float64)
+    au = O.gemv_q8chain(O.MXFP4, Wu[e], xq_row, K, N)[0].astype(np.float64)
+    eta_g, eta_u = sum_noise(ag, bg[e]), sum_noise(au, bu[e])
+    gc, uc = f16_candidates(ag + bg[e], eta_g), f16_candidates(au + bu[e], eta_u)
+    outs = [f16(O.swiglu_oai_np(gg.astype(np.float32), uu.astype(np.float32))) for gg in gc for uu in uc]
+    return np.min(outs, axis=0), np.max(outs, axis=0), gc[1].astype(np.float32), uc[1].astype(np.float32), eta_g, eta_u
 
 
 def ulp16(v):
@@ -130,7 +146,9 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     xg, z = np.minimum(g16, 7.0), np.clip(u16, -7.0, 7.0)
     sg = 1.0 / (1.0 + np.exp(-1.702 * xg))
     glu, dglu = xg * sg, np.where(g16 < 7.0, sg * (1.0 + 1.702 * xg * (1.0 - sg)), 0.0)
-    budget = ulp16(g16) * np.abs(dglu) * np.abs(z + 1.0) + np.where(np.abs(u16) < 7.0, ulp16(u16), 0.0) * np.abs(glu) + ulp16(centre)
+    eta_g, eta_u = np.stack([e[4] for e in env]), np.stack([e[5] for e in env])
+    budget = ((ulp16(g16) + eta_g) * np.abs(dglu) * np.abs(z + 1.0) + np.where(np.abs(u16) < 7.0, ulp16(u16) + eta_u, 0.0) * np.abs(glu)
+              + ulp16(centre))
     explained_outliers(h_h, centre, budget, "moe gate_up swiglu_oai (decode) T=%d" % T, 0.999)
     hq = ops.quantize_q8_1(h)
     hq_h = host(hq)
@@ -144,8 +162,10 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     inf = np.float16(np.inf)
     lo, hi, ctr, a16s = [], [], [], []
     for s_ in range(T * Kt):   # out = half(half(acc) + bias): envelope over half(acc) moving by one ulp (the sum can cancel)
-        a16 = f16(O.gemv_q8chain(O.MXFP4, Wd[ids.ravel()[s_]], hq_h[s_ * hrb:(s_ + 1) * hrb], EF, H)[0]).astype(np.float16)
-        c = [f16(v.astype(np.float32) + bd[ids.ravel()[s_]]) for v in (np.nextafter(a16, -inf), a16, np.nextafter(a16, inf))]
+        acc = O.gemv_q8chain(O.MXFP4, Wd[ids.ravel()[s_]], hq_h[s_ * hrb:(s_ + 1) * hrb], EF, H)[0].astype(np.float64)
+        cands = f16_candidates(acc, sum_noise(acc))
+        a16 = cands[1]
+        c = [f16(v.astype(np.float32) + bd[ids.ravel()[s_]]) for v in cands]
         lo.append(np.min(c, axis=0))
         hi.append(np.max(c, axis=0))
         ctr.append(c[1])
