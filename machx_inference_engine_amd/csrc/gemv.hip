@@ -22,7 +22,8 @@ struct GemvSeg {
 
 // Formats whose T = 1 kernels hold a second set of units in registers (requested ahead of the row group being
 // summed, or ahead of the activation staging): the ones where that was measured to pay and that stay within the
-// 128 VGPRs the four-workgroups-per-CU launch wants.  Q6_K loses on both counts (82 -> 129 VGPRs).
+// 128 VGPRs the four-workgroups-per-CU launch wants.  Q6_K does not gain from it (12.1 -> 12.2 us on 4096 -> 14336,
+// 95.8 -> 98.5 us on the 151936-row output projection with the two alternating sets).
 template <class F>
 constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value;
 
@@ -51,42 +52,29 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
         // Measured on 4096 -> 14336: Q8_0 planes 13.2 -> 12.4 us (T = 2: 14.2 -> 13.0), Q4_K 8.6 -> 8.4 us (T = 2:
         // 10.2 -> 9.2).  Batches of four and more lose (the second set of units costs occupancy next to R x T sums).
         // The first row group's weights are requested before the activation row is staged: they do not depend on it.
-        typename F::Cursor cn[R];
-        typename F::Raw nxt[R];
-        uint32_t rg = blockIdx.x;
-        if (rg < n_rg) {
-            const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
+        // Two register sets take turns (never copied: a copy would wait for the load), so the loads of one row group are
+        // in flight while the other one is summed; a slot past the last row group reads one broadcast line.  The first
+        // row group's weights are requested between the activation loads and their LDS writes.
+        typename F::Cursor ca[R], cb[R];
+        typename F::Raw ra[R], rb[R];
+        const uint32_t stride = gridDim.x;
+        auto request = [&](uint32_t rgq, typename F::Cursor (&c)[R], typename F::Raw (&w)[R]) {
+            const bool live = rgq < n_rg;
+            const uint32_t row0 = rgq * ROWS_PER_WG + (wave * GROUPS + grp) * R;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                cn[r] = F::cursor(seg.w, (row0 + r < N) ? row0 + r : N - 1, gl);
-                nxt[r] = load_unit<F, G>(cn[r], 0, false);
+                c[r] = F::cursor(seg.w, live ? ((row0 + r < N) ? row0 + r : N - 1) : 0u, live ? gl : 0u);
+                w[r] = load_unit<F, G>(c[r], 0, false);
             }
-        }
-        act = stage_act<F::SUM_GRAN, T>(lds, xrow, 0, K, KT, q8_split != 0);
-        __syncthreads();
-        for (; rg < n_rg; rg += gridDim.x) {
-            const uint32_t row0 = rg * ROWS_PER_WG + (wave * GROUPS + grp) * R;
-            typename F::Cursor cu[R];
-            typename F::Raw raw[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                cu[r] = cn[r];
-                raw[r] = nxt[r];
-            }
-            if (rg + gridDim.x < n_rg) {
-                const uint32_t rown = (rg + gridDim.x) * ROWS_PER_WG + (wave * GROUPS + grp) * R;
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    cn[r] = F::cursor(seg.w, (rown + r < N) ? rown + r : N - 1, gl);
-                    nxt[r] = load_unit<F, G>(cn[r], 0, false);
-                }
-            }
+        };
+        auto finish = [&](uint32_t rgq, const typename F::Cursor (&c)[R], const typename F::Raw (&w)[R]) {
+            const uint32_t row0 = rgq * ROWS_PER_WG + (wave * GROUPS + grp) * R;
             float acc[R][T];
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int t = 0; t < T; ++t) acc[r][t] = 0.f;
-            gemv_step<F, T, R>(raw, cu, gl, act, acc);
+            gemv_step<F, T, R>(w, c, gl, act, acc);
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -97,6 +85,17 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> 
                         store_out(seg.y + (size_t)t * N + row0 + r, v);
                     }
                 }
+        };
+        uint32_t rg = blockIdx.x;
+        act = stage_act<F::SUM_GRAN, T>(lds, xrow, 0, K, KT, q8_split != 0, [&]() { request(rg, ca, ra); });
+        __syncthreads();
+        for (; rg < n_rg; rg += 2 * stride) {
+            request(rg + stride, cb, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            finish(rg, ca, ra);
+            request(rg + 2 * stride, ca, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            if (rg + stride < n_rg) finish(rg + stride, cb, rb);
         }
         return;
     }

@@ -52,11 +52,19 @@ __device__ __forceinline__ uint32_t act_slot(uint32_t q) { return q ^ (((q >> 4)
 // include/ie/quant_blocks.hpp:174-181); the stored half sums are used as they are
 // (src/ops/gemv_q8dot.cpp:483-597): per 16 they are the same numbers (s0 = d * float(sum of the
 // half)); per 32 the sum s0 + s1 carries one more fp32 rounding than d * float(sum32).
-template <int SUM_GRAN, int T, class RowFn>
-__device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc, bool split = false) {
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+// `between`: called once by every thread after its first round of activation loads has been requested and before they
+// are written to LDS.  Loads return in order, so weight words requested there stay in flight while the tile is built
+// (requested before the activation loads, the tile would wait for them too).
+template <int SUM_GRAN, int T, class RowFn, class Hook = NoHook>
+__device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc, bool split = false,
+                                             Hook between = Hook()) {
     uint4* qs = reinterpret_cast<uint4*>(lds);
     uint8_t* hdr = lds + (size_t)T * KT_alloc;
     const uint32_t halves = (kt + 63) / 64 * 4;   // padded to whole 64-element units with zeros
+    bool hooked = false;
     for (uint32_t i = threadIdx.x; i < (uint32_t)T * halves; i += blockDim.x) {
         const uint32_t t = i / halves, hb = i - t * halves;
         uint2 q0 = make_uint2(0, 0), q1 = q0;
@@ -74,6 +82,11 @@ __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t 
             } else {
                 ds = *reinterpret_cast<const float2*>(blk);
             }
+        }
+        if (!hooked) {
+            between();
+            __builtin_amdgcn_sched_barrier(0);
+            hooked = true;
         }
         qs[(size_t)t * (KT_alloc / 16) + act_slot<SUM_GRAN>(hb)] = make_uint4(q0.x, q0.y, q1.x, q1.y);
         if (SUM_GRAN == 16) {
@@ -93,6 +106,7 @@ __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t 
                 reinterpret_cast<float*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = ds.x;
         }
     }
+    if (!hooked) between();
     return ActTile{qs, hdr, KT_alloc};
 }
 
