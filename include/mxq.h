@@ -336,9 +336,10 @@ int mx_gemm_q4_0(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, u
  *   gemm_fp16          include/ie/ops.hpp:275-286, src/ops/gemm_fp16.cpp:46-178    C fp32 [M,N]
  *   gemm_fp16_onednn   include/ie/ops.hpp:460-465, src/ops/gemm_onednn.cpp:75-111  y fp16 [M,N]
  * A fp16 [M,K] row-major, B fp16 [K,N] row-major (the Bt the mx_dequant_*_to_Bt functions write),
- * fp32 accumulation.  Argument order (M, N, K) as in the reference.  Both run rocBLAS' gemm_ex (the
- * reference's second one is a library matmul too); the library is loaded on first use and
- * MX_ERR_UNSUPPORTED is returned where it is not installed.  */
+ * fp32 accumulation.  Argument order (M, N, K) as in the reference.  mx_gemm_fp16 is a hand-tiled matrix-core kernel
+ * (both tiles through LDS, B transposed on the way; ragged M, N, K into an exactly sized C); mx_gemm_fp16_onednn runs the
+ * vendor library (rocBLAS' gemm_ex, as the reference runs oneDNN), loaded on first use: MX_ERR_UNSUPPORTED where it is
+ * not installed.  */
 int mx_gemm_fp16(mx_stream_t s, const uint16_t* A, const uint16_t* B, float* C, uint32_t M, uint32_t N, uint32_t K);
 int mx_gemm_fp16_onednn(mx_stream_t s, const uint16_t* A, const uint16_t* B, uint16_t* y, uint32_t M, uint32_t N, uint32_t K);
 /* Expert-grouped GEMM over expert-sorted fp16 rows (Q8_0 SoA expert banks): the matrix-core
@@ -361,17 +362,37 @@ int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d
  *   moe_prefill_down_packed_q4k / _q6k (and _v2)              include/ie/ops.hpp:968-983, src/ops/moe_fused.cpp:1090-1572
  * sorted_w may be NULL: the rows are then written unweighted, as the reference's packed down
  * kernels do (the weights are applied by moe_prefill_reduce); with sorted_w the product
- * half(sorted_w[row] * acc) is folded into the store.  H % 256 == 0 and E_ffn % 256 == 0;
- * the reference's `soa` flag (per-expert SoA views) is not taken: AoS banks only.  */
+ * half(sorted_w[row] * acc) is folded into the store.  H % 256 == 0 and E_ffn % 256 == 0.
+ * soa != 0 as in the reference (include/ie/ops.hpp:918,927,997,1005): every expert region holds its blocks as
+ * per-field streams (mx_repack_moe_q4k_soa / _q6k_soa, include/ie/quant_soa.hpp:33-51); total_rows follows it.  */
 int mx_moe_gemm_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x_packed, const void* gate_W, const void* up_W,
                                  const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
-                                 uint64_t expert_stride_bytes, uint32_t total_rows);
+                                 uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
                          const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
-                         uint64_t expert_stride_bytes, uint32_t total_rows);
+                         uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
 int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets,
                          const uint16_t* sorted_w, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
-                         uint64_t expert_stride_bytes, uint32_t total_rows);
+                         uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
+/* MXFP4 planes and Q5_K blocks through the fused matrix-core kernel.  The reference has no fused form for them: it
+ * dequantizes to a [K, N] fp16 matrix and runs a plain GEMM (dequant_mxfp4_soa_to_Bt + gemm_fp16, src/ops/gemv_mxfp4.cpp:
+ * 316-341, src/model/gptoss.cpp:389-392; dequant_q5_K_to_Bt, include/ie/dequant.hpp:81-86); these compute the same
+ * y = A . half(deq(W))^T without writing that matrix.  mx_gemm_mxfp4_soa takes the planes of gemv_mxfp4_soa_q8
+ * (include/ie/ops.hpp, gemv_mxfp4.cpp:120-141), K % 64 == 0 (gpt-oss: K = 2880); mx_gemm_q5_K the GGUF block stream
+ * (176-byte blocks, 16-byte aligned), K % 256 == 0.  The grouped forms are the fp16-row counterparts of
+ * mx_moe_grouped_gate_up_oai_mxfp4 / mx_moe_grouped_down_mxfp4 (same arithmetic after the matrix product:
+ * half(swiglu_oai(half(g + bias), half(u + bias))) and half(half(acc) + bias); biases may be NULL).  */
+int mx_gemm_q5_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+int mx_gemm_mxfp4_soa(mx_stream_t s, const uint16_t* A, const uint8_t* qs_W, const uint8_t* e_W, uint16_t* y, uint32_t M,
+                      uint32_t K, uint32_t N);
+int mx_moe_gemm_gate_up_oai_mxfp4(mx_stream_t s, const uint16_t* x_packed, const uint8_t* g_qs, const uint8_t* g_e,
+                                  const uint8_t* u_qs, const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride,
+                                  const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets,
+                                  uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha,
+                                  float limit);
+int mx_moe_gemm_down_mxfp4(mx_stream_t s, const uint16_t* h_packed, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride,
+                           uint64_t e_stride, const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed,
+                           uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
 /* Q4_0 expert banks (Gemma-4 MoE) and the dense W4A8 GEMM; plain projections, no epilogue:
  *   moe_prefill_proj_q4_0_q8      include/ie/ops.hpp:166-177   block_q8_1s rows, GGUF blocks, expert e at W + e*expert_stride_bytes
  *   moe_prefill_proj_q4_0_soa_q8  include/ie/ops.hpp:179-190   block_q8_1s rows, planes: qs_bank + e*qs_stride bytes, d_bank + e*d_stride entries

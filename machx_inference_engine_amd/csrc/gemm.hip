@@ -11,9 +11,9 @@
 // Tiling (wave64, v_mfma_f32_32x32x16_f16):
 //   workgroup = 4 waves, 128 tokens x (4 x 64) weight rows, K walked in chunks of 128;
 //   wave      = 128 tokens x 64 rows = 4 x 2 MFMA tiles (128 accumulator VGPRs);
-//   tokens    : the fp16 A chunk [128 x 128] is staged in LDS (double buffered, row
-//               pitch padded to 272 B so a fragment read is bank-conflict free) and
-//               shared by the four waves;
+//   tokens    : the fp16 A chunk [128 x 128] is staged in LDS (double buffered, unpadded
+//               256-byte rows whose 16-byte columns are XOR-swizzled by the row number, so a
+//               fragment read is bank-conflict free) and shared by the four waves;
 //   weights   : lane (r = lane%32, h = lane/32) of a wave owns weight row r of a tile
 //               and the 64 consecutive elements [64h, 64h+64) of the chunk: it loads
 //               them from global as 128-bit words (32 B of Q4_K nibbles or 64 B of
@@ -23,6 +23,8 @@
 //               trip and no redundant dequantisation inside a workgroup.
 // The k order inside a chunk is (lanes 0-31: 8s.., lanes 32-63: 64+8s..); the
 // A fragments are read from LDS with the same order, so the products pair up.
+#include <type_traits>
+
 #include "mxq_formats.h"
 #include "mxq_host.h"
 
@@ -402,8 +404,210 @@ struct GemmQ6K {
     }
 };
 
+// Q5_K (176-byte blocks: d, dmin, scales[12], qh[32], qs[128]; include/ie/quant_blocks.hpp): Q4_K's nibbles plus one
+// high bit per element, bit j of qh[l] for sub-block j and position l.  Same chunk / lane-half split as Q4_K (lane half h
+// owns qs[32 g, 32 g + 32), g = 2 (kc % 2) + h: sub-blocks 2 g in the low and 2 g + 1 in the high nibbles); the lane also
+// keeps all 32 bytes of qh.  value = half(fma(d*sc, q, -(dmin*m))), q the 5-bit code held as an fp16 subnormal.
+struct GemmQ5K {
+    struct W {
+        const uint8_t* base;
+        uint32_t row_bytes;
+    };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint32_t row_bytes;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.base + (size_t)e * b.expert_stride_bytes, b.row_bytes}; }
+    struct Raw {
+        uint4 hdr, h0, h1, q0, q1;
+    };
+    struct Dec {
+        float d1[2], c1[2];
+        uint32_t bit;   // sub-block number of the low nibbles = bit of qh
+    };
+    static constexpr uint32_t K_ALIGN = 256;
+    static constexpr uint32_t H_COL = 8;
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)S; }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
+        const uint8_t* blk = w.base + (size_t)n * w.row_bytes + (size_t)(kc >> 1) * 176u;
+        const uint4* q = reinterpret_cast<const uint4*>(blk + 48 + (2u * (kc & 1u) + h) * 32u);
+        Raw r;
+        r.hdr = *reinterpret_cast<const uint4*>(blk);
+        r.h0 = *reinterpret_cast<const uint4*>(blk + 16);
+        r.h1 = *reinterpret_cast<const uint4*>(blk + 32);
+        r.q0 = q[0];
+        r.q1 = q[1];
+        return r;
+    }
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t kc, uint32_t h) {
+        const uint32_t g = 2u * (kc & 1u) + h;
+        uint32_t sc, mn;
+        q4k_scale_pair(r.hdr.y, r.hdr.z, r.hdr.w, (int)g, sc, mn);
+        const float d = h2f(r.hdr.x & 0xFFFFu), dmin = h2f(r.hdr.x >> 16);
+        Dec o;
+        o.d1[0] = d * (float)(sc & 0xFFu) * 16777216.f;
+        o.d1[1] = d * (float)(sc >> 8) * 16777216.f;
+        o.c1[0] = -(dmin * (float)(mn & 0xFFu));
+        o.c1[1] = -(dmin * (float)(mn >> 8));
+        o.bit = 2u * g;
+        return o;
+    }
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int sub = S / 4, p = S % 4, wi = 2 * p + HF;   // word wi of the 32-byte nibble slice and of qh
+        const uint32_t w = wi == 0 ? r.q0.x : wi == 1 ? r.q0.y : wi == 2 ? r.q0.z : wi == 3 ? r.q0.w : wi == 4 ? r.q1.x : wi == 5 ? r.q1.y : wi == 6 ? r.q1.z : r.q1.w;
+        const uint32_t qh = wi == 0 ? r.h0.x : wi == 1 ? r.h0.y : wi == 2 ? r.h0.z : wi == 3 ? r.h0.w : wi == 4 ? r.h1.x : wi == 5 ? r.h1.y : wi == 6 ? r.h1.z : r.h1.w;
+        const uint32_t code = ((sub ? w >> 4 : w) & 0x0F0F0F0Fu) | (((qh >> (dc.bit + sub)) & 0x01010101u) << 4);
+        const half2_t ev = as_h2(code & 0x00FF00FFu), od = as_h2((code >> 8) & 0x00FF00FFu);   // bytes (0,2), (1,3)
+        const float d1 = dc.d1[sub], c1 = dc.c1[sub];
+        f.u[2 * HF] = mix_pair(ev.x, od.x, d1, c1);
+        f.u[2 * HF + 1] = mix_pair(ev.y, od.y, d1, c1);
+    }
+    template <int S>
+    __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
+    }
+};
+
+// MXFP4 planes (E2M1 codes, element j in the low and j + 16 in the high nibble of byte j of a 16-byte block; one E8M0
+// exponent per block; include/ie/quant_blocks.hpp:46-54): lane half h owns blocks 4 kc + 2 h and + 1.  A code goes
+// through the byte table of the int-dot kernels (doubled E2M1 value as int8), is bias-flipped into an unsigned byte and
+// then takes the Q8_0 route: half(fma((b ^ 0x80) * 2^-24, s * 2^24, -128 s)) = half(b * s) with s = 2^(e-128), which is
+// half(e2m1 * 2^(e-127)), the reference's dequantized weight (src/ops/dequant_kernels.cpp:325-390), bit for bit.
+// Rows may end half way through a chunk (K % 128 = 64, e.g. K = 2880): the dead lane half re-reads the live one's
+// bytes and gets scale 0.
+struct GemmMxfp4Soa {
+    struct W {
+        const uint8_t* qs;
+        const uint8_t* e;
+        uint32_t K;
+    };
+    struct Bank {
+        const uint8_t* qs;
+        const uint8_t* e;
+        uint64_t qs_stride, e_stride;
+        uint32_t K;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return {b.qs + (size_t)e * b.qs_stride, b.e + (size_t)e * b.e_stride, b.K}; }
+    struct Raw {
+        uint4 q[2];
+        uint32_t e0, e1;
+        uint32_t live;
+    };
+    struct Dec {
+        float d[2], o[2];
+    };
+    static constexpr uint32_t K_ALIGN = 64;
+    static constexpr uint32_t H_COL = 8;
+    __device__ static constexpr uint32_t step_col(int S) { return (uint32_t)S; }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
+        const bool live = 128u * kc + 64u * h < w.K;
+        const uint32_t b0 = 4u * kc + (live ? 2u * h : 0u);
+        const uint4* p = reinterpret_cast<const uint4*>(w.qs + (size_t)n * (w.K >> 1) + (size_t)b0 * 16u);
+        const uint8_t* e = w.e + (size_t)n * (w.K >> 5) + b0;
+        Raw r;
+        r.q[0] = p[0];
+        r.q[1] = p[1];
+        r.e0 = e[0];
+        r.e1 = e[1];
+        r.live = live ? 1u : 0u;
+        return r;
+    }
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t, uint32_t) {
+        const float s0 = r.live ? e8m0_half(r.e0) : 0.f, s1 = r.live ? e8m0_half(r.e1) : 0.f;
+        Dec o;
+        o.d[0] = s0 * 16777216.f;
+        o.d[1] = s1 * 16777216.f;
+        o.o[0] = -128.f * s0;
+        o.o[1] = -128.f * s1;
+        return o;
+    }
+    template <int S, int HF>
+    __device__ static __forceinline__ void frag_half(const Raw& r, const Dec& dc, Frag& f) {
+        constexpr int blk = S / 4, j = 2 * (S % 2) + HF, hi = (S % 4) / 2;   // word j of the block, nibble half
+        const uint32_t w = j == 0 ? r.q[blk].x : j == 1 ? r.q[blk].y : j == 2 ? r.q[blk].z : r.q[blk].w;
+        const uint32_t nib = hi ? w >> 4 : w;
+        const uint32_t b = mxfp4_lut4(nib & 0x07070707u, ((nib >> 1) & 0x04040404u) | 0x03020100u) ^ 0x80808080u;
+        const float d = dc.d[blk], o = dc.o[blk];
+        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, b, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, b, 0x0C030C02u));
+        f.u[2 * HF] = mix_pair(w01.x, w01.y, d, o);
+        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, d, o);
+    }
+    template <int S>
+    __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
+        frag_half<S, 0>(r, dc, f);
+        frag_half<S, 1>(r, dc, f);
+    }
+};
+
+// K-quant expert regions stored as per-field streams (include/ie/quant_soa.hpp:33-51,127-157: Q4_K qs[128] x nb |
+// scales[12] x nb | {d,dmin}[4] x nb; Q6_K ql[128] x nb | qh[64] x nb | scales[16] x nb | d[2] x nb): the same words as
+// the AoS blocks from other addresses, so fragments, scales and arithmetic are inherited.
+struct GemmQ4KStr : GemmQ4K {
+    struct W {
+        const uint8_t* qs;
+        const uint8_t* sc;
+        const uint8_t* dm;
+        uint32_t bpr;
+    };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint64_t nb;
+        uint32_t bpr;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) {
+        const uint8_t* p = b.base + (size_t)e * b.expert_stride_bytes;
+        return {p, p + b.nb * 128u, p + b.nb * 140u, b.bpr};
+    }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t h) {
+        const size_t ib = (size_t)n * w.bpr + (kc >> 1);
+        const uint4* q = reinterpret_cast<const uint4*>(w.qs + ib * 128u + (2u * (kc & 1u) + h) * 32u);
+        const uint32_t* sc = reinterpret_cast<const uint32_t*>(w.sc + ib * 12u);
+        Raw r;
+        r.hdr = make_uint4(*reinterpret_cast<const uint32_t*>(w.dm + ib * 4u), sc[0], sc[1], sc[2]);
+        r.q0 = q[0];
+        r.q1 = q[1];
+        return r;
+    }
+};
+struct GemmQ6KStr : GemmQ6K {
+    struct W {
+        const uint8_t* ql;
+        const uint8_t* qh;
+        const uint8_t* sc;
+        const uint8_t* d;
+        uint32_t bpr;
+    };
+    struct Bank {
+        const uint8_t* base;
+        uint64_t expert_stride_bytes;
+        uint64_t nb;
+        uint32_t bpr;
+    };
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) {
+        const uint8_t* p = b.base + (size_t)e * b.expert_stride_bytes;
+        return {p, p + b.nb * 128u, p + b.nb * 192u, p + b.nb * 208u, b.bpr};
+    }
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t kc, uint32_t j) {
+        const size_t ib = (size_t)n * w.bpr + (kc >> 1);
+        const uint32_t c = kc & 1u;
+        Raw r;
+        r.qla = load_u4_a2(w.ql + ib * 128u + 64u * c + 16u * j);
+        r.qlb = load_u4_a2(w.ql + ib * 128u + 64u * c + 32u + 16u * j);
+        r.qh = load_u4_a2(w.qh + ib * 64u + 32u * c + 16u * j);
+        r.sc = load_u2_a2(w.sc + ib * 16u + 8u * c);
+        r.d = *reinterpret_cast<const uint16_t*>(w.d + ib * 2u);
+        return r;
+    }
+};
+
 // ---------------------------------------------------------------- kernel
-enum { GEMM_DENSE = 0, GEMM_MOE_GATE_UP_SILU = 1, GEMM_MOE_DOWN = 2 };
+// GEMM_MOE_GATE_UP_OAI: gpt-oss gate/up, out = half(swiglu_oai(half(g + bias_g), half(u + bias_u))) (src/ops/elementwise.cpp:
+// 468-492); GEMM_MOE_DOWN with `bias0`: out = half(half(acc) + bias) (gemv out, then add_bias, elementwise.cpp:782-793).
+enum { GEMM_DENSE = 0, GEMM_MOE_GATE_UP_SILU = 1, GEMM_MOE_DOWN = 2, GEMM_MOE_GATE_UP_OAI = 3 };
 
 struct GemmArgs {
     const half_t* A;                  // [M, K] fp16 (dense) or expert-sorted rows [TK, K]
@@ -416,9 +620,16 @@ struct GemmArgs {
     uint32_t tiles_m, tiles_n;        // dense tile grid; grouped: tiles_m is an upper bound
     uint32_t k_split;                 // dense only: K slices per output tile (above 1: fp32 partial sums go to split_acc)
     float* split_acc;                 // [k_split][M][N] partial sums of a K-sliced launch
+    const float* bias0;               // [E][N] fp32 or NULL: gate bias (GEMM_MOE_GATE_UP_OAI), down bias (GEMM_MOE_DOWN)
+    const float* bias1;               // [E][N] up bias
+    float alpha, limit;               // swiglu_oai
 };
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
+__device__ __forceinline__ float swiglu_oai_f(float g, float u, float alpha, float limit) {
+    const float x = fminf(g, limit), z = fmaxf(fminf(u, limit), -limit);
+    return (x / (1.f + __expf(alpha * -x))) * (z + 1.f);
+}
 
 // Dense launches with too few output tiles for the chip (a short batch against a narrow matrix) cut K into up to
 // eight slices: every slice writes its fp32 partial sums to its own plane of a scratch buffer, and a last launch adds
@@ -550,20 +761,38 @@ struct TileCtx {
     const uint8_t* lds_raw;
     uint32_t frag0, n_chunks, mi;
     uint32_t c0;   // first chunk of this K slice (chunk numbers below are slice-local)
+    uint32_t tail_chunk;   // row-relative number of the chunk whose upper 64 columns lie past K (0xFFFFFFFF: none)
+    uint32_t row_step;     // (BM / 4) * wave, for the A column of a lane
 };
+
+// The A rows of chunk `c` (slice-local) into the LDS buffer at `dst`.  In a chunk that ends half way (K % 128 = 64) a lane
+// whose column lies past K reads the column 8 below instead (the same row, inside K): the weights of those columns are
+// zero, so any finite value will do, and nothing is read past the row.
+template <class QF, int NA>
+__device__ __forceinline__ void a_rows_to_lds(const TileCtx<QF, NA>& t, const uint32_t (&a_off)[2 * NA], uint32_t c, uint32_t dst) {
+    const uint8_t* src = t.a_glb + (size_t)c * (kBK * 2u);
+    if (QF::K_ALIGN == 64 && t.c0 + c == t.tail_chunk) {
+        const uint32_t lane = threadIdx.x & 63u;
+#pragma unroll
+        for (int j = 0; j < 2 * NA; ++j) {
+            const uint32_t R = t.row_step + 4u * j + (lane >> 4), col = (lane & 15u) ^ (R & 15u);
+            load_to_lds16(src, a_off[j] - ((col & 8u) << 4), dst + 1024u * j);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2 * NA; ++j) load_to_lds16(src, a_off[j], dst + 1024u * j);
+    }
+}
 
 // Chunk c out of register set P; meanwhile (`more`) the A rows of chunk c+1 and the weights of chunk c+DEPTH are requested.
 template <class QF, bool PARTIAL, int NA, int DEPTH, int P>
 __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint32_t (&a_off)[2 * NA], typename QF::Raw (&raw)[DEPTH + 1][2],
                                            float16_t (&acc)[NA][2], uint32_t c, bool more) {
-    constexpr int NSET = DEPTH + 1, PN = (P + DEPTH) % NSET, NL = 2 * NA;
+    constexpr int NSET = DEPTH + 1, PN = (P + DEPTH) % NSET;
     constexpr uint32_t ABUF = 32u * NA * kBK * 2u;
     constexpr int W_LOADS_MIN = 2 * (int)((sizeof(typename QF::Raw) + 15) / 16);
     if (more) {
-        const uint8_t* a_next = t.a_glb + (size_t)(c + 1) * (kBK * 2u);
-        const uint32_t dst = t.a_dst + ((c + 1) & 1u) * ABUF;
-#pragma unroll
-        for (int j = 0; j < NL; ++j) load_to_lds16(a_next, a_off[j], dst + 1024u * j);
+        a_rows_to_lds<QF, NA>(t, a_off, c + 1, t.a_dst + ((c + 1) & 1u) * ABUF);
         const uint32_t cn = (c + DEPTH < t.n_chunks) ? c + DEPTH : t.n_chunks - 1;   // past the end: the last chunk again, unused
         raw[PN][0] = QF::load(t.w0, t.wrow0, t.c0 + cn, t.h);
         raw[PN][1] = QF::load(t.w1, t.wrow1, t.c0 + cn, t.h);
@@ -595,16 +824,17 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
 template <class QF, int MODE, bool PIPE, int NA, int DEPTH>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::W& w0, const typename QF::W& w1, const uint32_t (&wrow)[2],
                                           uint32_t row_lo, uint32_t row_hi, uint32_t n_base, uint8_t* lds_raw, uint32_t c0 = 0,
-                                          uint32_t n_chunks_slice = 0, uint32_t ks = 0) {
+                                          uint32_t n_chunks_slice = 0, uint32_t ks = 0, uint32_t e = 0) {
     static_assert(DEPTH == 1 || DEPTH == 2, "prefetch depth");
     static_assert(!PIPE || NA == 4, "the pipelined chunk is written for four token tiles");
-    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
+    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI;
     constexpr bool PARTIAL = MODE != GEMM_DENSE && !PIPE;
     constexpr uint32_t BM = 32u * NA;
     constexpr int NL = 2 * NA;   // 1 KB loads per wave per chunk
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 31u, h = lane >> 5;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t n_chunks = n_chunks_slice ? n_chunks_slice : g.K / kBK;   // chunks of this K slice (all of K unless split)
+    const uint32_t n_all = (g.K + kBK - 1) / kBK;                             // a row that ends half way through its last chunk counts it
+    const uint32_t n_chunks = n_chunks_slice ? n_chunks_slice : n_all;       // chunks of this K slice (all of K unless split)
     const uint32_t live_rows = (row_hi - row_lo) >= BM ? BM : row_hi - row_lo;
     const uint32_t mi = (live_rows + 31u) / 32u;
 
@@ -636,8 +866,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
     // over the sets so that no set is ever copied into another (a register copy of loaded data waits for the load).
     constexpr int NSET = DEPTH + 1;
     typename QF::Raw raw[NSET][2];
-#pragma unroll
-    for (int j = 0; j < NL; ++j) load_to_lds16(a_glb, a_off[j], a_dst + 1024u * j);
+    const TileCtx<QF, NA> ctx{w0, w1, wrow[0], wrow[1], h, a_glb, a_dst, lds_raw, frag0, n_chunks, mi, c0,
+                              (g.K % kBK) ? n_all - 1u : 0xFFFFFFFFu, (BM / 4u) * wave};
+    a_rows_to_lds<QF, NA>(ctx, a_off, 0, a_dst);
     raw[0][0] = QF::load(w0, wrow[0], c0, h);
     raw[0][1] = QF::load(w1, wrow[1], c0, h);
     wait_vmcnt<0>();
@@ -649,7 +880,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
         raw[d][1] = QF::load(w1, wrow[1], c0 + cd, h);
     }
 
-    const TileCtx<QF, NA> ctx{w0, w1, wrow[0], wrow[1], h, a_glb, a_dst, lds_raw, frag0, n_chunks, mi, c0};
 #define CHUNK(P, c, more) gemm_chunk<QF, PARTIAL, NA, DEPTH, P>(ctx, a_off, raw, acc, c, more)
     if constexpr (DEPTH == 1) {
         // two sets, and the set just loaded is copied into set 0 at the end of a chunk, where it has to have arrived anyway
@@ -682,7 +912,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
             if (row >= row_hi) continue;
             if (GATE_UP) {
                 const uint32_t n = n_base + r;
-                if (n < g.N) g.Y[(size_t)row * g.N + n] = (half_t)silu_mul_f(acc[i][0][v], acc[i][1][v]);
+                if (n >= g.N) continue;
+                if (MODE == GEMM_MOE_GATE_UP_OAI) {
+                    const float gg = (float)(half_t)(acc[i][0][v] + (g.bias0 ? g.bias0[(size_t)e * g.N + n] : 0.f));
+                    const float uu = (float)(half_t)(acc[i][1][v] + (g.bias1 ? g.bias1[(size_t)e * g.N + n] : 0.f));
+                    g.Y[(size_t)row * g.N + n] = (half_t)swiglu_oai_f(gg, uu, g.alpha, g.limit);
+                } else {
+                    g.Y[(size_t)row * g.N + n] = (half_t)silu_mul_f(acc[i][0][v], acc[i][1][v]);
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -694,6 +931,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
                         __hip_atomic_fetch_add(g.y_acc + (size_t)g.row_token[row] * g.N + n, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     else if (MODE == GEMM_DENSE && g.k_split > 1)
                         g.split_acc[((size_t)ks * g.M + row) * g.N + n] = o;
+                    else if (MODE == GEMM_MOE_DOWN && g.bias0)
+                        g.Y[(size_t)row * g.N + n] = (half_t)((float)(half_t)o + g.bias0[(size_t)e * g.N + n]);
                     else
                         g.Y[(size_t)row * g.N + n] = (half_t)o;
                 }
@@ -707,7 +946,7 @@ template <class QF, int MODE, int NI>
 __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     constexpr uint32_t BM = 32u * NI;   // tokens per tile
-    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU;
+    constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI;
     constexpr uint32_t BN = GATE_UP ? 4 * 32 : 4 * kWaveN;   // output columns per workgroup
 
     // ---- which tile: XCD-aware order (workgroup i runs on XCD i % 8; each XCD walks a
@@ -784,7 +1023,7 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     if (wrow[1] >= g.N) wrow[1] = g.N - 1;
 
     if constexpr (MODE == GEMM_DENSE) {
-        const uint32_t n_all = g.K / kBK, per = (n_all + ksplit - 1) / ksplit;
+        const uint32_t n_all = (g.K + kBK - 1) / kBK, per = (n_all + ksplit - 1) / ksplit;
         const uint32_t c0 = ks * per, c1 = (c0 + per < n_all) ? c0 + per : n_all;
         gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, c0, c1 - c0, ks);
     } else {
@@ -792,16 +1031,16 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
         // expert-grouped tiles: a full one takes the same pipelined chunk as the dense GEMM; one with at most 64
         // live rows keeps half the accumulators and spends the registers on a second chunk of weights in flight
         const uint32_t live = row_hi - row_lo;
-        if (live >= BM) gemm_tile<QF, MODE, true, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
-        else if (live <= 64u) gemm_tile<QF, MODE, false, 2, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
-        else gemm_tile<QF, MODE, false, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw);
+        if (live >= BM) gemm_tile<QF, MODE, true, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
+        else if (live <= 64u) gemm_tile<QF, MODE, false, 2, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
+        else gemm_tile<QF, MODE, false, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
     }
 }
 
 // ---------------------------------------------------------------- host side
 template <class QF, int MODE, int NI>
 static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
-    constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU) ? 128 : 256, BM = 32u * NI, lds = 2u * BM * kBK * 2u;
+    constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI) ? 128 : 256, BM = 32u * NI, lds = 2u * BM * kBK * 2u;
     g.tiles_n = (g.N + BN - 1) / BN;
     g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + BM - 1) / BM : rows_bound / BM + g.E;   // grouped: an upper bound, workgroups past the real count leave at once
     if (MODE != GEMM_DENSE || g.k_split == 0) g.k_split = 1;
@@ -841,7 +1080,7 @@ static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typenam
         const uint64_t cus = (uint64_t)gemm_cu_count();
         const uint64_t tiles128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 255) / 256);
         const uint64_t tiles64 = (uint64_t)((g.M + 63) / 64) * ((g.N + 255) / 256);
-        const uint64_t mn = (uint64_t)g.M * g.N, n_chunks = g.K / kBK;
+        const uint64_t mn = (uint64_t)g.M * g.N, n_chunks = (g.K + kBK - 1) / kBK;
         const uint64_t cap = caller_ws ? caller_ws->elems : kGemmSplitElems;   // partial sums the scratch holds
         // K slices a tiling could take: until every CU has a workgroup, each slice at least 8 chunks deep, the partial
         // sums within the scratch
@@ -909,9 +1148,15 @@ static int moe_gemm_aos(mx_stream_t s, const uint16_t* rows, const void* W0, con
     g.A = reinterpret_cast<const half_t*>(rows); g.Y = reinterpret_cast<half_t*>(out); g.expert_offsets = expert_offsets;
     g.route_w = reinterpret_cast<const half_t*>(sorted_w); g.M = total_rows; g.K = K; g.N = N; g.E = E;
     g.row_token = row_token; g.y_acc = y_acc;
-    const uint32_t row_bytes = K / 256 * block_bytes;
-    typename QF::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
-    return launch_gemm<QF, MODE>(s, b0, b1, g, total_rows);
+    if constexpr (std::is_same<QF, GemmQ4KStr>::value || std::is_same<QF, GemmQ6KStr>::value) {
+        const uint64_t nb = (uint64_t)N * (K / 256);
+        typename QF::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, nb, K / 256}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, nb, K / 256};
+        return launch_gemm<QF, MODE>(s, b0, b1, g, total_rows);
+    } else {
+        const uint32_t row_bytes = K / 256 * block_bytes;
+        typename QF::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, row_bytes}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, row_bytes};
+        return launch_gemm<QF, MODE>(s, b0, b1, g, total_rows);
+    }
 }
 
 // Dense entry points.  ws = NULL: K-sliced launches keep their partial sums in the library's per-device scratch.
@@ -1025,22 +1270,71 @@ int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d
     return launch_gemm<GemmQ8Soa, GEMM_MOE_DOWN>(s, b, b, g, total_rows);
 }
 
+// soa != 0: every expert region holds its blocks as per-field streams (include/ie/quant_soa.hpp:33-51)
 int mx_moe_gemm_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x_packed, const void* gate_W, const void* up_W, const uint32_t* expert_offsets,
-                                 uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+                                 uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
+    if (soa)
+        return moe_gemm_aos<GemmQ4KStr, GEMM_MOE_GATE_UP_SILU>(s, x_packed, gate_W, up_W, expert_stride_bytes, expert_offsets, nullptr, h_packed, E, H, E_ffn,
+                                                               total_rows, kQ4KBytes, 16);
     return moe_gemm_aos<GemmQ4K, GEMM_MOE_GATE_UP_SILU>(s, x_packed, gate_W, up_W, expert_stride_bytes, expert_offsets, nullptr, h_packed, E, H, E_ffn,
                                                         total_rows, kQ4KBytes, 16);
 }
 
 int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const uint16_t* sorted_w,
-                         uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+                         uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
+    if (soa)
+        return moe_gemm_aos<GemmQ4KStr, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
+                                                       total_rows, kQ4KBytes, 16);
     return moe_gemm_aos<GemmQ4K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
                                                 total_rows, kQ4KBytes, 16);
 }
 
 int mx_moe_gemm_down_q6k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const uint16_t* sorted_w,
-                         uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, uint32_t total_rows) {
+                         uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
+    if (soa)
+        return moe_gemm_aos<GemmQ6KStr, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
+                                                       total_rows, kQ6KBytes, 2);
     return moe_gemm_aos<GemmQ6K, GEMM_MOE_DOWN>(s, h_packed, down_W, down_W, expert_stride_bytes, expert_offsets, sorted_w, out_packed, E, E_ffn, H,
                                                 total_rows, kQ6KBytes, 2);
+}
+
+// ---- MXFP4 planes and Q5_K blocks through the fused kernel (the reference dequantizes both to a [K, N] fp16 matrix and
+// runs a plain GEMM: src/ops/gemv_mxfp4.cpp:316-341, src/model/gptoss.cpp:389-392, include/ie/dequant.hpp:81-86)
+int mx_gemm_q5_K(mx_stream_t s, const uint16_t* A, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    return gemm_dense_aos<GemmQ5K>(s, A, W, y, M, K, N, 256, 16, K / 256 * 176u, nullptr);
+}
+int mx_gemm_mxfp4_soa(mx_stream_t s, const uint16_t* A, const uint8_t* qs_W, const uint8_t* e_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    if (int rc = check_gemm(A, qs_W, y, M, K, N, 64)) return rc;
+    MX_REQUIRE_PTR(e_W);
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(A); g.Y = reinterpret_cast<half_t*>(y); g.M = M; g.K = K; g.N = N; g.E = 1;
+    GemmMxfp4Soa::Bank b{qs_W, e_W, 0, 0, K};
+    return launch_gemm<GemmMxfp4Soa, GEMM_DENSE>(s, b, b, g, M, nullptr);
+}
+int mx_moe_gemm_gate_up_oai_mxfp4(mx_stream_t s, const uint16_t* x_packed, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
+                                  uint64_t qs_stride, uint64_t e_stride, const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets,
+                                  uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha, float limit) {
+    if (int rc = check_gemm(x_packed, g_qs, h_packed, total_rows, H, E_ffn, 64)) return rc;
+    MX_REQUIRE_PTR(g_e); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_e); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(E > 0 && qs_stride % 16 == 0);
+    MX_REQUIRE_ALIGN(u_qs, 16);
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(x_packed); g.Y = reinterpret_cast<half_t*>(h_packed); g.expert_offsets = expert_offsets;
+    g.M = total_rows; g.K = H; g.N = E_ffn; g.E = E; g.bias0 = gate_bias; g.bias1 = up_bias; g.alpha = alpha; g.limit = limit;
+    GemmMxfp4Soa::Bank bg{g_qs, g_e, qs_stride, e_stride, H}, bu{u_qs, u_e, qs_stride, e_stride, H};
+    return launch_gemm<GemmMxfp4Soa, GEMM_MOE_GATE_UP_OAI>(s, bg, bu, g, total_rows);
+}
+int mx_moe_gemm_down_mxfp4(mx_stream_t s, const uint16_t* h_packed, const uint8_t* d_qs, const uint8_t* d_e, uint64_t qs_stride, uint64_t e_stride,
+                           const float* down_bias, const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                           uint32_t total_rows) {
+    if (int rc = check_gemm(h_packed, d_qs, out_packed, total_rows, E_ffn, H, 64)) return rc;
+    MX_REQUIRE_PTR(d_e); MX_REQUIRE_PTR(expert_offsets);
+    MX_REQUIRE_SHAPE(E > 0 && qs_stride % 16 == 0);
+    GemmArgs g{};
+    g.A = reinterpret_cast<const half_t*>(h_packed); g.Y = reinterpret_cast<half_t*>(out_packed); g.expert_offsets = expert_offsets;
+    g.M = total_rows; g.K = E_ffn; g.N = H; g.E = E; g.bias0 = down_bias;
+    GemmMxfp4Soa::Bank b{d_qs, d_e, qs_stride, e_stride, E_ffn};
+    return launch_gemm<GemmMxfp4Soa, GEMM_MOE_DOWN>(s, b, b, g, total_rows);
 }
 
 // moe_prefill_proj_q4_0_xmx (include/ie/ops.hpp:192-204): plain projection of expert-sorted fp16 rows through Q4_0 experts.

@@ -1,9 +1,7 @@
-// gemm_fp16.cpp — the plain fp16 x fp16 GEMM the dequant-to-Bt route feeds (formats without a fused
-// quant-GEMM: Q5_K, MXFP4, anything a caller has already dequantized).  The reference has a
-// hand-tiled joint_matrix kernel (gemm_fp16, src/ops/gemm_fp16.cpp:46-178) and a oneDNN matmul
-// (gemm_fp16_onednn, src/ops/gemm_onednn.cpp:75-111); a plain dense GEMM is library work, so both map
-// onto rocBLAS' gemm_ex here (fp16 operands, fp32 accumulate).  rocBLAS is loaded on first use, so
-// the rest of the library carries no dependency on it.
+// gemm_fp16.cpp — gemm_fp16_onednn: the reference's vendor-library matmul (oneDNN, src/ops/gemm_onednn.cpp:75-111;
+// fp16 in and out, fp32 accumulate) maps onto the vendor library of this platform, rocBLAS' gemm_ex.  rocBLAS is loaded
+// on first use, so the rest of the library carries no dependency on it.  (The reference's own tiled kernel, gemm_fp16
+// with fp32 output, is the hand-written kernel in gemm_f16_tiled.hip.)
 #include <dlfcn.h>
 #include <rocblas/rocblas.h>
 
@@ -29,8 +27,9 @@ rocblas_handle g_handle[kMaxDevices] = {};
 bool load_api() {
     if (g_tried) return g_api.ok;
     g_tried = true;
-    void* h = dlopen("librocblas.so.5", RTLD_NOW | RTLD_LOCAL);
-    if (!h) h = dlopen("librocblas.so", RTLD_NOW | RTLD_LOCAL);
+    void* h = dlopen("librocblas.so", RTLD_NOW | RTLD_LOCAL);   // the unversioned name first, then the sonames ROCm 6 / 7 ship
+    for (const char* name : {"librocblas.so.5", "librocblas.so.4"})
+        if (!h) h = dlopen(name, RTLD_NOW | RTLD_LOCAL);
     if (!h) return false;
     g_api.create = reinterpret_cast<decltype(g_api.create)>(dlsym(h, "rocblas_create_handle"));
     g_api.set_stream = reinterpret_cast<decltype(g_api.set_stream)>(dlsym(h, "rocblas_set_stream"));
@@ -66,9 +65,6 @@ int gemm_rowmajor(mx_stream_t s, const void* A, const void* B, void* C, rocblas_
 
 extern "C" {
 
-int mx_gemm_fp16(mx_stream_t s, const uint16_t* A, const uint16_t* B, float* C, uint32_t M, uint32_t N, uint32_t K) {
-    return gemm_rowmajor(s, A, B, C, rocblas_datatype_f32_r, M, N, K);
-}
 int mx_gemm_fp16_onednn(mx_stream_t s, const uint16_t* A, const uint16_t* B, uint16_t* y, uint32_t M, uint32_t N, uint32_t K) {
     return gemm_rowmajor(s, A, B, y, rocblas_datatype_f16_r, M, N, K);
 }

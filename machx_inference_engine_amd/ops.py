@@ -714,18 +714,48 @@ def gemm_q8_0(A, W, M, K, N, y=None):
     return y
 
 
-def moe_gemm_gate_up_silu_q4k(x_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None):
+def moe_gemm_gate_up_silu_q4k(x_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None, soa=False):
+    """soa: the expert regions hold per-field streams (repack_moe_kquant_soa) instead of GGUF blocks."""
     h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
     _call("mx_moe_gemm_gate_up_silu_q4k", _f16(x_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
-          expert_stride_bytes, TK)
+          expert_stride_bytes, 1 if soa else 0, TK)
     return h_packed
 
 
-def moe_gemm_down_kquant(fmt, h_packed, down_W, expert_offsets, sorted_w, TK, E, H, E_ffn, expert_stride_bytes, out_packed=None):
+def moe_gemm_down_kquant(fmt, h_packed, down_W, expert_offsets, sorted_w, TK, E, H, E_ffn, expert_stride_bytes, out_packed=None, soa=False):
     """fmt in ('q4k', 'q6k'); sorted_w None -> unweighted packed rows."""
     out_packed = _out(out_packed, (TK, H), torch.float16, h_packed)
     _call("mx_moe_gemm_down_%s" % fmt, _f16(h_packed), _u8(down_W), _ptr(expert_offsets), _f16(sorted_w) if sorted_w is not None else None,
-          _ptr(out_packed), E, H, E_ffn, expert_stride_bytes, TK)
+          _ptr(out_packed), E, H, E_ffn, expert_stride_bytes, 1 if soa else 0, TK)
+    return out_packed
+
+
+def gemm_q5_K(A, W, M, K, N, y=None):
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_q5_K", _f16(A), _u8(W), _ptr(y), M, K, N)
+    return y
+
+
+def gemm_mxfp4_soa(A, qs_plane, e_plane, M, K, N, y=None):
+    """y[M,N] = A . half(deq(W))^T for MXFP4 planes, K % 64 == 0 (fused: no [K,N] fp16 matrix is written)."""
+    y = _out(y, (M, N), torch.float16, A)
+    _call("mx_gemm_mxfp4_soa", _f16(A), _u8(qs_plane), _u8(e_plane), _ptr(y), M, K, N)
+    return y
+
+
+def moe_gemm_gate_up_oai_mxfp4(x_packed, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, expert_offsets, TK, E, H, E_ffn,
+                               alpha=1.702, limit=7.0, h_packed=None):
+    h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
+    _call("mx_moe_gemm_gate_up_oai_mxfp4", _f16(x_packed), _u8(g_qs), _u8(g_e), _u8(u_qs), _u8(u_e), qs_stride, e_stride,
+          _ptr(gate_bias) if gate_bias is not None else None, _ptr(up_bias) if up_bias is not None else None, _ptr(expert_offsets), _ptr(h_packed),
+          E, H, E_ffn, TK, float(alpha), float(limit))
+    return h_packed
+
+
+def moe_gemm_down_mxfp4(h_packed, d_qs, d_e, qs_stride, e_stride, down_bias, expert_offsets, TK, E, H, E_ffn, out_packed=None):
+    out_packed = _out(out_packed, (TK, H), torch.float16, h_packed)
+    _call("mx_moe_gemm_down_mxfp4", _f16(h_packed), _u8(d_qs), _u8(d_e), qs_stride, e_stride, _ptr(down_bias) if down_bias is not None else None,
+          _ptr(expert_offsets), _ptr(out_packed), E, H, E_ffn, TK)
     return out_packed
 
 

@@ -62,21 +62,42 @@ def onehot_weights_through_gemm(gemm, K, N):
     """A = rows of the identity: Y[t, n] is the kernel's own fp16 weight W16[n, k0 + t]."""
     out = np.zeros((N, K), np.float32)
     for k0 in range(0, K, 128):
+        n = min(128, K - k0)
         A = np.zeros((128, K), np.float32)
-        A[np.arange(128), k0 + np.arange(128)] = 1.0
-        out[:, k0:k0 + 128] = host(gemm(dev(A).half())).astype(np.float32).T
+        A[np.arange(n), k0 + np.arange(n)] = 1.0
+        out[:, k0:k0 + n] = host(gemm(dev(A).half())).astype(np.float32).T[:, :n]
     return out
 
 
-@pytest.mark.parametrize("fmt,K", [("q4_K", 512), ("q6_K", 512), ("q8_0", 256)])
+def q5k_blocks(seed, N, K):
+    """Q5_K blocks from Q4_K ones: same header and nibbles, seeded high bits (the oracle has no Q5_K quantizer)."""
+    b4 = O.quantize(O.Q4_K, O.normal(seed, (N, K), 0.0, 0.02)).reshape(-1, 144)
+    return np.ascontiguousarray(np.concatenate([b4[:, :16], O.rand_bytes(seed + 1, b4.shape[0] * 32).reshape(-1, 32), b4[:, 16:]], axis=1)).reshape(-1)
+
+
+@pytest.mark.parametrize("fmt,K", [("q4_K", 512), ("q6_K", 512), ("q8_0", 256), ("q5_K", 512), ("mxfp4", 320)])
 def test_gemm_weight_fragments_bit_exact(mx, fmt, K):
     """The fp16 weights the GEMM multiplies by equal half(reference dequant) element for element
-    (include/ie/dequant_ref.hpp), read back through one-hot activations."""
-    F = {"q4_K": O.Q4_K, "q6_K": O.Q6_K, "q8_0": O.Q8_0}[fmt]
+    (include/ie/dequant_ref.hpp), read back through one-hot activations.  MXFP4 at K = 320: the row ends half way
+    through its last 128-element chunk, as K = 2880 does."""
+    F = {"q4_K": O.Q4_K, "q6_K": O.Q6_K, "q8_0": O.Q8_0, "q5_K": O.Q5_K, "mxfp4": O.MXFP4}[fmt]
     N = 256
-    W = weights(F, 2300, N, K)
+    if fmt == "q5_K":
+        W = q5k_blocks(2300, N, K)
+    elif fmt == "mxfp4":
+        W = O.quantize(F, O.normal(2300, (N, K), 0.0, 0.02))
+        # a few blocks at exponents where half(value) is zero, subnormal or near the top of the fp16 range (finite: a
+        # weight that is inf would turn the one-hot read-back of its whole row into nan)
+        Wb = W.reshape(-1, 17)
+        Wb[:8, 0] = np.array([0, 1, 100, 112, 126, 127, 139, 140], np.uint8)
+    else:
+        W = weights(F, 2300, N, K)
     ref = f16(O.dequant(F, W, N * K).reshape(N, K))
-    fn = {"q4_K": mx.ops.gemm_q4_K, "q6_K": mx.ops.gemm_q6_K, "q8_0": mx.ops.gemm_q8_0}[fmt]
+    if fmt == "mxfp4":
+        qs, e = O.repack_mxfp4_to_soa(W)
+        fn = lambda A, _W, M, K_, N_: mx.ops.gemm_mxfp4_soa(A, dev(qs), dev(e), M, K_, N_)
+    else:
+        fn = {"q4_K": mx.ops.gemm_q4_K, "q6_K": mx.ops.gemm_q6_K, "q8_0": mx.ops.gemm_q8_0, "q5_K": mx.ops.gemm_q5_K}[fmt]
     got = onehot_weights_through_gemm(lambda A: fn(A, dev(W), 128, K, N), K, N)
     # value equality: a zero weight may come out as +0 where the reference expression gives -0
     # (Q6_K code 32 under a negative scale); the sign of a zero cannot change a dot product
@@ -243,6 +264,11 @@ def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
             u = O.gemv_f64(O.Q4_K, Wu[e], xs[rows], H, EF, round_w_fp16=True)
             h_ref[rows] = O.swiglu_np(g.astype(np.float32), u.astype(np.float32))
     check(hp_h, h_ref, "moe grouped gate_up silu q4k (MFMA)")
+    # soa = 1: the same blocks as per-field streams per expert region: the same fragments, so the same bits
+    nb_gu = EF * H // 256
+    Wg_s, Wu_s = ops.repack_moe_kquant_soa("q4k", Wg, E, nb_gu), ops.repack_moe_kquant_soa("q4k", Wu, E, nb_gu)
+    hp_s = ops.moe_gemm_gate_up_silu_q4k(xp, dev(Wg_s), dev(Wu_s), dev(off), TK, E, H, EF, stride_gu, soa=True)
+    assert torch.equal(hp_s, hp), "soa gate/up differs from the AoS bank"
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wd = mk(F, 5100, H, EF)
         o_ref = np.zeros((TK, H), np.float64)
@@ -254,6 +280,9 @@ def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
         check(host(op).astype(np.float32), o_ref, "moe grouped down %s unweighted (MFMA)" % fmt)
         opw = ops.moe_gemm_down_kquant(fmt, hp, dev(Wd), dev(off), dev(wp).half(), TK, E, H, EF, Wd[0].size)
         check(host(opw).astype(np.float32), o_ref * f16(wp)[:, None], "moe grouped down %s weighted (MFMA)" % fmt)
+        Wd_s = ops.repack_moe_kquant_soa(fmt, Wd, E, H * EF // 256)
+        opw_s = ops.moe_gemm_down_kquant(fmt, hp, dev(Wd_s), dev(off), dev(wp).half(), TK, E, H, EF, Wd[0].size, soa=True)
+        assert torch.equal(opw_s, opw), "soa down %s differs from the AoS bank" % fmt
         # unweighted rows + moe_prefill_reduce (weights applied there) == the reference's two-step path
         y = ops.moe_prefill_reduce(op, dev(t2p.astype(np.uint32)), dev(wp).half(), torch.zeros((T, H), dtype=torch.float16, device="cuda"), T, Kt, H)
         y_ref = (host(op).astype(np.float32) * f16(wp)[:, None])[t2p].reshape(T, Kt, H).sum(axis=1)
@@ -269,14 +298,17 @@ def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
         assert np.array_equal(host(ym), (y0 + host(y32)).astype(np.float16))
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8, 32), (33, 130, 288), (256, 512, 2048)])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 32), (33, 130, 288), (256, 512, 2048), (200, 135, 73), (129, 257, 1000)])
 def test_gemm_fp16_plain(mx, M, N, K):
-    """gemm_fp16 (fp32 C) and gemm_fp16_onednn (fp16 y): A[M,K] . B[K,N], fp32 accumulation
-    (include/ie/ops.hpp:275-286,460-465), against fp64 on the same fp16 operands."""
+    """gemm_fp16 (fp32 C, the hand-tiled kernel; ragged M, N and K into an exactly sized C) and gemm_fp16_onednn (fp16 y,
+    the vendor library): A[M,K] . B[K,N], fp32 accumulation (include/ie/ops.hpp:275-286,460-465), against fp64 on the
+    same fp16 operands."""
     A = O.round_fp16(O.normal(3000 + M, (M, K), 0.0, 1.0))
     B = O.round_fp16(O.normal(3001 + N, (K, N), 0.0, 0.05))
     ref = A.astype(np.float64) @ B.astype(np.float64)
-    C = mx.ops.gemm_fp16(dev(A).half(), dev(B).half(), M, N, K)
+    guard = torch.full((M * N + 64,), 7.0, dtype=torch.float32, device="cuda")   # C sized exactly, canaries behind it
+    C = mx.ops.gemm_fp16(dev(A).half(), dev(B).half(), M, N, K, C=guard[:M * N].view(M, N))
+    assert bool((guard[M * N:] == 7.0).all()), "gemm_fp16 wrote past C"
     check(host(C).ravel(), ref.ravel(), "gemm_fp16 fp32 out", abs_floor=0.0, max_rel=2e-4)
     y = mx.ops.gemm_fp16(dev(A).half(), dev(B).half(), M, N, K, out_dtype=torch.float16)
     check(host(y).astype(np.float32).ravel(), ref.ravel(), "gemm_fp16_onednn fp16 out")
@@ -295,3 +327,71 @@ def test_q5_K_prefill_route(mx):
     assert np.array_equal(host(Bt).astype(np.float32), wd.T)
     y = mx.ops.gemm_fp16(dev(A).half(), Bt, M, N, K, out_dtype=torch.float16)
     check(host(y).astype(np.float32).ravel(), (A.astype(np.float64) @ wd.T.astype(np.float64)).ravel(), "q5_K dequant + gemm_fp16")
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 512, 256), (77, 2880, 520), (300, 2880, 2880)])
+def test_gemm_mxfp4_and_q5_K_fused(mx, M, K, N):
+    """MXFP4 planes (K = 2880: 22 chunks and a half) and Q5_K blocks through the fused kernel, against fp64 over
+    half(dequant) weights; and against the reference's own route (dequant to [K, N] fp16 + plain GEMM) on the same bits."""
+    A = f16(O.normal(8100 + M, (M, K)))
+    W = O.quantize(O.MXFP4, O.normal(8101 + N, (N, K), 0.0, 0.02))
+    qs, e = O.repack_mxfp4_to_soa(W)
+    ref = O.gemv_f64(O.MXFP4, W, A, K, N, round_w_fp16=True)
+    got = mx.ops.gemm_mxfp4_soa(dev(A).half(), dev(qs), dev(e), M, K, N)
+    check(host(got).astype(np.float32), ref, "gemm_mxfp4_soa M=%d K=%d N=%d" % (M, K, N))
+    bt = mx.ops.dequant_soa_to_Bt("mxfp4_soa", (dev(qs), dev(e)), K, N)
+    two = mx.ops.gemm_fp16(dev(A).half(), bt, M, N, K, out_dtype=torch.float16)
+    check(host(got).astype(np.float32).ravel(), host(two).astype(np.float32).ravel(), "fused vs dequant + GEMM (mxfp4)", max_rel=2e-3)
+    if K % 256 == 0:
+        W5 = q5k_blocks(8200 + N, N, K)
+        ref5 = O.gemv_f64(O.Q5_K, W5, A, K, N, round_w_fp16=True)
+        got5 = mx.ops.gemm_q5_K(dev(A).half(), dev(W5), M, K, N)
+        check(host(got5).astype(np.float32), ref5, "gemm_q5_K M=%d K=%d N=%d" % (M, K, N))
+
+
+@pytest.mark.parametrize("T,E,Kt,H,EF", [(64, 8, 2, 320, 192), (96, 32, 4, 2880, 2880)])
+def test_moe_grouped_gemm_mxfp4(mx, T, E, Kt, H, EF):
+    """gpt-oss expert banks through the grouped matrix-core GEMM on fp16 rows: half(swiglu_oai(half(g + b), half(u + b)))
+    and half(half(acc) + b), against the float chain (fp64 over half(dequant) weights) at H = EF = 2880."""
+    from test_gpu_moe import make_experts, route
+    ops = mx.ops
+    Wg, gq, ge, qs_st, e_st = make_experts(O.MXFP4, 100, E, EF, H)
+    Wu, uq, ue, _, _ = make_experts(O.MXFP4, 200, E, EF, H)
+    Wd, dq, de, dqs_st, de_st = make_experts(O.MXFP4, 300, E, H, EF)
+    bg, bu, bd = O.normal(1, (E, EF)), O.normal(2, (E, EF)), O.normal(3, (E, H))
+    x = f16(O.normal(4, (T, H)))
+    ids, w = route(5, T, E, Kt)
+    off, si, wp, t2p = ops.build_moe_packing(ids, w, E)
+    TK = T * Kt
+    xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
+    hp = ops.moe_gemm_gate_up_oai_mxfp4(xp, dev(gq), dev(ge), dev(uq), dev(ue), qs_st, e_st, dev(bg), dev(bu), dev(off), TK, E, H, EF)
+    hp_h = host(hp).astype(np.float32)
+    xs = x[si]
+    rows = np.arange(TK) if TK <= 256 else np.random.default_rng(9).choice(TK, 48, replace=False)
+    exp_of = np.searchsorted(off, rows, side="right") - 1
+    lo, hi = [], []
+    for r_, e_ in zip(rows, exp_of):
+        g = O.gemv_f64(O.MXFP4, Wg[e_], xs[r_:r_ + 1], H, EF, round_w_fp16=True)[0].astype(np.float64) + bg[e_]
+        u = O.gemv_f64(O.MXFP4, Wu[e_], xs[r_:r_ + 1], H, EF, round_w_fp16=True)[0].astype(np.float64) + bu[e_]
+        inf = np.float16(np.inf)
+        gc = [np.nextafter(f16(g).astype(np.float16), -inf), f16(g).astype(np.float16), np.nextafter(f16(g).astype(np.float16), inf)]
+        uc = [np.nextafter(f16(u).astype(np.float16), -inf), f16(u).astype(np.float16), np.nextafter(f16(u).astype(np.float16), inf)]
+        outs = [f16(O.swiglu_oai_np(a.astype(np.float32), b.astype(np.float32))) for a in gc for b in uc]
+        lo.append(np.min(outs, axis=0)); hi.append(np.max(outs, axis=0))
+    got16 = hp_h[rows].astype(np.float16)
+    inf = np.float16(np.inf)
+    ok = (got16 >= np.nextafter(np.stack(lo).astype(np.float16), -inf)) & (got16 <= np.nextafter(np.stack(hi).astype(np.float16), inf))
+    print("grouped mxfp4 gate/up (MFMA): %d / %d inside the one-ulp envelope of the chain" % (ok.sum(), ok.size), flush=True)
+    assert ok.mean() > 0.9995, ok.mean()
+    op = ops.moe_gemm_down_mxfp4(hp, dev(dq), dev(de), dqs_st, de_st, dev(bd), dev(off), TK, E, H, EF)
+    # out = half(half(acc) + bias): the sum can cancel, so the gate is the set of values the chain can produce when
+    # half(acc) moves by the accumulation-order noise and one fp16 ulp (as in test_gpu_moe), plus closeness in rms terms
+    from test_gpu_moe import f16_candidates, sum_noise, check_envelope
+    lo, hi, ctr = [], [], []
+    for r_, e_ in zip(rows, exp_of):
+        acc = O.gemv_f64(O.MXFP4, Wd[e_], hp_h[r_:r_ + 1], EF, H, round_w_fp16=True)[0].astype(np.float64)
+        c = [f16(v.astype(np.float32) + bd[e_]) for v in f16_candidates(acc, sum_noise(acc))]
+        lo.append(np.min(c, axis=0)); hi.append(np.max(c, axis=0)); ctr.append(c[1])
+    op_h = host(op).astype(np.float32)[rows]
+    check_envelope(op_h, np.stack(lo), np.stack(hi), "grouped mxfp4 down + bias (MFMA)")
+    check(op_h, np.stack(ctr), "  ... against the centre of the envelope", max_rel=1.0)
