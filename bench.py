@@ -369,6 +369,13 @@ def main():
                         ent["vendor_fp16_gemm_TFLOPs"] = round(2.0 * T * N * K / us_g / 1e6, 1)
                         ent["dequant_plus_vendor_gemm_us"] = round(us_2, 1)
                         del bt
+                    if T == 2048:
+                        # the int-dot route over q8 rows (int8 matrix cores, fp32 fold per 32-element block): rows quantized once, outside the timing
+                        aq8 = ops.quantize_q8_1s(a16)
+                        us_q = kernel_avg_us(lambda i: ops.gemm_q8_rows("q4_K", aq8, (wq,), T, K, N, yg), 4)
+                        ent["q8_rows_int8_mfma_us"] = round(us_q, 1)
+                        ent["q8_rows_frac_int8_mfma"] = round(2.0 * T * N * K / us_q / 1e6 / 5000.0, 4)
+                        del aq8
                     detail["config3_gemm_q4_K_T%d_K%d_N%d" % (T, K, N)] = ent
                     del a16, yg
                 del wq

@@ -409,6 +409,13 @@ int mx_moe_prefill_proj_q4_0_xmx(mx_stream_t s, const uint16_t* x_fp16, const vo
                                  uint16_t* out_packed, uint32_t E, uint32_t K, uint32_t N, uint64_t expert_stride_bytes,
                                  uint32_t total_rows);
 int mx_gemm_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+/* The dense int-dot GEMM for the other formats (no counterpart in the reference, whose gemm_q4_0_q8 exists for Q4_0
+ * only): y[M,N] = q8(x)[M,K] . W[N,K]^T over block_q8_1s rows [M, K/32] (mx_quantize_q8_1s), any M; int8 matrix cores,
+ * one instruction per 32-element block, fp32 fold per block (the q8 chain of mx_gemv_*_q8, row for row).  */
+int mx_gemm_q4_K_q8(mx_stream_t s, const void* xq8s_packed, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+int mx_gemm_q6_K_q8(mx_stream_t s, const void* xq8s_packed, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N);
+int mx_gemm_q8_0_soa_q8(mx_stream_t s, const void* xq8s_packed, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M,
+                        uint32_t K, uint32_t N);
 /* Accumulate form of the down projection (the reference's first prefill path), same matrix-core kernel
  * with an atomic fp32 epilogue:
  *   moe_prefill_down_q4k / _q6k       include/ie/ops.hpp:930-954, src/ops/moe_fused.cpp:937-1085

@@ -345,17 +345,29 @@ static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, co
     a.bank0 = b0; a.bank1 = b1; a.xq8 = m.xq8; a.expert_offsets = m.expert_offsets; a.out = m.out; a.bias0 = m.bias0; a.bias1 = m.bias1;
     a.route_w = m.route_w; a.alpha = m.alpha; a.limit = m.limit; a.M = 0; a.K = m.K; a.N = m.N; a.E = E; a.q8_split = m.q8_split;
     a.act_f16 = m.act_f16;
+    if (!m.expert_offsets) {   // one matrix, rows [0, n_rows): the token tiles are dealt over gridDim.z
+        a.M = m.n_rows;
+        a.deal_rows = 1;
+    }
     constexpr uint32_t TT = 2 * TV, gran = 256u * WK;
     constexpr uint32_t red = (uint32_t)(NW * WR * WK) * TV * 64u * 4u;
     const uint32_t per256 = TT * (NATIVE ? 512u : 256u) + 8u * TT * 4u * (P::HAS_MIN ? 2u : 1u);
-    const uint32_t budget = ((TV == 16 || (NATIVE && TV == 8)) ? kMmqMoeLdsBudgetBig : (NATIVE ? 64u * 1024u : kMmqMoeLdsBudget)) - red;
-    uint32_t kr = (budget - 32u * TT) / per256 * 256u / gran * gran;
-    if (!kr) kr = gran;
+    const uint32_t budget = (TV == 16 || (NATIVE && TV == 8)) ? kMmqMoeLdsBudgetBig : (NATIVE ? 64u * 1024u : kMmqMoeLdsBudget);
     const uint32_t need = ((m.K + 255u) / 256u + WK - 1u) / WK * WK * 256u;
-    if (kr > need) kr = need;
+    auto range = [&](uint32_t bytes) {
+        uint32_t k = (bytes - 32u * TT) / per256 * 256u / gran * gran;
+        if (!k) k = gran;
+        return k > need ? need : k;
+    };
+    // the exchange area sits behind the image when both fit the budget with the whole K range staged (the image then
+    // survives from row block to row block); otherwise it overlays the image, which is rebuilt for every row block
+    uint32_t kr = range(budget - red);
+    const bool overlay = kr < need;
+    if (overlay) kr = range(budget);
     a.kr = kr;
-    a.red_off = (mmq_lds_bytes(TT, kr, TV, P::HAS_MIN, NATIVE) + 15u) & ~15u;
-    const uint32_t lds = a.red_off + red;
+    const uint32_t image = (mmq_lds_bytes(TT, kr, TV, P::HAS_MIN, NATIVE) + 15u) & ~15u;
+    a.red_off = overlay ? 0u : image;
+    const uint32_t lds = overlay ? (image > red ? image : red) : image + red;
     const uint32_t rgs = (m.N + 32u * WR - 1u) / (32u * WR);
     if (E > 65535u) return MX_ERR_SHAPE;
     if (lds > 64u * 1024u) {
@@ -373,14 +385,17 @@ static int launch_mmq_grouped_cfg(hipStream_t st, const typename P::Bank& b0, co
     // token tiles of an expert are dealt over gridDim.z workgroups: the expert sizes live on the device and are skewed (a few
     // experts hold most rows), so the split is sized for experts several times the average; workgroups without a tile leave at once
     uint32_t zt = 2;   // even with small experts a few hold more rows than one tile: their second tile gets a workgroup of its own
-    if (avg == 0 || avg > TT) {
+    if (!m.expert_offsets) {
+        zt = (m.n_rows + TT - 1u) / TT;   // every tile its own workgroup, up to the 32 that share a row block's weights through L2
+        if (zt > 32u) zt = 32u;
+    } else if (avg == 0 || avg > TT) {
         zt = avg ? (4u * avg + TT - 1u) / TT : 8u;
         if (zt > 32u) zt = 32u;
     }
     // workgroups per expert along the weight rows: when the staged image covers K, about two resident workgroups per CU in
     // all, each streaming several row blocks against its one image; otherwise one workgroup per row block
     uint32_t gx = rgs;
-    if (kr >= need && avg && avg <= TT) {   // known, small experts only: with skewed or unknown sizes the row blocks stay spread
+    if (!overlay && avg && avg <= TT) {   // known, small experts only: with skewed or unknown sizes the row blocks stay spread
         const uint64_t slots = 2ull * (uint64_t)cu_count_moe();
         const uint32_t per = (uint32_t)(((uint64_t)rgs * E + slots - 1u) / slots);   // nearly every expert has one tile
         if (per > 1u) gx = (rgs + per - 1u) / per;
@@ -480,6 +495,18 @@ static int moe_grouped_kquant(mx_stream_t s, const void* act_q8, bool split, con
 
 using namespace mxq;
 
+// The same for K-quant and Q8_0 matrices (no counterpart in the reference, whose dense int-dot GEMM exists for Q4_0 only):
+// y[M, N] = q8(x)[M, K] . W[N, K]^T over block_q8_1s rows, int8 matrix cores with the fp32 fold per block.
+template <class P, class F>
+static int gemm_q8_rows(mx_stream_t s, const void* xq8s_packed, const typename F::Bank& b, uint16_t* y, uint32_t M, uint32_t K, uint32_t N, uint32_t k_align) {
+    if (int rc = check_moe(xq8s_packed, y, K, N, 1)) return rc;
+    MX_REQUIRE_SHAPE(M > 0 && K % k_align == 0);
+    MX_REQUIRE_ALIGN(xq8s_packed, 16);
+    MoeArgs a{};
+    a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.out = reinterpret_cast<half_t*>(y);
+    a.act_div = 1; a.K = K; a.N = N; a.n_experts = 1; a.q8_split = 1; a.n_rows = M;
+    return launch_mmq_grouped<P, 1, MMQ_STORE>(s, b, b, a, 1, M);
+}
 extern "C" {
 
 // ------------------------------------------------------------ Q8_0 SoA experts, decode
@@ -702,7 +729,7 @@ int mx_moe_prefill_proj_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const vo
     a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out_packed);
     a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = 1;
     FmtQ40Aos::Bank b{static_cast<const uint8_t*>(W_q4_0), expert_stride_bytes, K / 32 * 18u};
-    return launch_moe<FmtQ40Aos, 1, EPI_DOWN_BIAS>(s, b, b, a, E, grouped_tt(total_rows, E));
+    return launch_mmq_grouped<MmqQ40Aos, 1, MMQ_DOWN_BIAS>(s, b, b, a, E, avg_rows(total_rows, E));
 }
 int mx_moe_prefill_proj_q4_0_soa_q8(mx_stream_t s, const void* xq8s_packed, const uint8_t* qs_bank, const uint16_t* d_bank,
                                     const uint32_t* expert_offsets, uint16_t* out_packed, uint32_t E, uint32_t K, uint32_t N, uint64_t qs_stride,
@@ -715,7 +742,7 @@ int mx_moe_prefill_proj_q4_0_soa_q8(mx_stream_t s, const void* xq8s_packed, cons
     a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.expert_offsets = expert_offsets; a.out = reinterpret_cast<half_t*>(out_packed);
     a.act_div = 1; a.K = K; a.N = N; a.n_experts = E; a.q8_split = 1;
     FmtQ40Soa::Bank b{qs_bank, d_bank, qs_stride, d_stride, K};
-    return launch_moe<FmtQ40Soa, 1, EPI_DOWN_BIAS>(s, b, b, a, E, grouped_tt(total_rows, E));
+    return launch_mmq_grouped<MmqQ40Soa, 1, MMQ_DOWN_BIAS>(s, b, b, a, E, avg_rows(total_rows, E));
 }
 // gemm_q4_0_q8: y[M, N] = q8(x)[M, K] . W[N, K]^T for any M, int-dot: the rows run as token tiles of 8 over one matrix.
 int mx_gemm_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
@@ -727,7 +754,20 @@ int mx_gemm_q4_0_q8(mx_stream_t s, const void* xq8s_packed, const void* W_q4_0, 
     a.xq8 = static_cast<const uint8_t*>(xq8s_packed); a.out = reinterpret_cast<half_t*>(y);
     a.act_div = 1; a.K = K; a.N = N; a.n_experts = 1; a.q8_split = 1; a.n_rows = M;
     FmtQ40Aos::Bank b{static_cast<const uint8_t*>(W_q4_0), 0, K / 32 * 18u};
-    return launch_moe<FmtQ40Aos, 1, EPI_DOWN_BIAS>(s, b, b, a, 1, M == 1 ? 1u : (M <= 4 ? 4u : 8u));
+    if (M >= 5) return launch_mmq_grouped<MmqQ40Aos, 1, MMQ_DOWN_BIAS>(s, b, b, a, 1, M);   // batches on the matrix cores
+    return launch_moe<FmtQ40Aos, 1, EPI_DOWN_BIAS>(s, b, b, a, 1, M == 1 ? 1u : 4u);
+}
+int mx_gemm_q4_K_q8(mx_stream_t s, const void* xq8s_packed, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(W); MX_REQUIRE_ALIGN(W, 16);
+    return gemm_q8_rows<MmqQ4K, FmtQ4K>(s, xq8s_packed, FmtQ4K::Bank{static_cast<const uint8_t*>(W), 0, K / 256 * (uint32_t)kQ4KBytes}, y, M, K, N, 256);
+}
+int mx_gemm_q6_K_q8(mx_stream_t s, const void* xq8s_packed, const void* W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(W); MX_REQUIRE_ALIGN(W, 2);
+    return gemm_q8_rows<MmqQ6K, FmtQ6K>(s, xq8s_packed, FmtQ6K::Bank{static_cast<const uint8_t*>(W), 0, K / 256 * (uint32_t)kQ6KBytes}, y, M, K, N, 256);
+}
+int mx_gemm_q8_0_soa_q8(mx_stream_t s, const void* xq8s_packed, const int8_t* qs_W, const uint16_t* d_W, uint16_t* y, uint32_t M, uint32_t K, uint32_t N) {
+    MX_REQUIRE_PTR(qs_W); MX_REQUIRE_PTR(d_W); MX_REQUIRE_ALIGN(qs_W, 16);
+    return gemm_q8_rows<MmqQ8Soa, FmtQ8Soa>(s, xq8s_packed, FmtQ8Soa::Bank{qs_W, d_W, 0, 0, K}, y, M, K, N, 32);
 }
 
 // ------------------------------------------------------------ row utilities

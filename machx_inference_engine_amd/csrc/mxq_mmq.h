@@ -324,6 +324,107 @@ struct MmqQ4K {
     }
 };
 
+// Q4_0 (32-element blocks: fp16 d, 16 bytes with element j in the low and j + 16 in the high nibble of byte j;
+// include/ie/quant_blocks.hpp:32-43): value = d (q - 8), so the codes stay unsigned and the -8 d folds on the stored
+// block sum of the activation row, like Q4_K's min term.  Lane half h takes the low (h = 0) or high nibbles of all 16
+// bytes, so both halves load the block's bytes.  Planes: qs[N][K/2], d[N][K/32]; GGUF blocks: 18 bytes, 2-byte aligned.
+struct MmqQ40Soa {
+    using W = FmtQ40Soa::W;
+    using Bank = FmtQ40Soa::Bank;
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return FmtQ40Soa::expert(b, e); }
+    static constexpr int SUBS = 1;
+    static constexpr bool HAS_MIN = true;
+    static constexpr uint32_t K_ALIGN = 32;
+    struct Raw {
+        uint4 q[8];
+        uint32_t d[4];   // 8 fp16 block scales
+    };
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t g, uint32_t, uint32_t nb) {
+        const uint8_t* p = w.qs + (size_t)n * (w.K >> 1) + (size_t)g * 128u;
+        Raw r;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) r.q[s] = *reinterpret_cast<const uint4*>(p + s * 16);
+        const uint4 dd = load_u4_a2(reinterpret_cast<const uint8_t*>(w.d + (size_t)n * nb) + 16u * g);
+        r.d[0] = dd.x; r.d[1] = dd.y; r.d[2] = dd.z; r.d[3] = dd.w;
+        return r;
+    }
+    __device__ static __forceinline__ Raw load_tail(const W& w, uint32_t n, uint32_t g, uint32_t, uint32_t nb) {
+        const uint8_t* p = w.qs + (size_t)n * (w.K >> 1);
+        const uint16_t* d = w.d + (size_t)n * nb;
+        Raw r;
+        uint32_t ds[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint32_t b = 8u * g + s, bc = b < nb ? b : nb - 1u;
+            r.q[s] = *reinterpret_cast<const uint4*>(p + (size_t)bc * 16u);
+            ds[s] = b < nb ? (uint32_t)d[bc] : 0u;   // fp16 +0: the block contributes nothing (its activation sum is zero as well)
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) r.d[s] = ds[2 * s] | (ds[2 * s + 1] << 16);
+        return r;
+    }
+    template <int S>
+    __device__ static __forceinline__ v4i_t operand(const Raw& r, uint32_t h) {
+        const uint32_t sh = 4u * h;
+        v4i_t o;
+        o.x = (int)((r.q[S].x >> sh) & 0x0F0F0F0Fu); o.y = (int)((r.q[S].y >> sh) & 0x0F0F0F0Fu);
+        o.z = (int)((r.q[S].z >> sh) & 0x0F0F0F0Fu); o.w = (int)((r.q[S].w >> sh) & 0x0F0F0F0Fu);
+        return o;
+    }
+    struct Dec {
+        float c[8], m[8];
+    };
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t) {
+        Dec o;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            o.c[s] = h2f((s & 1) ? r.d[s >> 1] >> 16 : r.d[s >> 1] & 0xFFFFu);
+            o.m[s] = 8.f * o.c[s];
+        }
+        return o;
+    }
+};
+struct MmqQ40Aos {
+    using W = FmtQ40Aos::W;
+    using Bank = FmtQ40Aos::Bank;
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return FmtQ40Aos::expert(b, e); }
+    static constexpr int SUBS = 1;
+    static constexpr bool HAS_MIN = true;
+    static constexpr uint32_t K_ALIGN = 32;
+    using Raw = MmqQ40Soa::Raw;
+    using Dec = MmqQ40Soa::Dec;
+    __device__ static __forceinline__ Raw load(const W& w, uint32_t n, uint32_t g, uint32_t, uint32_t) {
+        const uint8_t* p = w.base + (size_t)n * w.row_bytes + (size_t)g * (8u * 18u);
+        Raw r;
+        uint32_t ds[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            r.q[s] = load_u4_a2(p + 18 * s + 2);
+            ds[s] = *reinterpret_cast<const uint16_t*>(p + 18 * s);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) r.d[s] = ds[2 * s] | (ds[2 * s + 1] << 16);
+        return r;
+    }
+    __device__ static __forceinline__ Raw load_tail(const W& w, uint32_t n, uint32_t g, uint32_t, uint32_t nb) {
+        const uint8_t* p = w.base + (size_t)n * w.row_bytes;
+        Raw r;
+        uint32_t ds[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint32_t b = 8u * g + s, bc = b < nb ? b : nb - 1u;
+            r.q[s] = load_u4_a2(p + (size_t)bc * 18u + 2);
+            ds[s] = b < nb ? (uint32_t)*reinterpret_cast<const uint16_t*>(p + (size_t)bc * 18u) : 0u;
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) r.d[s] = ds[2 * s] | (ds[2 * s + 1] << 16);
+        return r;
+    }
+    template <int S>
+    __device__ static __forceinline__ v4i_t operand(const Raw& r, uint32_t h) { return MmqQ40Soa::operand<S>(r, h); }
+    __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t h) { return MmqQ40Soa::prepare(r, h); }
+};
+
 // Q6_K AoS blocks (210 B, 2-byte aligned): element 128 hf + 32 sub + l has its low nibble in nibble (sub >> 1) of
 // ql[64 hf + 32 (sub & 1) + l] and its two high bits at 2 sub of qh[32 hf + l]; scale scales[8 hf + 2 sub + l / 16]
 // (include/ie/dequant_ref.hpp:78-96).  Lane half h owns l = 16 h .. +15, which is exactly the 16-element scale
@@ -797,7 +898,8 @@ struct MmqArgs {
     uint32_t M, K, N, E;
     uint32_t q8_split;
     uint32_t kr;                      // staged k range per pass (multiple of 256 WK)
-    uint32_t red_off;                 // byte offset of the partial-sum exchange area in LDS (behind the staged image)
+    uint32_t red_off;                 // byte offset of the partial-sum exchange area in LDS: behind the staged image, or 0 = over it
+    uint32_t deal_rows;               // one matrix with many rows [0, M): gridDim.z deals the token tiles (no K ranges, no `part`)
 };
 
 __device__ __forceinline__ float mmq_silu_mul(float g, float u) { return (g / (1.f + __expf(-g))) * u; }
@@ -833,13 +935,13 @@ __global__ __launch_bounds__(64 * NW * WR * WK, 2) void mmq_kernel(MmqArgs<P> a)
     const uint32_t n_rb = (a.N + 32u * WR - 1u) / (32u * WR);
     // gridDim.z: dense launches split K into ranges (partial sums to `part`); grouped launches deal the token tiles of an
     // expert round-robin, so that an expert with many rows is spread over many workgroups
-    const bool grouped = a.expert_offsets != nullptr;
+    const bool grouped = a.expert_offsets != nullptr || a.deal_rows != 0;
     const uint32_t kz = grouped ? 1u : gridDim.z, kzi = grouped ? 0u : blockIdx.z;
     const uint32_t gz = (n_groups + kz - 1u) / kz;
     const uint32_t G0 = kzi * gz, G1 = G0 + gz < n_groups ? G0 + gz : n_groups;
     const uint32_t t_step = grouped ? gridDim.z * 2u * TV : 2u * TV, t_first = grouped ? blockIdx.z * 2u * TV : 0u;
     const uint32_t gp = a.kr / 256u;                     // groups per pass (multiple of WK)
-    const bool single = G1 - G0 <= gp;                   // one image covers the K range
+    const bool single = G1 - G0 <= gp && a.red_off != 0; // one image covers the K range and is not overlaid by the exchange area
     const size_t q8_row_bytes = (size_t)nb * (a.q8_split ? kQ81sBytes : kQ81xBytes);
     float* red = reinterpret_cast<float*>(lds + a.red_off);
 

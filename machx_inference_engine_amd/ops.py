@@ -777,3 +777,10 @@ def moe_gemm_down_q8(h_packed, d_qs, d_d, qs_stride, d_stride, expert_offsets, s
     _call("mx_moe_gemm_down_q8", _f16(h_packed), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(expert_offsets), _f16(sorted_w),
           _ptr(out_packed), E, H, E_ffn, TK)
     return out_packed
+
+
+def gemm_q8_rows(fmt, xq8s, wargs, M, K, N, y=None):
+    """Dense int-dot GEMM over block_q8_1s rows: fmt in ('q4_K', 'q6_K', 'q8_0_soa'); wargs = weight tensors in C-ABI order."""
+    y = _out(y, (M, N), torch.float16, xq8s)
+    _call("mx_gemm_%s_q8" % fmt, _u8(xq8s), *[_ptr(w) for w in wargs], _ptr(y), M, K, N)
+    return y

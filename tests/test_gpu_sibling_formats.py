@@ -127,7 +127,7 @@ def test_moe_prefill_proj_q4_0(mx, T, E, Kt, K, N):
         check(host(got_x).astype(np.float32).ravel(), ref_x.ravel(), "moe_prefill_proj_q4_0_xmx")
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 64, 8), (5, 736, 130), (37, 2048, 300)])
+@pytest.mark.parametrize("M,K,N", [(1, 64, 8), (5, 736, 130), (37, 2048, 300), (300, 1056, 200)])
 def test_gemm_q4_0_q8(mx, M, K, N):
     """gemm_q4_0_q8 (include/ie/ops.hpp:538-548): int-dot GEMM over block_q8_1s rows, any M, any K % 32 == 0."""
     W = weights(O.Q4_0, 6600 + M, N, K)
@@ -136,3 +136,22 @@ def test_gemm_q4_0_q8(mx, M, K, N):
     y = mx.ops.gemm_q4_0_q8(xq_s, dev(W), M, K, N)
     ref = O.gemv_q8chain(O.Q4_0, W, O.quantize_q8_1(x), K, N)
     check(host(y).astype(np.float32).ravel(), ref.ravel(), "gemm_q4_0_q8 M=%d" % M)
+
+
+@pytest.mark.parametrize("M,K,N", [(7, 512, 96), (70, 1024, 260), (600, 2048, 512)])
+def test_gemm_q8_rows_dense(mx, M, K, N):
+    """Dense int-dot GEMM over block_q8_1s rows for Q4_K / Q6_K / Q8_0 planes (int8 matrix cores, token tiles dealt over
+    workgroups): every row against the q8 chain with the stored half sums (the arithmetic of mx_gemv_*_q8s)."""
+    x = acts(6700 + M, M, K)
+    xq_s = mx.ops.quantize_q8_1s(dev(x).half())
+    xq_h = host(xq_s)
+    for fmt, F in (("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
+        W = weights(F, 6701 + N, N, K)
+        y = mx.ops.gemm_q8_rows(fmt, xq_s, (dev(W),), M, K, N)
+        ref = O.gemv_q8schain(F, W, xq_h, K, N)
+        check(host(y).astype(np.float32).ravel(), ref.ravel(), "gemm_%s_q8 M=%d" % (fmt, M))
+    W = weights(O.Q8_0, 6702 + N, N, K)
+    qs, d = O.repack_q8_0_to_soa(W)
+    y = mx.ops.gemm_q8_rows("q8_0_soa", xq_s, (dev(qs), dev(d)), M, K, N)
+    ref = O.gemv_q8chain(O.Q8_0, W, O.quantize_q8_1(x), K, N)
+    check(host(y).astype(np.float32).ravel(), ref.ravel(), "gemm_q8_0_soa_q8 M=%d" % M)
