@@ -234,7 +234,7 @@ def main():
         # the fused gate + up launch: two 4096 -> 14336 matrices, one activation row, two output rows
         dom_us = kernel_avg_us(lambda i: gate_up("q8_0", sets[i % len(sets)]), 4 * len(sets))
         dom_bytes = 2 * gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1) - (H // 32) * 40
-        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 124885402 + 233882
+        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 125019703 + 230809
     # yardstick: a pure read of the same number of bytes with the same launch geometry (rotating buffers, no arithmetic)
     n_read = (dom_bytes + 15) // 16 * 16
     rd = [torch.empty(n_read, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(8)]
@@ -263,7 +263,7 @@ def main():
                      "flop_per_launch": gemm_flop, "avg_launch_us": round(gemm_us, 2),
                      # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt);
                      # algorithmic bytes: W 33,030,144 + A 16,777,216 + Y 58,720,256
-                     "traffic": 254400000 + 58900000, "algorithmic_bytes": Ng * synth.row_bytes("q4_K", Kg) + Tg * Kg * 2 + Tg * Ng * 2}
+                     "traffic": 254396345 + 58720358, "algorithmic_bytes": Ng * synth.row_bytes("q4_K", Kg) + Tg * Kg * 2 + Tg * Ng * 2}
     del wq, a16, yg
 
     out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
