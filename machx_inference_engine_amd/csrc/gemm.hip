@@ -804,7 +804,9 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
     mma_chunk<QF, PARTIAL, NA>(raw[P], dec, t.lds_raw, (c & 1u) * ABUF + t.frag0, acc, t.mi);
     if (more) {
         wait_vmcnt<(DEPTH > 1 ? W_LOADS_MIN : 0)>();   // A rows of chunk c+1 are in LDS (DEPTH > 1: the newest weight loads stay in flight)
-        __syncthreads();
+        // A barrier that waits for the LDS traffic only: __syncthreads() carries a fence that waits for every
+        // outstanding load, the weight words requested for later chunks included.
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 }
 
