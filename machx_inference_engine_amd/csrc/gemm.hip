@@ -694,46 +694,52 @@ __device__ __forceinline__ void mma_step(const typename QF::Raw (&raw)[2], const
         }
 }
 
-// Full tiles: the chunk as one software pipeline.  A step is cut into four segments, one per
-// token tile: its 2 MFMAs, the LDS read that refills that A fragment for step S+1 (first use
-// 6 MFMAs later), and a quarter of the dequantisation of the weight fragments of step S+1 into
-// the other fragment pair.  The scheduling fences between segments keep that interleaving, so
-// neither the VALU work nor the LDS latency ends up between two clusters of MFMAs.
-template <int S, class QF>
+// The chunk as one software pipeline over NI token tiles, all of them multiplied (no branch inside a chunk: a branch
+// per token tile ends the scheduling region, and each step then runs as LDS read, wait, dequantisation, MFMAs one after
+// the other).  A step is cut into NI segments, one per token tile: its 2 MFMAs, the LDS read that refills that A
+// fragment for step S+1, and 4 / NI of the four half-fragment dequantisations of the weight fragments of step S+1
+// into the other fragment pair.  The scheduling fences between segments keep that interleaving, so neither the VALU
+// work nor the LDS latency ends up between two clusters of MFMAs.
+template <int S, class QF, int NI>
 __device__ __forceinline__ void mma_pipe(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
-                                         float16_t (&acc)[4][2], Frag (&af)[4], Frag (&bf)[2][2]) {
+                                         float16_t (&acc)[NI][2], Frag (&af)[NI], Frag (&bf)[2][2]) {
+    static_assert(NI == 1 || NI == 2 || NI == 4, "token tiles per pipelined chunk");
     if constexpr (S < 8) {
         constexpr int cur = S & 1, nxt = cur ^ 1, SN = (S + 1) & 7;
         constexpr bool more = S + 1 < 8;
+        constexpr int per = 4 / NI;   // half fragments dequantized per segment
         const uint32_t a_n = a_frag0 ^ (QF::step_col(SN) << 4);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NI; ++i) {
             acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[cur][0].v, acc[i][0], 0, 0, 0);
             acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i].v, bf[cur][1].v, acc[i][1], 0, 0, 0);
             if (more) {
                 af[i].q = *reinterpret_cast<const uint4*>(lds + a_n + i * 8192);
-                if (i == 0) QF::template frag_half<SN, 0>(raw[0], dec[0], bf[nxt][0]);
-                if (i == 1) QF::template frag_half<SN, 1>(raw[0], dec[0], bf[nxt][0]);
-                if (i == 2) QF::template frag_half<SN, 0>(raw[1], dec[1], bf[nxt][1]);
-                if (i == 3) QF::template frag_half<SN, 1>(raw[1], dec[1], bf[nxt][1]);
+#pragma unroll
+                for (int q = i * per; q < (i + 1) * per; ++q) {
+                    if (q == 0) QF::template frag_half<SN, 0>(raw[0], dec[0], bf[nxt][0]);
+                    if (q == 1) QF::template frag_half<SN, 1>(raw[0], dec[0], bf[nxt][0]);
+                    if (q == 2) QF::template frag_half<SN, 0>(raw[1], dec[1], bf[nxt][1]);
+                    if (q == 3) QF::template frag_half<SN, 1>(raw[1], dec[1], bf[nxt][1]);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        mma_pipe<S + 1, QF>(raw, dec, lds, a_frag0, acc, af, bf);
+        mma_pipe<S + 1, QF, NI>(raw, dec, lds, a_frag0, acc, af, bf);
     }
 }
 
-template <class QF, bool PARTIAL, int NI>
+template <class QF, bool PIPE, bool PARTIAL, int NI>
 __device__ __forceinline__ void mma_chunk(const typename QF::Raw (&raw)[2], const typename QF::Dec (&dec)[2], const uint8_t* lds, uint32_t a_frag0,
                                           float16_t (&acc)[NI][2], uint32_t mi) {
-    if constexpr (!PARTIAL && NI == 4) {
-        Frag af[4], bf[2][2];
+    if constexpr (PIPE) {
+        Frag af[NI], bf[2][2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[i].q = *reinterpret_cast<const uint4*>(lds + a_frag0 + i * 8192);
+        for (int i = 0; i < NI; ++i) af[i].q = *reinterpret_cast<const uint4*>(lds + a_frag0 + i * 8192);
         QF::template frag<0>(raw[0], dec[0], bf[0][0]);
         QF::template frag<0>(raw[1], dec[1], bf[0][1]);
         __builtin_amdgcn_sched_barrier(0);   // prologue stays ahead of the pipelined steps
-        mma_pipe<0, QF>(raw, dec, lds, a_frag0, acc, af, bf);
+        mma_pipe<0, QF, NI>(raw, dec, lds, a_frag0, acc, af, bf);
     } else {
         mma_step<0, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
         mma_step<1, QF, PARTIAL, NI>(raw, dec, lds, a_frag0, acc, mi);
@@ -785,7 +791,7 @@ __device__ __forceinline__ void a_rows_to_lds(const TileCtx<QF, NA>& t, const ui
 }
 
 // Chunk c out of register set P; meanwhile (`more`) the A rows of chunk c+1 and the weights of chunk c+DEPTH are requested.
-template <class QF, bool PARTIAL, int NA, int DEPTH, int P>
+template <class QF, bool PIPE, bool PARTIAL, int NA, int DEPTH, int P>
 __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint32_t (&a_off)[2 * NA], typename QF::Raw (&raw)[DEPTH + 1][2],
                                            float16_t (&acc)[NA][2], uint32_t c, bool more) {
     constexpr int NSET = DEPTH + 1, PN = (P + DEPTH) % NSET;
@@ -801,7 +807,7 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
     typename QF::Dec dec[2];
     dec[0] = QF::prepare(raw[P][0], t.c0 + c, t.h);
     dec[1] = QF::prepare(raw[P][1], t.c0 + c, t.h);
-    mma_chunk<QF, PARTIAL, NA>(raw[P], dec, t.lds_raw, (c & 1u) * ABUF + t.frag0, acc, t.mi);
+    mma_chunk<QF, PIPE, PARTIAL, NA>(raw[P], dec, t.lds_raw, (c & 1u) * ABUF + t.frag0, acc, t.mi);
     if (more) {
         wait_vmcnt<(DEPTH > 1 ? W_LOADS_MIN : 0)>();   // A rows of chunk c+1 are in LDS (DEPTH > 1: the newest weight loads stay in flight)
         // A barrier that waits for the LDS traffic only: __syncthreads() carries a fence that waits for every
@@ -828,7 +834,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
                                           uint32_t row_lo, uint32_t row_hi, uint32_t n_base, uint8_t* lds_raw, uint32_t c0 = 0,
                                           uint32_t n_chunks_slice = 0, uint32_t ks = 0, uint32_t e = 0) {
     static_assert(DEPTH == 1 || DEPTH == 2, "prefetch depth");
-    static_assert(!PIPE || NA == 4, "the pipelined chunk is written for four token tiles");
+    static_assert(!PIPE || NA == 1 || NA == 2 || NA == 4, "the pipelined chunk is written for one, two or four token tiles");
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI;
     constexpr bool PARTIAL = MODE != GEMM_DENSE && !PIPE;
     constexpr uint32_t BM = 32u * NA;
@@ -882,7 +888,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
         raw[d][1] = QF::load(w1, wrow[1], c0 + cd, h);
     }
 
-#define CHUNK(P, c, more) gemm_chunk<QF, PARTIAL, NA, DEPTH, P>(ctx, a_off, raw, acc, c, more)
+#define CHUNK(P, c, more) gemm_chunk<QF, PIPE, PARTIAL, NA, DEPTH, P>(ctx, a_off, raw, acc, c, more)
     if constexpr (DEPTH == 1) {
         // two sets, and the set just loaded is copied into set 0 at the end of a chunk, where it has to have arrived anyway
         for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
@@ -972,20 +978,21 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     uint32_t e = 0, row_lo = 0, row_hi = g.M;
     if (MODE != GEMM_DENSE) {
         // Tile order over all experts: every full BM-row tile first (expert by expert), then the experts' partial last
-        // tiles.  Full tiles cost the most, so the workgroups dispatched last are the cheap ones and the launch ends
-        // without a few full tiles running alone.  Wave 0 scans the per-expert counts, 64 experts at a time; pass 0
-        // walks the full tiles, pass 1 the partial ones.
+        // tiles, those with the most live 32-row sub-tiles first.  A tile's cost grows with its live sub-tiles, so the
+        // workgroups dispatched last are the cheapest ones and the launch does not end with a few expensive tiles
+        // running alone (list scheduling, longest first).  Wave 0 scans the per-expert counts, 64 experts at a time:
+        // pass 0 walks the full tiles, pass k the partial tiles with NI + 1 - k live sub-tiles.
         __shared__ uint32_t s_tile[3];
         const uint32_t ln = threadIdx.x & 63u;
         if (threadIdx.x < 64) {
             uint32_t base = 0;
             bool found = false;
-            for (uint32_t pass = 0; pass < 2 && !found; ++pass)
+            for (uint32_t pass = 0; pass <= (uint32_t)NI && !found; ++pass)
                 for (uint32_t e0 = 0; e0 < g.E && !found; e0 += 64) {
                     const uint32_t ee = e0 + ln;
                     const uint32_t lo = ee < g.E ? g.expert_offsets[ee] : 0u, hi = ee < g.E ? g.expert_offsets[ee + 1] : 0u;
-                    const uint32_t full = (hi - lo) / BM;
-                    const uint32_t nt = pass == 0 ? full : ((hi - lo) % BM ? 1u : 0u);
+                    const uint32_t full = (hi - lo) / BM, rem = (hi - lo) % BM;
+                    const uint32_t nt = pass == 0 ? full : ((rem && (rem + 31u) / 32u == (uint32_t)NI + 1u - pass) ? 1u : 0u);
                     uint32_t incl = nt;
 #pragma unroll
                     for (int d = 1; d < 64; d <<= 1) {
@@ -1030,12 +1037,14 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
         gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, c0, c1 - c0, ks);
     } else {
         (void)ks;
-        // expert-grouped tiles: a full one takes the same pipelined chunk as the dense GEMM; one with at most 64
-        // live rows keeps half the accumulators and spends the registers on a second chunk of weights in flight
+        // expert-grouped tiles: the pipelined chunk over as many 32-token tiles as the tile's live rows need (one, two,
+        // or four; the token tiles past the live rows are multiplied too, on copies of the last live row, and dropped
+        // by the epilogue).  A tile with at most 64 live rows keeps half (a quarter) of the accumulators and spends
+        // the registers on a second chunk of weights in flight.
         const uint32_t live = row_hi - row_lo;
-        if (live >= BM) gemm_tile<QF, MODE, true, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
-        else if (live <= 64u) gemm_tile<QF, MODE, false, 2, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
-        else gemm_tile<QF, MODE, false, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
+        if (live > 64u) gemm_tile<QF, MODE, true, 4, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
+        else if (live > 32u) gemm_tile<QF, MODE, true, 2, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
+        else gemm_tile<QF, MODE, true, 1, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, 0, 0, 0, e);
     }
 }
 
