@@ -759,7 +759,8 @@ struct FmtMxfp4Soa {
             r.e2 = e[0];
         } else {
             r.qb = p[1];
-            r.e2 = (uint32_t)e[0] | ((uint32_t)e[1] << 8);
+            struct __attribute__((packed, aligned(1))) E2 { uint16_t v; };   // one request for both exponents (any byte address)
+            r.e2 = reinterpret_cast<const E2*>(e)->v;
         }
         return r;
     }
