@@ -29,9 +29,12 @@ constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is
 
 // Persistent workgroups: each stages the activation tile(s) and then streams
 // its share of row groups.  With a single K-tile (every decode shape at T <= 2)
-// the activation is staged once per workgroup.
+// the activation is staged once per workgroup.  The single-token instances are compiled
+// for the four workgroups per CU they are launched with (128 registers): left alone the
+// compiler takes a few more for some formats and a workgroup per CU is lost (Q6_K planes,
+// 4096 -> 14336: 15.5 -> 13.5 us with three registers spilled; no other format changes).
 template <class F, int T, int R, int G, int U, class OutT>
-__global__ __launch_bounds__(kGemvThreads) void gemv_q8_kernel(GemvSeg<F, OutT> seg0, GemvSeg<F, OutT> seg1, const uint8_t* xq8,
+__global__ __launch_bounds__(kGemvThreads, (T == 1 ? 4 : 1)) void gemv_q8_kernel(GemvSeg<F, OutT> seg0, GemvSeg<F, OutT> seg1, const uint8_t* xq8,
                                                                 uint32_t K, uint32_t N, uint32_t KT, uint32_t T_real, uint32_t q8_split) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int GROUPS = 64 / G;
