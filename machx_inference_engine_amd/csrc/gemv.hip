@@ -733,7 +733,11 @@ static int launch_q8(mx_stream_t s, GemvSeg<F, OutT> s0, GemvSeg<F, OutT> s1, in
         // T = 8: 20.4 vs 17.6; Q6_K T = 8: 26.2 vs 22.0; batches of 9 .. 16 take one pass here instead of two there
         // (GGUF Q8_0 blocks: the 2-byte aligned block walk loses below a full second pass, 24.4 vs 30.9 us at T = 8)
         constexpr uint32_t kMmqFromT = std::is_same<F, FmtQ8Aos>::value ? 9u : 5u;
-        if (T >= kMmqFromT && nseg == 1 && !s0.bias) return launch_mmq_dense<P>(as_stream(s), mmq_bank(s0.w), x, s0.y, K, N, T, split, ws);
+        // long rows (14336 -> 4096): batches of four cross over one row earlier for Q8_0 planes (19.6 vs 18.9 us) and Q6_K
+        // (24.1 vs 22.7 us); Q4_K does not (15.4 vs 15.5 us)
+        constexpr bool kEarlier = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ6K>::value;
+        const uint32_t from = (kEarlier && K >= 8192u) ? kMmqFromT - 1u : kMmqFromT;
+        if (T >= from && nseg == 1 && !s0.bias) return launch_mmq_dense<P>(as_stream(s), mmq_bank(s0.w), x, s0.y, K, N, T, split, ws);
     }
     for (uint32_t t0 = 0; t0 < T; t0 += 8) {
         const uint32_t tn = (T - t0 < 8) ? T - t0 : 8;
