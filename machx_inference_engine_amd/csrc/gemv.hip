@@ -543,6 +543,32 @@ static int cu_count() {
 }
 
 constexpr uint32_t kLdsBudget = 48 * 1024;
+// Workgroups of `kernel` that fit one CU at once (registers and `lds` bytes of dynamic LDS), asked once per kernel.
+// Persistent grids are sized with it: a workgroup that does not fit next to the others would run alone after them.
+static uint32_t resident_wgs(const void* kernel, uint32_t lds) {
+    constexpr int kSlots = 512;   // a fixed table (nothing is allocated): kernels beyond it are asked about every time
+    static std::atomic<const void*> key[kSlots];
+    static std::atomic<uint32_t> val[kSlots];
+    for (int i = 0; i < kSlots; ++i) {
+        const void* k = key[i].load(std::memory_order_acquire);
+        if (k == kernel) {
+            const uint32_t v = val[i].load(std::memory_order_acquire);
+            if (v) return v;
+            break;   // another thread is filling the slot: ask as well
+        }
+        if (!k) break;
+    }
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, (int)kGemvThreads, lds) != hipSuccess || n < 1) n = 1;
+    for (int i = 0; i < kSlots; ++i) {
+        const void* expected = nullptr;
+        if (key[i].compare_exchange_strong(expected, kernel, std::memory_order_acq_rel) || expected == kernel) {
+            val[i].store((uint32_t)n, std::memory_order_release);
+            break;
+        }
+    }
+    return (uint32_t)n;
+}
 constexpr int kRows = 2;             // rows per lane group, float-activation kernels
 constexpr uint32_t kWgsPerCu = 4;    // persistent grid: workgroups per CU
 // rows per lane group / unroll of the unit walk: one row and two units in flight for a single
@@ -619,9 +645,14 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     // launch is balanced per CU, not per workgroup: with a whole number of workgroups per CU
     // the dispatcher gives every CU the same number of them, and the strided row-group loop
     // hands each CU the same number of row groups to within one per workgroup.
-    const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu / nseg;
-    dim3 grid(n_rg < cap ? n_rg : cap, nseg);
+    // The persistent grid holds as many workgroups per CU as are resident at once, at most kWgsPerCu: the batched
+    // instances of some formats need more than 128 registers (Q6_K with three or four rows: 148 - 151), so only three
+    // fit, and a fourth per CU would run alone after the others.
     const uint32_t lds = act_tile_bytes(T, KT, F::SUM_GRAN);
+    uint32_t per_cu = resident_wgs(reinterpret_cast<const void*>(&gemv_q8_kernel<F, T, R, G, U, OutT>), lds);
+    if (per_cu > kWgsPerCu) per_cu = kWgsPerCu;
+    const uint32_t cap = (uint32_t)cu_count() * per_cu / nseg;
+    dim3 grid(n_rg < cap ? n_rg : (cap ? cap : 1u), nseg);
     hipLaunchKernelGGL((gemv_q8_kernel<F, T, R, G, U, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real, split ? 1u : 0u);
     return launch_status();
 }
@@ -794,7 +825,13 @@ static int launch_fact(mx_stream_t s, const typename F::W& w, const ActT* A, Out
     const uint32_t G = pick_group((K + 63) / 64);
     const uint32_t rows_per_wg = kGemvWaves * (64 / G) * (PAIR ? 1 : kRows);
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
-    const uint32_t cap = (uint32_t)cu_count() * kWgsPerCu / nseg;   // persistent and CU-balanced, as the int-dot launch
+    const void* kernel = G == 16   ? reinterpret_cast<const void*>(&gemv_fact_kernel<F, kRows, 16, ActT, OutT, EPI>)
+                         : G == 32 ? reinterpret_cast<const void*>(&gemv_fact_kernel<F, kRows, 32, ActT, OutT, EPI>)
+                                   : reinterpret_cast<const void*>(&gemv_fact_kernel<F, kRows, 64, ActT, OutT, EPI>);
+    uint32_t per_cu = resident_wgs(kernel, lds);   // these kernels take 177 - 211 registers: two workgroups per CU
+    if (per_cu > kWgsPerCu) per_cu = kWgsPerCu;
+    uint32_t cap = (uint32_t)cu_count() * per_cu / nseg;   // persistent and CU-balanced, as the int-dot launch
+    if (!cap) cap = 1;
     dim3 grid((n_rg < cap ? n_rg : cap) + (EPI == FACT_SILU_PAIR ? 1 : 0), nseg);
     if (G == 16)
         hipLaunchKernelGGL((gemv_fact_kernel<F, kRows, 16, ActT, OutT, EPI>), grid, dim3(kGemvThreads), lds, as_stream(s), w, w1, A, y, y_b, accum_scale, tail, K, N, KT);
