@@ -301,7 +301,7 @@ static uint32_t pick_group_moe(uint32_t units) {
 
 template <class F, int TT, int NW, int G, int EPI>
 static int launch_moe_tg(hipStream_t st, const typename F::Bank& b0, const typename F::Bank& b1, MoeArgs a, uint32_t n_seg) {
-    constexpr int R = (NW == 2) ? 1 : 2;
+    constexpr int R = (NW == 2 || TT == 1) ? 1 : 2;
     constexpr int U = (TT == 1) ? 2 : 1;
     constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
     const uint32_t per32 = 32 + hdr_bytes_per32(F::SUM_GRAN);
