@@ -395,3 +395,60 @@ def test_moe_grouped_gemm_mxfp4(mx, T, E, Kt, H, EF):
     op_h = host(op).astype(np.float32)[rows]
     check_envelope(op_h, np.stack(lo), np.stack(hi), "grouped mxfp4 down + bias (MFMA)")
     check(op_h, np.stack(ctr), "  ... against the centre of the envelope", max_rel=1.0)
+
+
+def test_moe_grouped_gemm_q8_random_shapes(mx):
+    """Random expert counts (empty experts, a few rows, several tiles) against random depths and widths, including the
+    depths whose scale rows end in a half piece of the LDS scale table (K = 128, 384, 640).  Floating-point kernel: the
+    reference is the same product in fp32 on the dequantized (fp16-rounded) weights; relative error against
+    |ref| + 2 % of mean |ref| (an output that cancels to nothing carries the fp16 rounding of its terms)."""
+    from machx_inference_engine_amd import synth
+    ops = mx.ops
+    d0 = "cuda:0"
+    rng = np.random.default_rng(123)
+
+    def deq(blocks, N, K):
+        b = blocks.reshape(N, K // 32, 34)
+        d = b[:, :, 0:2].contiguous().view(torch.float16).float()
+        q = b[:, :, 2:].contiguous().view(torch.int8).float()
+        return (d * q).half().float().reshape(N, K)
+
+    worst = 0.0
+    for it in range(12):
+        E = int(rng.integers(1, 24))
+        H = int(rng.choice([128, 256, 384, 512, 640, 1024, 2048]))
+        EF = int(rng.choice([128, 256, 384, 768]))
+        counts = rng.integers(0, 140, size=E)
+        counts[rng.integers(0, E)] += int(rng.integers(0, 300))
+        if counts.sum() == 0:
+            counts[0] = 5
+        off = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+        TK = int(off[-1])
+        g = torch.Generator(device=d0)
+        g.manual_seed(it)
+        Wg = synth.random_weights("q8_0", E * EF, H, seed=10 + it, device=d0)
+        Wu = synth.random_weights("q8_0", E * EF, H, seed=500 + it, device=d0)
+        Wd = synth.random_weights("q8_0", E * H, EF, seed=900 + it, device=d0)
+        gq, gd = synth.split_q8_0(Wg)
+        uq, ud = synth.split_q8_0(Wu)
+        dq, dd = synth.split_q8_0(Wd)
+        x = (torch.randn((TK, H), device=d0, generator=g) * 0.5).half()
+        wp = torch.rand((TK,), device=d0, generator=g).half()
+        offd = torch.from_numpy(off).to(d0)
+        hp = ops.moe_gemm_gate_up_silu_q8(x, gq, gd, uq, ud, EF * H, EF * H // 32, offd, TK, E, H, EF)
+        op = ops.moe_gemm_down_q8(hp, dq, dd, H * EF, H * EF // 32, offd, wp, TK, E, H, EF)
+        torch.cuda.synchronize()
+        Wgf, Wuf, Wdf = deq(Wg, E * EF, H).reshape(E, EF, H), deq(Wu, E * EF, H).reshape(E, EF, H), deq(Wd, E * H, EF).reshape(E, H, EF)
+        for e in range(E):
+            lo, hi = int(off[e]), int(off[e + 1])
+            if lo == hi:
+                continue
+            xe = x[lo:hi].float()
+            gg, uu = xe @ Wgf[e].T, xe @ Wuf[e].T
+            href = (gg / (1 + torch.exp(-gg))) * uu
+            e1 = ((hp[lo:hi].float() - href).abs() / (href.abs() + 0.02 * href.abs().mean() + 1e-6)).max().item()
+            oref = (hp[lo:hi].float() @ Wdf[e].T) * wp[lo:hi].float()[:, None]
+            e2 = ((op[lo:hi].float() - oref).abs() / (oref.abs() + 0.02 * oref.abs().mean() + 1e-6)).max().item()
+            worst = max(worst, e1, e2)
+            assert e1 < 2e-3 and e2 < 2e-3, (it, E, H, EF, e, lo, hi, e1, e2)
+    print("grouped q8_0 GEMM, 12 random layers: worst relative error %.2e" % worst, flush=True)
