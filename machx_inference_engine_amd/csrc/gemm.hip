@@ -852,17 +852,22 @@ __device__ __forceinline__ void a_rows_to_lds(const TileCtx<QF, NA>& t, const ui
 }
 
 // Chunk c out of register set P; meanwhile (`more`) the A rows of chunk c+1 and the weights of chunk c+DEPTH are requested.
-template <class QF, bool PIPE, bool PARTIAL, int NA, int DEPTH, int P>
+// TAIL = one of the last chunks of the K loop, where chunk c+DEPTH may lie past the end: then no weight loads are issued
+// (loads nobody reads may be dropped by the compiler, and the wait below counts on them) and the A rows are waited for
+// with vmcnt(0).
+template <class QF, bool PIPE, bool PARTIAL, int NA, int DEPTH, int P, bool TAIL>
 __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint32_t (&a_off)[2 * NA], typename QF::Raw (&raw)[DEPTH + 1][2],
                                            const typename GemmWin<QF>::type (&win)[2], float16_t (&acc)[NA][2], uint32_t c, bool more) {
     constexpr int NSET = DEPTH + 1, PN = (P + DEPTH) % NSET;
     constexpr uint32_t ABUF = 32u * NA * kBK * 2u;
     constexpr int W_LOADS_MIN = 2 * (int)((sizeof(typename QF::Raw) + 15) / 16);
+    const bool w_next = !TAIL || c + DEPTH < t.n_chunks;   // the weights of chunk c+DEPTH exist
     if (more) {
         a_rows_to_lds<QF, NA>(t, a_off, c + 1, t.a_dst + ((c + 1) & 1u) * ABUF);
-        const uint32_t cn = (c + DEPTH < t.n_chunks) ? c + DEPTH : t.n_chunks - 1;   // past the end: the last chunk again, unused
-        raw[PN][0] = QF::load(t.w0, t.wrow0, t.c0 + cn, t.h);
-        raw[PN][1] = QF::load(t.w1, t.wrow1, t.c0 + cn, t.h);
+        if (w_next) {
+            raw[PN][0] = QF::load(t.w0, t.wrow0, t.c0 + c + DEPTH, t.h);
+            raw[PN][1] = QF::load(t.w1, t.wrow1, t.c0 + c + DEPTH, t.h);
+        }
         __builtin_amdgcn_sched_barrier(0);   // the scheduler must not sink these loads towards their uses
     }
     typename QF::Dec dec[2];
@@ -870,7 +875,10 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
     dec[1] = gemm_prepare<QF>(raw[P][1], win[1], t.c0 + c, t.h);
     mma_chunk<QF, PIPE, PARTIAL, NA>(raw[P], dec, t.lds_raw, (c & 1u) * ABUF + t.frag0, acc, t.mi);
     if (more) {
-        wait_vmcnt<(DEPTH > 1 ? W_LOADS_MIN : 0)>();   // A rows of chunk c+1 are in LDS (DEPTH > 1: the newest weight loads stay in flight)
+        // A rows of chunk c+1 are in LDS.  DEPTH > 1: the weight loads issued behind them in this chunk stay in flight
+        // (memory returns in order, so at most that many outstanding loads means the A rows have landed).
+        if (DEPTH > 1 && w_next) wait_vmcnt<W_LOADS_MIN>();
+        else wait_vmcnt<0>();
         // A barrier that waits for the LDS traffic only: __syncthreads() carries a fence that waits for every
         // outstanding load, the weight words requested for later chunks included.
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -989,26 +997,29 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
         raw[d][1] = QF::load(w1, wrow[1], c0 + cd, h);
     }
 
-#define CHUNK(P, c, more) gemm_chunk<QF, PIPE, PARTIAL, NA, DEPTH, P>(ctx, a_off, raw, win, acc, c, more)
+#define CHUNK(P, c, more, tail) gemm_chunk<QF, PIPE, PARTIAL, NA, DEPTH, P, tail>(ctx, a_off, raw, win, acc, c, more)
     if constexpr (DEPTH == 1) {
         // two sets, and the set just loaded is copied into set 0 at the end of a chunk, where it has to have arrived anyway
         for (uint32_t c = 0; c + 1 < n_chunks; ++c) {
-            CHUNK(0, c, true);
+            CHUNK(0, c, true, false);
             raw[0][0] = raw[1][0];
             raw[0][1] = raw[1][1];
         }
-        CHUNK(0, n_chunks - 1, false);
+        CHUNK(0, n_chunks - 1, false, true);
     } else {
+        // three sets in rotation; inside the loop every chunk has its chunk c+2 (c + 4 < n_chunks), the last one to four
+        // chunks check for it
         uint32_t c = 0;
-        for (; c + 3 < n_chunks; c += 3) {
-            CHUNK(0, c, true);
-            CHUNK(1, c + 1, true);
-            CHUNK(2, c + 2, true);
+        for (; c + 4 < n_chunks; c += 3) {
+            CHUNK(0, c, true, false);
+            CHUNK(1, c + 1, true, false);
+            CHUNK(2, c + 2, true, false);
         }
-        const uint32_t left = n_chunks - c;   // 1..3
-        CHUNK(0, c, left > 1);
-        if (left > 1) CHUNK(1, c + 1, left > 2);
-        if (left > 2) CHUNK(2, c + 2, false);
+        const uint32_t left = n_chunks - c;   // 1..4
+        CHUNK(0, c, left > 1, true);
+        if (left > 1) CHUNK(1, c + 1, left > 2, true);
+        if (left > 2) CHUNK(2, c + 2, left > 3, true);
+        if (left > 3) CHUNK(0, c + 3, false, true);
     }
 
 #undef CHUNK

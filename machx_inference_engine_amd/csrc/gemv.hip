@@ -543,15 +543,18 @@ static int cu_count() {
 }
 
 constexpr uint32_t kLdsBudget = 48 * 1024;
-// Workgroups of `kernel` that fit one CU at once (registers and `lds` bytes of dynamic LDS), asked once per kernel.
-// Persistent grids are sized with it: a workgroup that does not fit next to the others would run alone after them.
+// Workgroups of `kernel` that fit one CU at once (registers and `lds` bytes of dynamic LDS), asked once per kernel and
+// LDS size class (4 KB steps: the activation tile runs from a few KB to 48 KB with K and T, and the answer changes with
+// it).  Persistent grids are sized with it: a workgroup that does not fit next to the others would run alone after them.
 static uint32_t resident_wgs(const void* kernel, uint32_t lds) {
-    constexpr int kSlots = 512;   // a fixed table (nothing is allocated): kernels beyond it are asked about every time
-    static std::atomic<const void*> key[kSlots];
+    constexpr int kSlots = 1024;   // a fixed table (nothing is allocated): entries beyond it are asked about every time
+    static std::atomic<uintptr_t> key[kSlots];
     static std::atomic<uint32_t> val[kSlots];
+    const uint32_t cls = (lds + 4095u) / 4096u;                                  // 0 .. 40
+    const uintptr_t want = reinterpret_cast<uintptr_t>(kernel) * 64u + cls;     // user-space addresses leave the top bits free
     for (int i = 0; i < kSlots; ++i) {
-        const void* k = key[i].load(std::memory_order_acquire);
-        if (k == kernel) {
+        const uintptr_t k = key[i].load(std::memory_order_acquire);
+        if (k == want) {
             const uint32_t v = val[i].load(std::memory_order_acquire);
             if (v) return v;
             break;   // another thread is filling the slot: ask as well
@@ -559,10 +562,10 @@ static uint32_t resident_wgs(const void* kernel, uint32_t lds) {
         if (!k) break;
     }
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, (int)kGemvThreads, lds) != hipSuccess || n < 1) n = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, (int)kGemvThreads, cls * 4096u) != hipSuccess || n < 1) n = 1;
     for (int i = 0; i < kSlots; ++i) {
-        const void* expected = nullptr;
-        if (key[i].compare_exchange_strong(expected, kernel, std::memory_order_acq_rel) || expected == kernel) {
+        uintptr_t expected = 0;
+        if (key[i].compare_exchange_strong(expected, want, std::memory_order_acq_rel) || expected == want) {
             val[i].store((uint32_t)n, std::memory_order_release);
             break;
         }
@@ -1027,12 +1030,16 @@ static int check_ws(const void* ws, uint64_t ws_bytes, uint32_t K, uint32_t N, u
 int mx_gemv_batched_ws_bytes(uint32_t K, uint32_t N, uint32_t T, uint64_t* bytes) {
     MX_REQUIRE_PTR(bytes);
     MX_REQUIRE_SHAPE(K > 0 && N > 0 && T >= 1 && T <= 16);
-    // the K ranges the launch would like on this device (none: the row blocks fill the chip), T x N partial sums each
-    // batches of 5 and more run on the matrix cores (K ranges as the row blocks need them); smaller ones split K >= 8192 over up
-    // to kSplitMaxSlices slices
+    // The query carries no weight format, and which kernel a batch runs on depends on the format (launch_q8: the
+    // matrix-core kernel from T = 4 or 5 for most formats, from T = 9 for GGUF Q8_0 blocks), so the answer covers both
+    // routes: the vector kernels (batches up to 8) split K >= 8192 over up to kSplitMaxSlices slices, the matrix-core
+    // kernel takes the K ranges its row blocks leave room for; T x N partial sums per slice either way.
     uint32_t Z = 1;
-    if (T >= 5) Z = T <= 8 ? mmq_dense_ranges(K, N, 1, 4) : mmq_dense_ranges(K, N, 2, 2);
-    else if (T >= 2 && K >= 8192) Z = kSplitMaxSlices;
+    if (T >= 2 && T <= 8 && K >= 8192) Z = kSplitMaxSlices;
+    if (T >= 4) {
+        const uint32_t zm = T <= 8 ? mmq_dense_ranges(K, N, 1, 4) : mmq_dense_ranges(K, N, 2, 2);
+        if (zm > Z) Z = zm;
+    }
     *bytes = Z > 1 ? (uint64_t)Z * T * N * sizeof(float) : 0;
     return MX_OK;
 }

@@ -84,3 +84,23 @@ def test_workspace_forms_validate_before_any_hip_call(lib):
     assert l.mx_gemm_ws_bytes(128, 14336, 4096, None) == NULL
     assert l.mx_gemm_q4_K_ws(None, p16, p16, p16, 128, 14336, 4096, None, 64) == NULL
     assert l.mx_gemm_q4_K_ws(None, p16, p16, p16, 128, 14336, 4096, 0x1004, 64) == ALIGN
+
+
+def test_query_sized_workspace_is_never_refused(lib):
+    """mx_gemv_batched_ws_bytes carries no weight format, while the launch picks its kernel (and with it the number of K
+    slices) by format: whatever the format, batch and shape, a workspace of the size the query names must not come back
+    as MX_ERR_WORKSPACE.  Without a GPU the call gets past the workspace check and fails at the launch instead."""
+    l, _ = lib
+    WORKSPACE = 9
+    p16 = 0x1000
+    n = C.c_uint64(0)
+    shapes = [(14336, 4096), (14336, 1000), (8192, 14336), (8192, 512), (4096, 14336), (4096, 4096), (12288, 256), (16384, 151936)]
+    for K, N in shapes:
+        for T in range(2, 17):
+            assert l.mx_gemv_batched_ws_bytes(K, N, T, C.addressof(n)) == 0
+            ws = p16 if n.value else None
+            for rc in (l.mx_gemv_q8_0_soa_q8_batched_ws(None, p16, p16, p16, p16, K, N, T, ws, n.value),
+                       l.mx_gemv_q4_K_q8_batched_ws(None, p16, p16, p16, K, N, T, ws, n.value),
+                       l.mx_gemv_q6_K_q8_batched_ws(None, p16, p16, p16, K, N, T, ws, n.value),
+                       l.mx_gemv_q8_0_q8_batched_ws(None, p16, p16, p16, K, N, T, ws, n.value)):
+                assert rc != WORKSPACE, (K, N, T, n.value)

@@ -119,7 +119,44 @@ def check_envelope(got, lo, hi, what):
     assert ok.all(), (what, np.argwhere(~ok)[:5], got[~ok][:5], lo[~ok][:5], hi[~ok][:5])
 
 
-@pytest.mark.parametrize("T,H,EF,E,Kt", [(1, 2880, 2880, 32, 4), (3, 512, 320, 6, 2), (32, 704, 384, 8, 4), (32, 2880, 2880, 32, 4)])
+
+def check_gate_up_oai_rows(got, env, what, min_frac=0.999):
+    """Rows of half(swiglu_oai(half(g + bias), half(u + bias))) against the oracle: envelope of the reference chain,
+    cosine, and every element beyond 1e-3 of the fp64 chain explained by its own cancellation.  `env` holds one
+    ref_gate_up_oai() result per row."""
+    check_envelope(got, np.stack([e[0] for e in env]), np.stack([e[1] for e in env]), what)
+    g16, u16 = np.stack([e[2] for e in env]).astype(np.float64), np.stack([e[3] for e in env]).astype(np.float64)
+    centre = f16(O.swiglu_oai_np(g16.astype(np.float32), u16.astype(np.float32)))
+    check(got, centre, "  ... cosine against the fp64 chain", max_rel=1.0, cos=0.99999)
+    # first-order effect of one-ulp moves of g16 and u16 plus the output's own rounding
+    xg, z = np.minimum(g16, 7.0), np.clip(u16, -7.0, 7.0)
+    sg = 1.0 / (1.0 + np.exp(-1.702 * xg))
+    glu, dglu = xg * sg, np.where(g16 < 7.0, sg * (1.0 + 1.702 * xg * (1.0 - sg)), 0.0)
+    eta_g, eta_u = np.stack([e[4] for e in env]), np.stack([e[5] for e in env])
+    budget = ((ulp16(g16) + eta_g) * np.abs(dglu) * np.abs(z + 1.0) + np.where(np.abs(u16) < 7.0, ulp16(u16) + eta_u, 0.0) * np.abs(glu)
+              + ulp16(centre))
+    explained_outliers(got, centre, budget, what, min_frac)
+
+
+def check_down_bias_rows(got, Wd, bd, experts, hq_rows, EF, H, what, min_frac=0.999):
+    """Rows of half(half(acc) + bias) against the oracle: `experts[r]` is the expert of row r, `hq_rows` the block_q8_1x
+    bytes the kernel read (one row of EF / 32 * 40 bytes per output row)."""
+    hrb = EF // 32 * 40
+    lo, hi, ctr, a16s = [], [], [], []
+    for r, e in enumerate(experts):   # envelope over half(acc) moving by one ulp (the sum with the bias can cancel)
+        acc = O.gemv_q8chain(O.MXFP4, Wd[e], hq_rows[r * hrb:(r + 1) * hrb], EF, H)[0].astype(np.float64)
+        cands = f16_candidates(acc, sum_noise(acc))
+        c = [f16(v.astype(np.float32) + bd[e]) for v in cands]
+        lo.append(np.min(c, axis=0))
+        hi.append(np.max(c, axis=0))
+        ctr.append(c[1])
+        a16s.append(cands[1].astype(np.float32))
+    check_envelope(got, np.stack(lo), np.stack(hi), what)
+    ctr = np.stack(ctr)
+    explained_outliers(got, ctr, ulp16(np.stack(a16s)) + ulp16(ctr), what, min_frac)
+
+
+@pytest.mark.parametrize("T,H,EF,E,Kt", [(1, 2880, 2880, 32, 4), (3, 512, 320, 6, 2), (32, 704, 384, 8, 4), (48, 704, 384, 4, 2), (32, 2880, 2880, 32, 4)])
 def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     """gpt-oss style layer: gate/up (+bias, swiglu_oai) -> quantize -> down (+bias) -> weighted reduce.
     H=EF=2880, E=32, top-4 at T=1 and T=32 are BASELINE config 4's two cases at full size (every packed row of
@@ -138,18 +175,7 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     h = ops.moe_gate_up_oai_mxfp4(dev(xq), D["gq"], D["ge"], D["uq"], D["ue"], qs_st, e_st, D["bg"], D["bu"], dev(ids.ravel()), T, Kt, H, EF, E)
     h_h = host(h).astype(np.float32)
     env = [ref_gate_up_oai(Wg, Wu, bg, bu, ids[t, k], xq[t * rb:(t + 1) * rb], H, EF) for t in range(T) for k in range(Kt)]
-    check_envelope(h_h, np.stack([e[0] for e in env]), np.stack([e[1] for e in env]), "moe gate_up swiglu_oai (decode) T=%d" % T)
-    g16, u16 = np.stack([e[2] for e in env]).astype(np.float64), np.stack([e[3] for e in env]).astype(np.float64)
-    centre = f16(O.swiglu_oai_np(g16.astype(np.float32), u16.astype(np.float32)))
-    check(h_h, centre, "  ... cosine against the fp64 chain", max_rel=1.0, cos=0.99999)
-    # first-order effect of one-ulp moves of g16 and u16 plus the output's own rounding
-    xg, z = np.minimum(g16, 7.0), np.clip(u16, -7.0, 7.0)
-    sg = 1.0 / (1.0 + np.exp(-1.702 * xg))
-    glu, dglu = xg * sg, np.where(g16 < 7.0, sg * (1.0 + 1.702 * xg * (1.0 - sg)), 0.0)
-    eta_g, eta_u = np.stack([e[4] for e in env]), np.stack([e[5] for e in env])
-    budget = ((ulp16(g16) + eta_g) * np.abs(dglu) * np.abs(z + 1.0) + np.where(np.abs(u16) < 7.0, ulp16(u16) + eta_u, 0.0) * np.abs(glu)
-              + ulp16(centre))
-    explained_outliers(h_h, centre, budget, "moe gate_up swiglu_oai (decode) T=%d" % T, 0.999)
+    check_gate_up_oai_rows(h_h, env, "moe gate_up swiglu_oai (decode) T=%d" % T)
     hq = ops.quantize_q8_1(h)
     hq_h = host(hq)
     assert np.array_equal(hq_h, O.quantize_q8_1(h_h))
@@ -158,21 +184,7 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     # h taken as fp16 and quantized while staged: the same q8 tile, so the same bits out
     out_f = ops.moe_down_mxfp4_f16(h, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(ids.ravel()), T, Kt, EF, H, E)
     assert np.array_equal(host(out_f), host(out)), "down on fp16 h != quantize + down"
-    hrb = EF // 32 * 40
-    inf = np.float16(np.inf)
-    lo, hi, ctr, a16s = [], [], [], []
-    for s_ in range(T * Kt):   # out = half(half(acc) + bias): envelope over half(acc) moving by one ulp (the sum can cancel)
-        acc = O.gemv_q8chain(O.MXFP4, Wd[ids.ravel()[s_]], hq_h[s_ * hrb:(s_ + 1) * hrb], EF, H)[0].astype(np.float64)
-        cands = f16_candidates(acc, sum_noise(acc))
-        a16 = cands[1]
-        c = [f16(v.astype(np.float32) + bd[ids.ravel()[s_]]) for v in cands]
-        lo.append(np.min(c, axis=0))
-        hi.append(np.max(c, axis=0))
-        ctr.append(c[1])
-        a16s.append(a16.astype(np.float32))
-    check_envelope(out_h, np.stack(lo), np.stack(hi), "moe down + bias (decode)")
-    ctr = np.stack(ctr)
-    explained_outliers(out_h, ctr, ulp16(np.stack(a16s)) + ulp16(ctr), "moe down + bias (decode) T=%d" % T, 0.999)
+    check_down_bias_rows(out_h, Wd, bd, ids.ravel(), hq_h, EF, H, "moe down + bias (decode) T=%d" % T)
     y = torch.zeros((T, H), dtype=torch.float16, device="cuda")
     ident = dev(np.arange(T * Kt, dtype=np.uint32))
     ops.moe_prefill_reduce(out, ident, dev(w.ravel()).half(), y, T, Kt, H)
@@ -187,12 +199,19 @@ def test_moe_mxfp4_decode_and_grouped(mx, T, H, EF, E, Kt):
     assert np.array_equal(host(xp), x[si].astype(np.float16))
     xpq = ops.quantize_q8_1(xp)
     hp = ops.moe_grouped_gate_up_oai_mxfp4(xpq, D["gq"], D["ge"], D["uq"], D["ue"], qs_st, e_st, D["bg"], D["bu"], dev(off), TK, E, H, EF)
-    # same products per (token, expert); only the compiler's fma grouping may differ between the
-    # 1-row and the tiled instantiation, so rows agree to fp16 rounding of an fp32-noise difference
-    check_rows(host(hp)[t2p], host(h), "grouped gate_up == decode rows")
+    # The grouped kernels (for H, EF >= 256 the scaled FP8 x FP4 matrix instruction) against the oracle itself: packed row
+    # t2p[slot] holds the same token and expert as decode slot `slot`, and its q8 row is the same bytes, so the
+    # per-slot envelopes apply to it unchanged.
+    assert np.array_equal(host(xpq).reshape(TK, -1)[t2p].ravel(), xq.reshape(T, -1).repeat(Kt, axis=0).ravel())
+    check_gate_up_oai_rows(host(hp).astype(np.float32)[t2p], env, "moe gate_up swiglu_oai (grouped) T=%d" % T)
+    check_rows(host(hp)[t2p], host(h), "grouped gate_up vs decode rows")
     hpq = ops.quantize_q8_1(hp)
+    hpq_h = host(hpq)
+    assert np.array_equal(hpq_h, O.quantize_q8_1(host(hp).astype(np.float32)))
     op = ops.moe_grouped_down_mxfp4(hpq, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(off), TK, E, H, EF)
-    check_rows(host(op)[t2p], host(out), "grouped down == decode rows")
+    row_expert = np.repeat(np.arange(E), np.diff(off.astype(np.int64)))
+    check_down_bias_rows(host(op).astype(np.float32), Wd, bd, row_expert, hpq_h, EF, H, "moe down + bias (grouped) T=%d" % T)
+    check_rows(host(op)[t2p], host(out), "grouped down vs decode rows")
     op_f = ops.moe_grouped_down_mxfp4_f16(hp, D["dq"], D["de"], dqs_st, de_st, D["bd"], dev(off), TK, E, H, EF)
     assert np.array_equal(host(op_f), host(op)), "grouped down on fp16 h != quantize + grouped down"
     y2 = torch.zeros((T, H), dtype=torch.float16, device="cuda")
@@ -234,11 +253,102 @@ def test_moe_q8_0_decode_and_grouped(mx, T, H, EF, E, Kt):
     TK = T * Kt
     xpq = ops.quantize_q8_1(ops.moe_gather_rows(dev(x).half(), dev(si), TK, H))
     hp = ops.moe_prefill_gate_up_silu_q8(xpq, dev(gq), dev(gd), dev(uq), dev(ud), qs_st, d_st, dev(off), TK, E, H, EF)
-    check_rows(host(hp)[t2p], host(h), "grouped gate_up == decode rows")
-    op = ops.moe_prefill_down_q8(ops.quantize_q8_1(hp), dev(dq), dev(dd), dqs_st, dd_st, dev(off), dev(wp).half(), TK, E, H, EF)
-    check_rows(host(op)[t2p], host(yp), "grouped down == decode rows")
+    check(host(hp).astype(np.float32)[t2p], h_ref, "moe_prefill_gate_up_silu_q8 (grouped) T=%d" % T)
+    check_rows(host(hp)[t2p], host(h), "grouped gate_up vs decode rows")
+    hpq = ops.quantize_q8_1(hp)
+    hpq_h = host(hpq)
+    op = ops.moe_prefill_down_q8(hpq, dev(dq), dev(dd), dqs_st, dd_st, dev(off), dev(wp).half(), TK, E, H, EF)
+    row_expert = np.repeat(np.arange(E), np.diff(off.astype(np.int64)))
+    op_ref = np.stack([f16(wp[r]) * O.gemv_q8chain(O.Q8_0, Wd[row_expert[r]], hpq_h[r * hrb:(r + 1) * hrb], EF, H)[0] for r in range(TK)])
+    check(host(op).astype(np.float32), op_ref, "moe_prefill_down_q8 (grouped) T=%d" % T)
+    check_rows(host(op)[t2p], host(yp), "grouped down vs decode rows")
     y2 = ops.moe_prefill_reduce_sum(op, dev(t2p.astype(np.uint32)), T, Kt, H)
     check_rows(host(y2), host(y), "grouped layer output == decode layer output")
+
+
+def _mxfp4_bank(seed, E, N, K, e_choices):
+    """Random E2M1 codes and per-block exponents drawn from `e_choices` -> (AoS blocks [E, N, K/32*17], qs plane, e plane)."""
+    rng = np.random.default_rng(seed)
+    W = rng.integers(0, 256, size=(E, N, K // 32, 17), dtype=np.uint8)
+    W[..., 0] = rng.choice(np.asarray(e_choices, np.uint8), size=(E, N, K // 32))
+    W = W.reshape(E, N, K // 32 * 17)
+    qs, e = O.repack_mxfp4_to_soa(W)
+    return W, qs, e
+
+
+def _q8_rows(seed, rows, K, d, qmax):
+    """Hand-built block_q8_1x rows: every block {d, d * sum(q), q[32]} with q uniform in [-qmax, qmax]."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(-qmax, qmax + 1, size=(rows, K // 32, 32)).astype(np.int8)
+    buf = np.zeros((rows, K // 32, 40), np.uint8)
+    buf[..., 0:4] = np.frombuffer(np.float32(d).tobytes(), np.uint8)
+    buf[..., 4:8] = (np.float32(d) * q.sum(axis=2).astype(np.float32)).astype(np.float32).view(np.uint8).reshape(rows, K // 32, 4)
+    buf[..., 8:] = q.view(np.uint8)
+    return buf.reshape(-1), q.reshape(rows, K).astype(np.int64)
+
+
+E2M1_X2 = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)   # doubled E2M1 values, include/ie/quant_blocks.hpp:46-60
+
+
+def _mxfp4_codes_x2(W, N, K):
+    """[E, N, K] doubled E2M1 values of a bank of 17-byte blocks (element j in the low, j + 16 in the high nibble of byte j)."""
+    b = W.reshape(W.shape[0], N, K // 32, 17)[..., 1:]
+    return np.concatenate([E2M1_X2[b & 15], E2M1_X2[b >> 4]], axis=-1).reshape(W.shape[0], N, K)
+
+
+@pytest.mark.parametrize("counts", [(5, 20, 33), (1, 0, 16, 17)])
+def test_moe_grouped_mxfp4_integer_part_exact(mx, counts):
+    """Grouped MXFP4 down projection with every scale a power of two (e = 127: weights are the E2M1 values themselves;
+    activation rows with d = 1 and small codes): the sum is an exact multiple of 1/2 well inside fp32's integer range,
+    so whatever the summation order the fp32 result is the brute-force integer sum and the output is its one rounding
+    to fp16, bit for bit.  Expert sizes cover one partial token pass, a full one, and one row beyond a full pass."""
+    ops = mx.ops
+    E, K, N = len(counts), 512, 96
+    W, qs, e = _mxfp4_bank(31, E, N, K, [127])
+    off = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    TK = int(off[-1])
+    xq, q = _q8_rows(32, TK, K, 1.0, 3)
+    bias = np.zeros((E, N), np.float32)
+    out = ops.moe_grouped_down_mxfp4(dev(xq), dev(qs), dev(e), N * K // 2, N * K // 32, dev(bias), dev(off), TK, E, N, K)
+    codes = _mxfp4_codes_x2(W, N, K)
+    row_expert = np.repeat(np.arange(E), counts)
+    exact = np.stack([codes[row_expert[r]] @ q[r] for r in range(TK)]).astype(np.float64) / 2.0   # e8m0_half(127) = 1/2 of the doubled value
+    assert np.abs(exact).max() < 2048
+    assert np.array_equal(host(out), exact.astype(np.float16)), "grouped MXFP4 down: integer part not exact"
+    # gate/up: with all-zero up codes u = 0 and z + 1 = 1, so h = half(glu(half(g))) is a function of the exact gate sum
+    # alone (2 fp16 ulps for the device exponential); then the same with the roles swapped through a constant gate.
+    EF = 64
+    Wg, gq, ge = _mxfp4_bank(33, E, EF, K, [120])       # scale 2^-8 of the doubled value: |g| stays below the clamp at 7
+    zero_q, zero_e = np.zeros_like(gq), np.full_like(ge, 120)
+    bz = np.zeros((E, EF), np.float32)
+    g_exact = np.stack([_mxfp4_codes_x2(Wg, EF, K)[row_expert[r]] @ q[r] for r in range(TK)]).astype(np.float64) / 256.0
+    assert np.abs(g_exact).max() < 7.0
+    g16 = g_exact.astype(np.float16).astype(np.float64)
+    hp = ops.moe_grouped_gate_up_oai_mxfp4(dev(xq), dev(gq), dev(ge), dev(zero_q), dev(zero_e), EF * K // 2, EF * K // 32, dev(bz), dev(bz), dev(off), TK, E, K, EF)
+    ref = g16 / (1.0 + np.exp(-1.702 * g16))
+    assert np.all(np.abs(host(hp).astype(np.float64) - ref) <= 2.0 * ulp16(ref) + 2.0 ** -24), "gate sums through swiglu_oai"
+    bg1 = np.ones((E, EF), np.float32)
+    hp = ops.moe_grouped_gate_up_oai_mxfp4(dev(xq), dev(zero_q), dev(zero_e), dev(gq), dev(ge), EF * K // 2, EF * K // 32, dev(bg1), dev(bz), dev(off), TK, E, K, EF)
+    ref = (1.0 / (1.0 + np.exp(-1.702))) * (g16 + 1.0)
+    assert np.all(np.abs(host(hp).astype(np.float64) - ref) <= 2.0 * ulp16(ref) + 2.0 ** -24), "up sums through swiglu_oai"
+
+
+def test_moe_grouped_mxfp4_exponent_range(mx):
+    """Exponent bytes across the range real MXFP4 tensors use and well beyond (2^-100 .. 2^+60 of the doubled value), with
+    activation scales that bring the products back into fp16 range: the grouped kernel hands the stored byte to the
+    matrix instruction as its block scale, the oracle goes through e8m0_half (include/ie/quant_blocks.hpp:46-54)."""
+    ops = mx.ops
+    E, K, N, counts = 2, 512, 64, (9, 20)
+    off = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    TK = int(off[-1])
+    bias = np.zeros((E, N), np.float32)
+    row_expert = np.repeat(np.arange(E), counts)
+    for e_lo, d in ((28, 2.0 ** 88), (100, 2.0 ** 16), (126, 2.0 ** -10), (186, 2.0 ** -70)):
+        W, qs, e = _mxfp4_bank(40 + e_lo, E, N, K, [e_lo, e_lo + 1, e_lo + 2])
+        xq, _ = _q8_rows(41, TK, K, d, 127)
+        out = ops.moe_grouped_down_mxfp4(dev(xq), dev(qs), dev(e), N * K // 2, N * K // 32, dev(bias), dev(off), TK, E, N, K)
+        ref = np.stack([O.gemv_q8chain(O.MXFP4, W[row_expert[r]], xq[r * (K // 32 * 40):(r + 1) * (K // 32 * 40)], K, N)[0] for r in range(TK)])
+        check(host(out).astype(np.float32), ref, "grouped MXFP4 down, exponents %d..%d" % (e_lo, e_lo + 2))
 
 
 def test_moe_grouped_skips_empty_and_single_row_experts(mx):
