@@ -447,6 +447,16 @@ int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const ui
                    uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
                    uint32_t K, uint32_t E_ffn, uint32_t H);
 int mx_moe_reduce_q8(mx_stream_t s, const uint16_t* y_packed, uint16_t* y, uint32_t T, uint32_t K, uint32_t H);
+/* The same two launches with the number of experts in the bank as a last argument (no counterpart in the reference,
+ * whose signatures carry no expert count): a slot whose id lies outside [0, n_experts) is skipped, its output row is
+ * left as it was.  Through the reference signatures above only negative ids can be recognised; a positive id past
+ * the bank would read past it.  */
+int mx_moe_gate_up_silu_q8_n(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
+                             const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx,
+                             uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H, uint32_t E_ffn, uint32_t n_experts);
+int mx_moe_down_q8_n(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                     uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
+                     uint32_t K, uint32_t E_ffn, uint32_t H, uint32_t n_experts);
 /* K-quant expert-major expert banks with fp16 activations, decode — the reference's fused
  * Q4_K / Q6_K expert kernels; fp32 fold acc += (d*sc)*sum(a*q) - (dmin*m)*sum(a):
  *   moe_decode_gate_up_silu_q4k  include/ie/ops.hpp:1034-1041, src/ops/moe_fused.cpp:82-211
@@ -478,7 +488,11 @@ int mx_moe_decode_down_q6k(mx_stream_t s, const uint16_t* h, const void* down_W,
  *                                         include/ie/ops.hpp:993-1006, src/ops/moe_fused.cpp:1603-1924
  *     out_packed[row, n] = half(down_e . h_row), unweighted (moe_prefill_reduce applies the weights);
  *     any E_ffn % 256 == 0 (the reference's register-resident variant needs E_ffn == 512).
-  */
+ * total_rows is the one argument the reference signatures do not have.  It only picks the launch shape (rows staged
+ * per workgroup and row blocks per workgroup are sized for total_rows / E rows per expert) and never changes a
+ * result: the rows that are computed are those expert_offsets names.  0xFFFFFFFF means "not known" and is always
+ * legal (the launch is then sized for large, uneven experts); a wrapper with the reference's exact argument list
+ * passes that value.  The same holds for every other total_rows argument of this header.  */
 int mx_moe_prefill_gate_up_silu_q4k_q8(mx_stream_t s, const void* xq8s_packed, const void* gate_W, const void* up_W,
                                        const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
                                        uint32_t E_ffn, uint64_t expert_stride_bytes, int soa, uint32_t total_rows);
@@ -524,7 +538,13 @@ int mx_moe_scatter_add(mx_stream_t s, const uint16_t* x_packed, const int32_t* i
  * device, with the same rounding points: h = half(swiglu_oai(half(gate.x + bg),
  * half(up.x + bu))), out = half(half(down.h) + bd).  Biases fp32 [E][N], may be NULL.
  * Decode form reads topk_idx; grouped form takes expert-sorted rows +
- * expert_offsets (total_rows = expert_offsets[E], known to the host from the packing).  */
+ * expert_offsets (total_rows = expert_offsets[E], known to the host from the packing).
+ * Exponent bytes: the grouped entry points with H (gate/up) or E_ffn (down) of 256 and more hand the stored E8M0 byte
+ * to the scaled matrix instruction, whose block sum is formed in fp32 before the activation scale is applied.  They
+ * agree with the decode kernels and with e8m0_half (include/ie/quant_blocks.hpp:46-54) for exponent bytes 2 .. 240
+ * (2^-126 .. 2^112 of the doubled E2M1 value; trained tensors sit near 2^-10); byte 255 is NaN to the instruction (as
+ * in the OCP MX definition) where e8m0_half returns 2^127, and beyond 240 a block sum can overflow fp32 before the
+ * activation scale brings it back.  */
 int mx_moe_gate_up_oai_mxfp4(mx_stream_t s, const void* x_q8, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs,
                              const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride, const float* gate_bias,
                              const float* up_bias, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
@@ -553,6 +573,9 @@ int mx_moe_grouped_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_packed_f16, c
 int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
                        uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
                        uint32_t K, uint32_t E_ffn, uint32_t H);
+int mx_moe_down_q8_f16_n(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
+                         uint64_t d_stride, const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T,
+                         uint32_t K, uint32_t E_ffn, uint32_t H, uint32_t n_experts);   /* ids outside [0, n_experts) skipped */
 /* ---------------------------------------------------------------- MoE routing and packing on the device
  *   moe_router             include/ie/ops.hpp:780-786, src/ops/moe.cpp:22-216
  *     logits = W_gate[E,H] (fp32) . x_t, softmax, top-k, renormalise, ascending expert id; any

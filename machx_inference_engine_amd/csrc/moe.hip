@@ -510,10 +510,12 @@ static int gemm_q8_rows(mx_stream_t s, const void* xq8s_packed, const typename F
 extern "C" {
 
 // ------------------------------------------------------------ Q8_0 SoA experts, decode
-int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d,
-                           uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
-                           uint32_t E_ffn) {
-    const uint32_t n_experts = 0x80000000u;   // the reference signature carries no expert count: only negative ids can be told apart (their slots are skipped)
+// The reference signatures carry no expert count, so through them only negative ids can be told apart (their slots are
+// skipped); the *_n forms take the count and skip every id outside [0, n_experts).
+constexpr uint32_t kAnyExpert = 0x80000000u;
+int mx_moe_gate_up_silu_q8_n(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d,
+                             uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
+                             uint32_t E_ffn, uint32_t n_experts) {
     if (int rc = check_moe(x_q8, h_out, H, E_ffn, T * K)) return rc;
     MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d); MX_REQUIRE_PTR(topk_idx);
     MX_REQUIRE_SHAPE(K > 0 && n_experts > 0 && qs_stride % 16 == 0);
@@ -524,9 +526,14 @@ int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, 
     FmtQ8Soa::Bank bg{g_qs, g_d, qs_stride, d_stride, H}, bu{u_qs, u_d, qs_stride, d_stride, H};
     return launch_moe<FmtQ8Soa, 2, EPI_SILU>(s, bg, bu, a, T * K, 1);
 }
-int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
-                   const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
-    const uint32_t n_experts = 0x80000000u;
+int mx_moe_gate_up_silu_q8(mx_stream_t s, const void* x_q8, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d,
+                           uint64_t qs_stride, uint64_t d_stride, const int32_t* topk_idx, uint16_t* h_out, uint32_t T, uint32_t K, uint32_t H,
+                           uint32_t E_ffn) {
+    return mx_moe_gate_up_silu_q8_n(s, x_q8, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, topk_idx, h_out, T, K, H, E_ffn, kAnyExpert);
+}
+int mx_moe_down_q8_n(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                     const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H,
+                     uint32_t n_experts) {
     if (int rc = check_moe(h_q8, y_packed, E_ffn, H, T * K)) return rc;
     MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(topk_w);
     MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
@@ -536,6 +543,10 @@ int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const ui
     a.out = reinterpret_cast<half_t*>(y_packed); a.act_div = 1; a.K = E_ffn; a.N = H; a.n_experts = n_experts;
     FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
     return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, T * K, 1);
+}
+int mx_moe_down_q8(mx_stream_t s, const void* h_q8, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                   const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
+    return mx_moe_down_q8_n(s, h_q8, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, y_packed, T, K, E_ffn, H, kAnyExpert);
 }
 // ------------------------------------------------------------ K-quant experts, fp16 activations, decode
 // soa != 0: every expert region holds its blocks as per-field streams (include/ie/quant_soa.hpp:33-51)
@@ -702,12 +713,12 @@ int mx_moe_grouped_down_mxfp4_f16(mx_stream_t s, const uint16_t* h_packed_f16, c
     return moe_mxfp4_down(s, h_packed_f16, d_qs, d_e, qs_stride, e_stride, down_bias, nullptr, expert_offsets, out_packed, E, E_ffn, H, E,
                           avg_rows(total_rows, E), true);
 }
-int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
-                       const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
-    const uint32_t n_experts = 0x80000000u;
+int mx_moe_down_q8_f16_n(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                         const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H,
+                         uint32_t n_experts) {
     if (int rc = check_moe(h_f16, y_packed, E_ffn, H, T * K)) return rc;
     MX_REQUIRE_PTR(d_qs); MX_REQUIRE_PTR(d_d); MX_REQUIRE_PTR(topk_idx); MX_REQUIRE_PTR(topk_w);
-    MX_REQUIRE_SHAPE(qs_stride % 16 == 0);
+    MX_REQUIRE_SHAPE(n_experts > 0 && qs_stride % 16 == 0);
     MX_REQUIRE_ALIGN(d_qs, 16); MX_REQUIRE_ALIGN(h_f16, 16);
     MoeArgs a{};
     a.act_f16 = reinterpret_cast<const half_t*>(h_f16); a.xq8 = reinterpret_cast<const uint8_t*>(h_f16); a.topk_idx = topk_idx;
@@ -715,6 +726,10 @@ int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs,
     a.n_experts = n_experts;
     FmtQ8Soa::Bank b{d_qs, d_d, qs_stride, d_stride, E_ffn};
     return launch_moe<FmtQ8Soa, 1, EPI_DOWN_WEIGHTED>(s, b, b, a, T * K, 1);
+}
+int mx_moe_down_q8_f16(mx_stream_t s, const uint16_t* h_f16, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
+                       const int32_t* topk_idx, const uint16_t* topk_w, uint16_t* y_packed, uint32_t T, uint32_t K, uint32_t E_ffn, uint32_t H) {
+    return mx_moe_down_q8_f16_n(s, h_f16, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, y_packed, T, K, E_ffn, H, kAnyExpert);
 }
 
 // ------------------------------------------------------------ Q4_0 experts (Gemma-4 MoE) and the dense W4A8 GEMM

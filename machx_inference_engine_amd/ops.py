@@ -251,25 +251,35 @@ def gemv_mxfp4_soa_f16(A, qs_plane, e_plane, K, N, y=None):
 
 
 # ---------------------------------------------------------------- MoE, expert-indexed GEMV
-def moe_gate_up_silu_q8(x_q8, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, topk_idx, T, K, H, E_ffn, h_out=None):
+def moe_gate_up_silu_q8(x_q8, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, topk_idx, T, K, H, E_ffn, h_out=None, n_experts=None):
+    """n_experts given: the *_n entry point, slots whose id lies outside [0, n_experts) are skipped."""
     h_out = _out(h_out, (T * K, E_ffn), torch.float16, x_q8)
-    _call("mx_moe_gate_up_silu_q8", _u8(x_q8), _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d), qs_stride, d_stride, _ptr(topk_idx),
-          _ptr(h_out), T, K, H, E_ffn)
+    args = (_u8(x_q8), _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d), qs_stride, d_stride, _ptr(topk_idx), _ptr(h_out), T, K, H, E_ffn)
+    if n_experts is None:
+        _call("mx_moe_gate_up_silu_q8", *args)
+    else:
+        _call("mx_moe_gate_up_silu_q8_n", *args, n_experts)
     return h_out
 
 
-def moe_down_q8(h_q8, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_ffn, H, y_packed=None):
+def moe_down_q8(h_q8, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_ffn, H, y_packed=None, n_experts=None):
     y_packed = _out(y_packed, (T * K, H), torch.float16, h_q8)
-    _call("mx_moe_down_q8", _u8(h_q8), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(topk_idx), _f16(topk_w), _ptr(y_packed),
-          T, K, E_ffn, H)
+    args = (_u8(h_q8), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(topk_idx), _f16(topk_w), _ptr(y_packed), T, K, E_ffn, H)
+    if n_experts is None:
+        _call("mx_moe_down_q8", *args)
+    else:
+        _call("mx_moe_down_q8_n", *args, n_experts)
     return y_packed
 
 
-def moe_down_q8_f16(h_f16, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_ffn, H, y_packed=None):
+def moe_down_q8_f16(h_f16, d_qs, d_d, qs_stride, d_stride, topk_idx, topk_w, T, K, E_ffn, H, y_packed=None, n_experts=None):
     """moe_down_q8 on fp16 h rows [T*K][E_ffn], quantized while they are staged (no quantize launch)."""
     y_packed = _out(y_packed, (T * K, H), torch.float16, h_f16)
-    _call("mx_moe_down_q8_f16", _f16(h_f16), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(topk_idx), _f16(topk_w), _ptr(y_packed),
-          T, K, E_ffn, H)
+    args = (_f16(h_f16), _u8(d_qs), _ptr(d_d), qs_stride, d_stride, _ptr(topk_idx), _f16(topk_w), _ptr(y_packed), T, K, E_ffn, H)
+    if n_experts is None:
+        _call("mx_moe_down_q8_f16", *args)
+    else:
+        _call("mx_moe_down_q8_f16_n", *args, n_experts)
     return y_packed
 
 

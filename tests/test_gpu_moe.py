@@ -351,6 +351,34 @@ def test_moe_grouped_mxfp4_exponent_range(mx):
         check(host(out).astype(np.float32), ref, "grouped MXFP4 down, exponents %d..%d" % (e_lo, e_lo + 2))
 
 
+def test_moe_q8_decode_skips_ids_outside_the_bank(mx):
+    """The *_n decode entry points: slots whose expert id is negative or not below n_experts are skipped (their output
+    rows keep their contents), every other slot equals the plain entry point's row."""
+    ops = mx.ops
+    T, Kt, E, H, EF = 3, 4, 4, 512, 256
+    Wg, gq, gd, qs_st, d_st = make_experts(O.Q8_0, 900, E, EF, H)
+    Wu, uq, ud, _, _ = make_experts(O.Q8_0, 910, E, EF, H)
+    Wd, dq, dd, dqs_st, dd_st = make_experts(O.Q8_0, 920, E, H, EF)
+    x = f16(O.normal(11, (T, H)))
+    ids = np.array([[0, 1, 2, 3], [3, E, 1, -1], [2, 7, 1 << 20, 0]], np.int32)
+    good = ((ids >= 0) & (ids < E)).ravel()
+    safe = np.where(good.reshape(ids.shape), ids, 0).astype(np.int32)
+    w16 = dev(f16(np.full(ids.size, 0.25, np.float32))).half()
+    xq = dev(O.quantize_q8_1(x))
+    args = (xq, dev(gq), dev(gd), dev(uq), dev(ud), qs_st, d_st)
+    h_ref = ops.moe_gate_up_silu_q8(*args, dev(safe.ravel()), T, Kt, H, EF)
+    h = torch.full((T * Kt, EF), 7.0, dtype=torch.float16, device="cuda")
+    ops.moe_gate_up_silu_q8(*args, dev(ids.ravel()), T, Kt, H, EF, h_out=h, n_experts=E)
+    assert np.array_equal(host(h)[good], host(h_ref)[good]) and np.all(host(h)[~good] == 7.0)
+    hq = ops.quantize_q8_1(h_ref)
+    dargs = (dev(dq), dev(dd), dqs_st, dd_st)
+    y_ref = ops.moe_down_q8(hq, *dargs, dev(safe.ravel()), w16, T, Kt, EF, H)
+    for fn, act in ((ops.moe_down_q8, hq), (ops.moe_down_q8_f16, h_ref)):
+        y = torch.full((T * Kt, H), 7.0, dtype=torch.float16, device="cuda")
+        fn(act, *dargs, dev(ids.ravel()), w16, T, Kt, EF, H, y_packed=y, n_experts=E)
+        assert np.array_equal(host(y)[good], host(y_ref)[good]) and np.all(host(y)[~good] == 7.0)
+
+
 def test_moe_grouped_skips_empty_and_single_row_experts(mx):
     """Experts with 0 rows write nothing; 1-row experts are exact (the reference notes
     wrong rows for tiny per-expert batches on its dense-GEMM route, gptoss_tp.cpp:702-765)."""
