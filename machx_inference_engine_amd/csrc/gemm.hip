@@ -1060,6 +1060,117 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
         }
 }
 
+// Expert-grouped tile `tm` -> (expert, first row, end of the expert's rows), found by one wave.
+// Tile order over all experts: every full BM-row tile first (expert by expert), then the experts' partial last tiles,
+// those with the most live 32-row sub-tiles first.  A tile's cost grows with its live sub-tiles, so the workgroups
+// dispatched last are the cheapest ones and the launch does not end with a few expensive tiles running alone (list
+// scheduling, longest first).  The per-expert row counts are read 256 experts at a time, every load of a block issued
+// before the first is used: with up to 256 experts the lookup costs one memory round trip (a loop that loads, scans
+// and decides expert group by expert group and class by class pays one per step, several microseconds per tile).
+// Returns false for a tile number past the last tile.
+template <uint32_t BM, int NI>
+__device__ __forceinline__ bool find_grouped_tile(const uint32_t* expert_offsets, uint32_t E, uint32_t tm, uint32_t ln, uint32_t (&out)[3]) {
+    constexpr int JU = 4;   // expert groups of 64 per block
+    struct Block {
+        uint32_t lo[JU], hi[JU], full[JU], cls[JU];
+    };
+    auto load = [&](uint32_t e0, Block& b) {
+#pragma unroll
+        for (int j = 0; j < JU; ++j) {
+            const uint32_t ee = e0 + 64u * j + ln;
+            b.lo[j] = ee < E ? expert_offsets[ee] : 0u;
+            b.hi[j] = ee < E ? expert_offsets[ee + 1] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < JU; ++j) {
+            const uint32_t n = b.hi[j] - b.lo[j], rem = n % BM;
+            b.full[j] = n / BM;
+            b.cls[j] = (rem + 31u) / 32u;   // live sub-tiles of the partial tile, 0: none
+        }
+    };
+    auto wave_sum = [&](uint32_t v) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) v += (uint32_t)__shfl_xor((int)v, d);
+        return v;
+    };
+    uint32_t tot_full = 0, n_cls[NI + 1] = {};
+    auto count = [&](const Block& b) {
+#pragma unroll
+        for (int j = 0; j < JU; ++j) {
+            tot_full += wave_sum(b.full[j]);
+#pragma unroll
+            for (int k = 1; k <= NI; ++k) n_cls[k] += (uint32_t)__popcll(__ballot(b.cls[j] == (uint32_t)k));
+        }
+    };
+    // locate state: the segment (full tiles, or class k) and the index inside it
+    uint32_t seg = 0, idx = tm, seen = 0;
+    bool found = false;
+    auto locate = [&](uint32_t e0, const Block& b) {
+#pragma unroll
+        for (int j = 0; j < JU; ++j) {
+            if (found) break;
+            const uint32_t ee = e0 + 64u * j + ln;
+            bool hit;
+            uint32_t first;
+            if (seg == 0) {
+                uint32_t incl = b.full[j];
+#pragma unroll
+                for (int d = 1; d < 64; d <<= 1) {
+                    const uint32_t v = (uint32_t)__shfl_up((int)incl, d);
+                    if (ln >= (uint32_t)d) incl += v;
+                }
+                const uint32_t excl = seen + incl - b.full[j];
+                hit = idx >= excl && idx < excl + b.full[j];
+                first = b.lo[j] + (idx - excl) * BM;
+                seen += (uint32_t)__shfl((int)incl, 63);
+            } else {
+                const unsigned long long m = __ballot(b.cls[j] == seg);
+                const uint32_t rank = (uint32_t)__popcll(m & ((1ull << ln) - 1ull));
+                hit = ((m >> ln) & 1ull) && seen + rank == idx;
+                first = b.lo[j] + b.full[j] * BM;
+                seen += (uint32_t)__popcll(m);
+            }
+            if (hit) {
+                out[0] = ee;
+                out[1] = first;
+                out[2] = b.hi[j];
+            }
+            found = __ballot(hit) != 0ull;
+        }
+    };
+    auto pick_segment = [&]() {   // false: tm lies past the last tile
+        if (idx < tot_full) return true;
+        idx -= tot_full;
+#pragma unroll
+        for (int k = NI; k >= 1; --k) {
+            if (idx < n_cls[k]) {
+                seg = (uint32_t)k;
+                return true;
+            }
+            idx -= n_cls[k];
+        }
+        return false;
+    };
+    Block b;
+    if (E <= 64u * JU) {
+        load(0, b);
+        count(b);
+        if (!pick_segment()) return false;
+        locate(0, b);
+    } else {
+        for (uint32_t e0 = 0; e0 < E; e0 += 64u * JU) {
+            load(e0, b);
+            count(b);
+        }
+        if (!pick_segment()) return false;
+        for (uint32_t e0 = 0; e0 < E && !found; e0 += 64u * JU) {
+            load(e0, b);
+            locate(e0, b);
+        }
+    }
+    return found;
+}
+
 // NI = 32-token tiles per workgroup tile: 4 (128 tokens, two workgroups per CU), or 2 (64 tokens,
 // three per CU) for dense launches whose 128-token tiles would leave CUs without work.
 template <class QF, int MODE, int NI>
@@ -1089,39 +1200,20 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     }
     uint32_t e = 0, row_lo = 0, row_hi = g.M;
     if (MODE != GEMM_DENSE) {
-        // Tile order over all experts: every full BM-row tile first (expert by expert), then the experts' partial last
-        // tiles, those with the most live 32-row sub-tiles first.  A tile's cost grows with its live sub-tiles, so the
-        // workgroups dispatched last are the cheapest ones and the launch does not end with a few expensive tiles
-        // running alone (list scheduling, longest first).  Wave 0 scans the per-expert counts, 64 experts at a time:
-        // pass 0 walks the full tiles, pass k the partial tiles with NI + 1 - k live sub-tiles.
-        uint32_t* s_tile = reinterpret_cast<uint32_t*>(lds_raw);   // the head of the dynamic LDS, free until the tile starts
-        const uint32_t ln = threadIdx.x & 63u;
+        // wave 0 finds the tile (find_grouped_tile) and leaves it at the head of the dynamic LDS, free until the tile starts
+        uint32_t* s_tile = reinterpret_cast<uint32_t*>(lds_raw);
         if (threadIdx.x < 64) {
-            uint32_t base = 0;
-            bool found = false;
-            for (uint32_t pass = 0; pass <= (uint32_t)NI && !found; ++pass)
-                for (uint32_t e0 = 0; e0 < g.E && !found; e0 += 64) {
-                    const uint32_t ee = e0 + ln;
-                    const uint32_t lo = ee < g.E ? g.expert_offsets[ee] : 0u, hi = ee < g.E ? g.expert_offsets[ee + 1] : 0u;
-                    const uint32_t full = (hi - lo) / BM, rem = (hi - lo) % BM;
-                    const uint32_t nt = pass == 0 ? full : ((rem && (rem + 31u) / 32u == (uint32_t)NI + 1u - pass) ? 1u : 0u);
-                    uint32_t incl = nt;
-#pragma unroll
-                    for (int d = 1; d < 64; d <<= 1) {
-                        const uint32_t v = (uint32_t)__shfl_up((int)incl, d);
-                        if (ln >= (uint32_t)d) incl += v;
-                    }
-                    const uint32_t excl = base + incl - nt;
-                    const bool hit = tm >= excl && tm < excl + nt;
-                    if (hit) {
-                        s_tile[0] = ee;
-                        s_tile[1] = lo + (pass == 0 ? tm - excl : full) * BM;
-                        s_tile[2] = hi;
-                    }
-                    found = __ballot(hit) != 0ull;
-                    base += (uint32_t)__shfl((int)incl, 63);
-                }
-            if (!found && ln == 0) s_tile[0] = 0xFFFFFFFFu;
+            uint32_t ent[3] = {0xFFFFFFFFu, 0u, 0u};
+            const bool ok = find_grouped_tile<BM, NI>(g.expert_offsets, g.E, tm, threadIdx.x & 63u, ent);
+            // the hit lane holds the entry; every other lane holds the "no tile" default
+            const unsigned long long m = __ballot(ok && ent[0] != 0xFFFFFFFFu);
+            if (m == 0ull) {
+                if (threadIdx.x == 0) s_tile[0] = 0xFFFFFFFFu;
+            } else if (ent[0] != 0xFFFFFFFFu) {
+                s_tile[0] = ent[0];
+                s_tile[1] = ent[1];
+                s_tile[2] = ent[2];
+            }
         }
         __syncthreads();
         e = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile[0]);
