@@ -302,8 +302,8 @@ int mx_gemv_q8_0_f32(mx_stream_t s, const float* A, const void* W, float* y, uin
  * as dequant_q8_0_soa_to_Bt + gemm_fp16, src/model/qwen35_dense.cpp:811-831).
  * A launch whose 128-token tiles would cover at most half of the CUs (a short batch against a narrow
  * matrix) and whose K is at least 2048 is cut into 2..8 K slices; their fp32 partial sums go through a
- * 16 MB per-device scratch array owned by the library (a file-scope device array resolved with hipGetSymbolAddress,
- * never allocated; slices * M * N <= 4 Mi floats, fewer slices beyond that) and are added in slice
+ * 32 MB per-device scratch array owned by the library (a file-scope device array resolved with hipGetSymbolAddress,
+ * never allocated; slices * M * N <= 8 Mi floats, fewer slices beyond that) and are added in slice
  * order by a second small launch: two such calls that overlap on one device race on it, as the
  * reference's static per-device scratch buffers would (src/model/dense_dispatch.hpp:547-560).  The *_ws forms
  * below keep the partial sums in the caller's workspace instead.  */

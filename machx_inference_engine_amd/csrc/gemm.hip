@@ -63,6 +63,20 @@ __device__ __forceinline__ uint32_t mix_pair(_Float16 x0, _Float16 x1, float sca
 }
 __device__ __forceinline__ half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 
+// Four int8 of a dword to four fp16 (sub-dword addressed converts with sign extension: exact, |q| <= 128), then times a
+// packed fp16 scale: half(d * q) with one rounding of the exact product, which is what rounding the fp32 product d * q
+// (exact in fp32: 11 + 8 bits) to fp16 gives.  Six instructions for four weights (bias flip, two byte permutes, four
+// mixed-precision multiply-adds and two packs before).
+__device__ __forceinline__ void q8x4_scaled(uint32_t w, uint32_t d2, uint32_t& o01, uint32_t& o23) {
+    uint32_t lo, hi;
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(lo) : "v"(w));
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1" : "+v"(lo) : "v"(w));
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(hi) : "v"(w));
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3" : "+v"(hi) : "v"(w));
+    o01 = __builtin_bit_cast(uint32_t, as_h2(lo) * as_h2(d2));
+    o23 = __builtin_bit_cast(uint32_t, as_h2(hi) * as_h2(d2));
+}
+
 union Frag {
     half8_t v;
     uint32_t u[4];
@@ -135,9 +149,8 @@ struct GemmQ4K {
 };
 
 // Q8_0 SoA planes: lane half h owns quants [128 kc + 64h, +64) of the row and the two
-// block scales.  value = half(d * q) (exact product, one RNE to fp16), computed as
-// fma((q ^ 0x80) * 2^-24, d * 2^24, -128 d): the bias-flipped byte is zero-extended into an
-// fp16 subnormal operand.
+// block scales.  value = half(d * q) (exact product, one RNE to fp16): the byte is converted to fp16
+// where it sits (q8x4_scaled) and multiplied by the fp16 scale in packed fp16.
 struct GemmQ8SoaLds;
 struct GemmQ8Soa {
     struct W {
@@ -157,7 +170,7 @@ struct GemmQ8Soa {
         uint32_t d2;
     };
     struct Dec {
-        float d[2], o[2];
+        uint32_t dh[2];   // the two block scales, each in both halves of a dword
     };
     static constexpr uint32_t K_ALIGN = 128;
     static constexpr uint32_t H_COL = 8;
@@ -172,12 +185,8 @@ struct GemmQ8Soa {
     }
     __device__ static __forceinline__ Dec dec_of(uint32_t d2) {
         Dec o;
-        o.d[0] = h2f(d2 & 0xFFFFu);
-        o.d[1] = h2f(d2 >> 16);
-        o.o[0] = -128.f * o.d[0];
-        o.o[1] = -128.f * o.d[1];
-        o.d[0] *= 16777216.f;
-        o.d[1] *= 16777216.f;
+        o.dh[0] = __builtin_amdgcn_perm(0u, d2, 0x01000100u);
+        o.dh[1] = __builtin_amdgcn_perm(0u, d2, 0x03020302u);
         return o;
     }
     __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t, uint32_t) { return dec_of(r.d2); }
@@ -185,11 +194,8 @@ struct GemmQ8Soa {
     template <int S, int HF, class RawT>
     __device__ static __forceinline__ void frag_half(const RawT& r, const Dec& dc, Frag& f) {
         constexpr int blk = S / 4, i = (S * 2) / 4, e = (S * 2) % 4;
-        const uint32_t w = (HF == 0 ? (e == 0 ? r.q[i].x : r.q[i].z) : (e == 0 ? r.q[i].y : r.q[i].w)) ^ 0x80808080u;
-        const float d = dc.d[blk], o = dc.o[blk];
-        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C030C02u));
-        f.u[2 * HF] = mix_pair(w01.x, w01.y, d, o);
-        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, d, o);
+        const uint32_t w = HF == 0 ? (e == 0 ? r.q[i].x : r.q[i].z) : (e == 0 ? r.q[i].y : r.q[i].w);
+        q8x4_scaled(w, dc.dh[blk], f.u[2 * HF], f.u[2 * HF + 1]);
     }
     template <int S, class RawT>
     __device__ static __forceinline__ void frag(const RawT& r, const Dec& dc, Frag& f) {
@@ -246,7 +252,7 @@ struct GemmQ8Aos {
         uint32_t w[17];
     };
     struct Dec {
-        float d[2], o[2];
+        uint32_t dh[2];   // the two block scales, each in both halves of a dword
     };
     static constexpr uint32_t K_ALIGN = 128;
     static constexpr uint32_t H_COL = 8;
@@ -264,12 +270,8 @@ struct GemmQ8Aos {
     }
     __device__ static __forceinline__ Dec prepare(const Raw& r, uint32_t, uint32_t) {
         Dec o;
-        o.d[0] = h2f(r.w[0] & 0xFFFFu);
-        o.d[1] = h2f(r.w[8] >> 16);
-        o.o[0] = -128.f * o.d[0];
-        o.o[1] = -128.f * o.d[1];
-        o.d[0] *= 16777216.f;
-        o.d[1] *= 16777216.f;
+        o.dh[0] = __builtin_amdgcn_perm(0u, r.w[0], 0x01000100u);
+        o.dh[1] = __builtin_amdgcn_perm(0u, r.w[8], 0x03020302u);
         return o;
     }
     template <int S, int HF>
@@ -278,11 +280,7 @@ struct GemmQ8Aos {
         uint32_t w;
         if (blk == 0) w = __builtin_amdgcn_alignbyte(r.w[j + 1], r.w[j], 2);   // bytes 2 + 4j .. 5 + 4j
         else w = r.w[9 + j];
-        w ^= 0x80808080u;
-        const float d = dc.d[blk], o = dc.o[blk];
-        const half2_t w01 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C010C00u)), w23 = as_h2(__builtin_amdgcn_perm(0u, w, 0x0C030C02u));
-        f.u[2 * HF] = mix_pair(w01.x, w01.y, d, o);
-        f.u[2 * HF + 1] = mix_pair(w23.x, w23.y, d, o);
+        q8x4_scaled(w, dc.dh[blk], f.u[2 * HF], f.u[2 * HF + 1]);
     }
     template <int S>
     __device__ static __forceinline__ void frag(const Raw& r, const Dec& dc, Frag& f) {
@@ -670,7 +668,7 @@ __device__ __forceinline__ float swiglu_oai_f(float g, float u, float alpha, flo
 // owns (no entry point allocates): one copy per device, keeping the last call's contents; every element the last
 // launch reads was written by the slices in front of it.  Launches that overlap on one device would race on it, as
 // with the reference's static per-device scratch buffers (src/model/dense_dispatch.hpp:547-560).
-constexpr uint64_t kGemmSplitElems = 4ull << 20;   // slices * M * N <= 4 Mi partial sums (16 MB)
+constexpr uint64_t kGemmSplitElems = 8ull << 20;   // slices * M * N <= 8 Mi partial sums (32 MB)
 constexpr uint32_t kGemmSplitMax = 8;
 static __device__ __align__(256) float g_gemm_splitk_acc[kGemmSplitElems];
 static std::atomic<void*> g_gemm_splitk_addr[kMaxDevices];
@@ -898,18 +896,22 @@ __device__ __forceinline__ void gemm_chunk(const TileCtx<QF, NA>& t, const uint3
 // them in the same iteration, of which there are at least 2 ceil(sizeof(Raw) / 16) (a load instruction
 // brings at most 16 bytes per lane), so waiting until at most that many loads are outstanding is enough
 // whatever the compiler made of QF::load.
-template <class QF, int MODE, bool PIPE, int NA, int DEPTH>
+// KW = 2: a workgroup of eight waves, waves 4 - 7 walking the second half of K over A buffers of their own (`lds_raw` is
+// then this half's buffer pair, `lds_red` the start of the workgroup's LDS); their sums meet the first half's in LDS
+// before the epilogue.  Both halves run the same number of chunks, so their barriers pair up.
+template <class QF, int MODE, bool PIPE, int NA, int DEPTH, int KW = 1>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::W& w0, const typename QF::W& w1, const uint32_t (&wrow)[2],
                                           uint32_t row_lo, uint32_t row_hi, uint32_t n_base, uint8_t* lds_raw, uint32_t c0 = 0,
-                                          uint32_t n_chunks_slice = 0, uint32_t ks = 0, uint32_t e = 0) {
+                                          uint32_t n_chunks_slice = 0, uint32_t ks = 0, uint32_t e = 0, uint8_t* lds_red = nullptr) {
     static_assert(DEPTH == 1 || DEPTH == 2, "prefetch depth");
+    static_assert(KW == 1 || (KW == 2 && MODE == GEMM_DENSE && NA == 4), "K halves inside a workgroup: dense full tiles only");
     static_assert(!PIPE || NA == 1 || NA == 2 || NA == 4, "the pipelined chunk is written for one, two or four token tiles");
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI;
     constexpr bool PARTIAL = MODE != GEMM_DENSE && !PIPE;
     constexpr uint32_t BM = 32u * NA;
     constexpr int NL = 2 * NA;   // 1 KB loads per wave per chunk
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 31u, h = lane >> 5;
-    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)((tid >> 6) & 3u));
     const uint32_t n_all = (g.K + kBK - 1) / kBK;                             // a row that ends half way through its last chunk counts it
     const uint32_t n_chunks = n_chunks_slice ? n_chunks_slice : n_all;       // chunks of this K slice (all of K unless split)
     const uint32_t live_rows = (row_hi - row_lo) >= BM ? BM : row_hi - row_lo;
@@ -1023,6 +1025,37 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
     }
 
 #undef CHUNK
+    if constexpr (KW == 2) {
+        // The second K half hands its sums over through LDS (32 KB per wave, the whole allocation for four waves: both
+        // halves are done with their A buffers behind the first barrier) and leaves; the first half adds them to its own.
+        typedef float f32x4_t __attribute__((ext_vector_type(4)));
+        const bool second = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 8)) != 0u;
+        f32x4_t* red = reinterpret_cast<f32x4_t*>(lds_red) + (size_t)wave * (NA * 2 * 4) * 64u + lane;
+        __syncthreads();
+        if (second) {
+#pragma unroll
+            for (int i = 0; i < NA; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int v4 = 0; v4 < 4; ++v4)
+                        red[((i * 2 + j) * 4 + v4) * 64] = f32x4_t{acc[i][j][4 * v4], acc[i][j][4 * v4 + 1], acc[i][j][4 * v4 + 2], acc[i][j][4 * v4 + 3]};
+        }
+        __syncthreads();
+        if (second) return;
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) {
+                    const f32x4_t t = red[((i * 2 + j) * 4 + v4) * 64];
+                    acc[i][j][4 * v4] += t.x;
+                    acc[i][j][4 * v4 + 1] += t.y;
+                    acc[i][j][4 * v4 + 2] += t.z;
+                    acc[i][j][4 * v4 + 3] += t.w;
+                }
+    }
     // ---- epilogue.  MFMA C layout: lane holds column n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4.
 #pragma unroll
     for (int i = 0; i < NA; ++i)
@@ -1173,8 +1206,8 @@ __device__ __forceinline__ bool find_grouped_tile(const uint32_t* expert_offsets
 
 // NI = 32-token tiles per workgroup tile: 4 (128 tokens, two workgroups per CU), or 2 (64 tokens,
 // three per CU) for dense launches whose 128-token tiles would leave CUs without work.
-template <class QF, int MODE, int NI>
-__global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
+template <class QF, int MODE, int NI, int KW = 1>
+__global__ __launch_bounds__(kGemmThreads * KW, KW == 2 ? 1 : NI == 2 ? 3 : 2) void gemm_kernel(typename QF::Bank bank0, typename QF::Bank bank1, GemmArgs g) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     constexpr uint32_t BM = 32u * NI;   // tokens per tile
     constexpr bool GATE_UP = MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI;
@@ -1227,7 +1260,7 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     const typename QF::W w0 = QF::expert(bank0, e), w1 = QF::expert(GATE_UP ? bank1 : bank0, e);
 
     const uint32_t tid = threadIdx.x, r = tid & 31u;
-    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)((tid >> 6) & 3u));
     const uint32_t n_base = tn * BN + wave * (GATE_UP ? 32 : kWaveN);
     // weight rows of the two MFMA column tiles of this wave (gate/up: same row in two matrices)
     uint32_t wrow[2];
@@ -1239,7 +1272,13 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
     if constexpr (MODE == GEMM_DENSE) {
         const uint32_t n_all = (g.K + kBK - 1) / kBK, per = (n_all + ksplit - 1) / ksplit;
         const uint32_t c0 = ks * per, c1 = (c0 + per < n_all) ? c0 + per : n_all;
-        gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, c0, c1 - c0, ks);
+        if constexpr (KW == 2) {
+            // the launcher takes this form for an even number of chunks and no K slices across workgroups
+            const uint32_t kw = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 8)), half = n_all / 2u;
+            gemm_tile<QF, MODE, true, 4, 1, 2>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw + kw * (2u * BM * kBK * 2u), kw * half, half, 0, 0, lds_raw);
+        } else {
+            gemm_tile<QF, MODE, NI == 4, NI, 1>(g, w0, w1, wrow, row_lo, row_hi, n_base, lds_raw, c0, c1 - c0, ks);
+        }
     } else {
         (void)ks;
         // expert-grouped tiles: the pipelined chunk over as many 32-token tiles as the tile's live rows need (one, two,
@@ -1271,10 +1310,10 @@ __global__ __launch_bounds__(kGemmThreads, NI == 2 ? 3 : 2) void gemm_kernel(typ
 }
 
 // ---------------------------------------------------------------- host side
-template <class QF, int MODE, int NI>
+template <class QF, int MODE, int NI, int KW = 1>
 static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const typename QF::Bank& b1, GemmArgs g, uint32_t rows_bound) {
     constexpr uint32_t BN = (MODE == GEMM_MOE_GATE_UP_SILU || MODE == GEMM_MOE_GATE_UP_OAI) ? 128 : 256, BM = 32u * NI;
-    constexpr uint32_t lds = 2u * BM * kBK * 2u + ((MODE != GEMM_DENSE && GemmLdsScales<QF>::on) ? kGemmLdsScaleBytes : 0u);
+    constexpr uint32_t lds = KW * 2u * BM * kBK * 2u + ((MODE != GEMM_DENSE && GemmLdsScales<QF>::on) ? kGemmLdsScaleBytes : 0u);
     g.tiles_n = (g.N + BN - 1) / BN;
     g.tiles_m = (MODE == GEMM_DENSE) ? (g.M + BM - 1) / BM : rows_bound / BM + g.E;   // grouped: an upper bound, workgroups past the real count leave at once
     if (MODE != GEMM_DENSE || g.k_split == 0) g.k_split = 1;
@@ -1283,7 +1322,7 @@ static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const type
     if (grid > 0x7FFFFFFFull) return MX_ERR_SHAPE;
     static bool attr_set = false;   // LDS at the 64 KB default limit: opt in once per kernel
     if (!attr_set) {
-        const hipError_t er = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<QF, MODE, NI>),
+        const hipError_t er = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<QF, MODE, NI, KW>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (er != hipSuccess) {
             g_last_hip_error = (int)er;
@@ -1291,7 +1330,7 @@ static int launch_gemm_ni(mx_stream_t s, const typename QF::Bank& b0, const type
         }
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<QF, MODE, NI>), dim3((uint32_t)grid), dim3(kGemmThreads), lds, as_stream(s), b0, b1, g);
+    hipLaunchKernelGGL((gemm_kernel<QF, MODE, NI, KW>), dim3((uint32_t)grid), dim3(kGemmThreads * KW), lds, as_stream(s), b0, b1, g);
     return launch_status();
 }
 
@@ -1338,6 +1377,11 @@ static int launch_gemm(mx_stream_t s, const typename QF::Bank& b0, const typenam
                 ni2 = true;
                 k_split = slices(tiles64);
             }
+        }
+        if (2 * tiles128 > cus && tiles128 <= cus && n_chunks % 2 == 0 && n_chunks >= 16) {
+            // One workgroup per CU would leave every SIMD with a single wave: eight-wave workgroups instead, each half of
+            // the waves walking half of K (no scratch, no second launch).  T = 512, K = 4096, N = 14336: 224 tiles.
+            return launch_gemm_ni<QF, MODE, 4, 2>(s, b0, b1, g, rows_bound);
         }
         if (k_split >= 2) {
             const uint32_t per = (uint32_t)((n_chunks + k_split - 1) / k_split);

@@ -452,3 +452,18 @@ def test_moe_grouped_gemm_q8_random_shapes(mx):
             worst = max(worst, e1, e2)
             assert e1 < 2e-3 and e2 < 2e-3, (it, E, H, EF, e, lo, hi, e1, e2)
     print("grouped q8_0 GEMM, 12 random layers: worst relative error %.2e" % worst, flush=True)
+
+
+@pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
+def test_gemm_eight_wave_workgroups(mx, fmt):
+    """Dense launches whose 128-token tiles cover between half and all of the CUs (here 2 x 70 = 140 tiles) run
+    eight-wave workgroups: waves 4 - 7 walk the second half of K and hand their sums over through LDS.  A ragged second
+    token tile, and output columns sampled across every column tile, against the oracle."""
+    M, K, N = 160, 2048, 256 * 70
+    W = weights(fmt, 2300, N, K)
+    A = f16(O.normal(2301, (M, K)))
+    fn = getattr(mx.ops, "gemm_%s" % O.FMT_NAMES[fmt])
+    got = host(fn(dev(A).half(), dev(W), M, K, N)).astype(np.float32)
+    cols = np.unique(np.concatenate([np.arange(0, 96), np.arange(N - 96, N), np.arange(0, N, 37)]))
+    ref = O.gemv_f64(fmt, np.ascontiguousarray(W[cols]), A, K, len(cols), round_w_fp16=True)
+    check(got[:, cols], ref, "gemm %s, eight-wave workgroups" % O.FMT_NAMES[fmt])
