@@ -25,7 +25,7 @@ struct GemvSeg {
 // 128 VGPRs the four-workgroups-per-CU launch wants.  Q6_K does not gain from it (12.1 -> 12.2 us on 4096 -> 14336,
 // 95.8 -> 98.5 us on the 151936-row output projection with the two alternating sets).
 template <class F>
-constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value;
+constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ8SoaW>::value || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value;
 
 // Persistent workgroups: each stages the activation tile(s) and then streams
 // its share of row groups.  With a single K-tile (every decode shape at T <= 2)
@@ -1005,6 +1005,10 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
     MX_REQUIRE_ALIGN(x, 8);
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
+    if (T == 1 && K % FmtQ8SoaW::K_ALIGN == 0) {   // one token: the interleaved unit walk (whole cache lines per load)
+        GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
+        return launch_q8<FmtQ8SoaW, half_t>(s, g, g, 1, x, K, N, 1, false, ws);
+    }
     GemvSeg<FmtQ8Soa, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
     return launch_q8<FmtQ8Soa, half_t>(s, g, g, 1, x, K, N, T, false, ws);
 }
@@ -1215,6 +1219,7 @@ int mx_gemv_q8_0_soa_q8_x2(mx_stream_t s, const void* x_q8, const int8_t* a_qs, 
     if (int rc = check_common(x_q8, y_a, K, N, 1, 32)) return rc;
     MX_REQUIRE_PTR(y_b); MX_REQUIRE_PTR(a_qs); MX_REQUIRE_PTR(a_d); MX_REQUIRE_PTR(b_qs); MX_REQUIRE_PTR(b_d);
     MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(a_qs, 16); MX_REQUIRE_ALIGN(b_qs, 16); MX_REQUIRE_ALIGN(a_d, 2); MX_REQUIRE_ALIGN(b_d, 2);
+    if (K % FmtQ8SoaW::K_ALIGN == 0) return gemv_x2<FmtQ8SoaW>(s, x_q8, {a_qs, a_d, K}, {b_qs, b_d, K}, y_a, y_b, K, N);
     return gemv_x2<FmtQ8Soa>(s, x_q8, {a_qs, a_d, K}, {b_qs, b_d, K}, y_a, y_b, K, N);
 }
 static int gemv_aos_x2(int fmt, mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
@@ -1303,6 +1308,7 @@ int mx_gemv_q8_0_soa_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const i
                              const uint16_t* u_d, uint16_t* h, uint32_t K, uint32_t N) {
     MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d);
     MX_REQUIRE_ALIGN(g_qs, 16); MX_REQUIRE_ALIGN(u_qs, 16); MX_REQUIRE_ALIGN(g_d, 2); MX_REQUIRE_ALIGN(u_d, 2);
+    if (K % FmtQ8SoaW::K_ALIGN == 0) return launch_ffn_x<FmtQ8SoaW, 2>(s, {g_qs, g_d, K}, {u_qs, u_d, K}, x, x_is_f16, h, K, N);
     return launch_ffn_x<FmtQ8Soa, 2>(s, {g_qs, g_d, K}, {u_qs, u_d, K}, x, x_is_f16, h, K, N);
 }
 static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, const void* W0, const void* W1, uint16_t* y, uint32_t K, uint32_t N) {
@@ -1334,6 +1340,7 @@ int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* q
     MX_REQUIRE_PTR(qs_W); MX_REQUIRE_PTR(d_W);
     MX_REQUIRE_ALIGN(qs_W, 16); MX_REQUIRE_ALIGN(d_W, 2);
     const FmtQ8Soa::W w{qs_W, d_W, K};
+    if (K % FmtQ8SoaW::K_ALIGN == 0) return launch_ffn_x<FmtQ8SoaW, 1>(s, w, w, x_f16, 1, y, K, N);
     return launch_ffn_x<FmtQ8Soa, 1>(s, w, w, x_f16, 1, y, K, N);
 }
 int mx_gemv_q4_K_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N) {

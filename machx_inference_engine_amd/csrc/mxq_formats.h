@@ -49,6 +49,14 @@ __device__ __forceinline__ uint32_t load_u1_a2(const uint8_t* p) {
     return reinterpret_cast<const U1*>(p)->x;
 }
 
+// A 16-byte load with the non-temporal hint, for weight words that one load instruction of a wave consumes whole cache
+// lines of (a line that several instructions touch is fetched again by each of them under this hint).
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_u4_stream(const void* p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // ---------------------------------------------------------------- Q4_K (AoS GGUF blocks)
 // Unit u = (block u/4, 64-element group g = u%4): the 32 bytes qs[32g, 32g+32),
 // whose low nibbles are sub-block 2g and high nibbles sub-block 2g+1
@@ -498,6 +506,63 @@ struct FmtQ8Soa {
         }
         o.c[0] = o.c[1] = h2f(r.d2 & 0xFFFFu);
         o.c[2] = o.c[3] = h2f(r.d2 >> 16);
+    }
+};
+
+// ---------------------------------------------------------------- Q8_0, SoA planes, interleaved units
+// The same planes, read so that one load instruction of a wave covers whole cache lines.  With units of 64 consecutive
+// bytes a lane's four 16-byte loads sit 64 bytes from its neighbour's, and the memory pipeline serves such a load at
+// about 18 bytes per clock and CU (measured on L2-resident data; 35 / 50 / 62 when two / four / eight neighbouring lanes
+// read adjacent 16-byte pieces).  Here eight consecutive units share a 512-element span of the row and unit 8 U + m
+// takes its 16-byte pieces m, m + 8, m + 16, m + 24: eight lanes read 128 contiguous bytes per load, and a line is
+// consumed by a single instruction, so the loads carry the non-temporal hint.  Group g of a unit = elements
+// 512 U + 16 m + 128 g .. + 15 = half of Q8_0 block 16 U + (m >> 1) + 4 g: four blocks, so four weight scales (picked from
+// the span's sixteen, 32 bytes that the eight lanes fetch together) and four activation scales per unit.  K % 512 == 0.
+struct FmtQ8SoaW {
+    typedef FmtQ8Soa::W W;
+    typedef FmtQ8Soa::Bank Bank;
+    __device__ static __forceinline__ W expert(const Bank& b, uint32_t e) { return FmtQ8Soa::expert(b, e); }
+    struct Cursor {
+        const uint4* qs;
+        const uint8_t* d;
+        uint32_t m;
+    };
+    struct Raw {
+        uint4 q[4];
+        uint4 d[2];   // the sixteen block scales of the span
+    };
+    static constexpr int SUM_GRAN = 0;
+    static constexpr bool PAIRED = false;
+    static constexpr uint32_t GROUP_OFF = 128;
+    static constexpr uint32_t K_ALIGN = 512;
+    static constexpr bool CODES_UNSIGNED = false;
+    __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return (u >> 3) * 512u + (u & 7u) * 16u; }
+    __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
+        return {reinterpret_cast<const uint4*>(w.qs + (size_t)n * w.K + (size_t)(u >> 3) * 512u + (u & 7u) * 16u),
+                reinterpret_cast<const uint8_t*>(w.d + (size_t)n * (w.K >> 5) + (size_t)(u >> 3) * 16u), u & 7u};
+    }
+    template <int G>
+    __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool = false) {
+        static_assert(G % 8 == 0, "a lane keeps its place in the span from step to step");
+        const uint4* p = cu.qs + (size_t)i * (G * 4);
+        const uint8_t* d = cu.d + (size_t)i * (G * 4);
+        Raw r;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) r.q[g] = load_u4_stream(p + 8 * g);
+        r.d[0] = load_u4_a2(d);
+        r.d[1] = load_u4_a2(d + 16);
+        return r;
+    }
+    __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) {
+        const bool hi = (cu.m & 4u) != 0;              // scale (m >> 1) + 4 g: word (m >> 2) + 2 g, half (m >> 1) & 1
+        const uint32_t sh = (cu.m & 2u) * 8u;
+        const uint32_t w[4] = {hi ? r.d[0].y : r.d[0].x, hi ? r.d[0].w : r.d[0].z, hi ? r.d[1].y : r.d[1].x, hi ? r.d[1].w : r.d[1].z};
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            o.q[g][0] = r.q[g].x; o.q[g][1] = r.q[g].y; o.q[g][2] = r.q[g].z; o.q[g][3] = r.q[g].w;
+            o.c[g] = h2f((w[g] >> sh) & 0xFFFFu);
+            o.m[g] = 0.f;
+        }
     }
 };
 

@@ -210,6 +210,18 @@ __device__ __forceinline__ void gemv_step(const typename F::Raw (&raw)[R], const
                 if (F::SUM_GRAN == 32) v -= un[r].m[0] * s0 + un[r].m[2] * s1;
                 acc[r][t] += v;
             }
+        } else if (F::SUM_GRAN == 0) {
+            // four groups in four activation blocks, no min term: one scale pair per group
+            float d8[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) d8[g] = reinterpret_cast<const float*>(act.hdr)[(size_t)t * (act.KT / 32) + ((e0 + g * F::GROUP_OFF) >> 5)];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float v = 0.f;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) v += un[r].c[g] * (d8[g] * (float)dot16(un[r].q[g], x[g], 0));
+                acc[r][t] += v;
+            }
         } else {
             float2 h[4];
 #pragma unroll
