@@ -581,6 +581,12 @@ template <int T, int SUM_GRAN> struct GemvShape {
     static constexpr int R = (T <= 2 || (T <= 4 && SUM_GRAN == 0)) ? 1 : 2, U = (T == 1) ? 2 : 1;
 };
 
+// Q8_0 planes, one token: rows that a wave covers in one round of loads (K <= 4096, whole 512-element spans) take the
+// interleaved unit walk (FmtQ8SoaW).  Longer rows keep the plain units: their kernels hold several rounds of units in
+// registers, and the interleaved form's cross-lane scale exchange costs them a workgroup per CU (14336 -> 4096:
+// 13.4 us plain, 15.7 - 18.4 us interleaved).
+static bool q8_soa_interleaved(uint32_t K) { return K % FmtQ8SoaW::K_ALIGN == 0 && K <= 4096u; }
+
 // lanes per row: the G in {16, 32, 64} that wastes the fewest lane slots, larger on ties
 static uint32_t pick_group(uint32_t units) {
     uint32_t best = 64, waste = (units + 63) / 64 * 64 - units;
@@ -1005,7 +1011,7 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
     MX_REQUIRE_ALIGN(x, 8);
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
-    if (T == 1 && K % FmtQ8SoaW::K_ALIGN == 0) {   // one token: the interleaved unit walk (whole cache lines per load)
+    if (T == 1 && q8_soa_interleaved(K)) {   // whole cache lines per load
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
         return launch_q8<FmtQ8SoaW, half_t>(s, g, g, 1, x, K, N, 1, false, ws);
     }
@@ -1219,7 +1225,7 @@ int mx_gemv_q8_0_soa_q8_x2(mx_stream_t s, const void* x_q8, const int8_t* a_qs, 
     if (int rc = check_common(x_q8, y_a, K, N, 1, 32)) return rc;
     MX_REQUIRE_PTR(y_b); MX_REQUIRE_PTR(a_qs); MX_REQUIRE_PTR(a_d); MX_REQUIRE_PTR(b_qs); MX_REQUIRE_PTR(b_d);
     MX_REQUIRE_ALIGN(x_q8, 8); MX_REQUIRE_ALIGN(a_qs, 16); MX_REQUIRE_ALIGN(b_qs, 16); MX_REQUIRE_ALIGN(a_d, 2); MX_REQUIRE_ALIGN(b_d, 2);
-    if (K % FmtQ8SoaW::K_ALIGN == 0) return gemv_x2<FmtQ8SoaW>(s, x_q8, {a_qs, a_d, K}, {b_qs, b_d, K}, y_a, y_b, K, N);
+    if (q8_soa_interleaved(K)) return gemv_x2<FmtQ8SoaW>(s, x_q8, {a_qs, a_d, K}, {b_qs, b_d, K}, y_a, y_b, K, N);
     return gemv_x2<FmtQ8Soa>(s, x_q8, {a_qs, a_d, K}, {b_qs, b_d, K}, y_a, y_b, K, N);
 }
 static int gemv_aos_x2(int fmt, mx_stream_t s, const void* x_q8, const void* W_a, const void* W_b, uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N) {
@@ -1308,7 +1314,7 @@ int mx_gemv_q8_0_soa_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const i
                              const uint16_t* u_d, uint16_t* h, uint32_t K, uint32_t N) {
     MX_REQUIRE_PTR(g_qs); MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d);
     MX_REQUIRE_ALIGN(g_qs, 16); MX_REQUIRE_ALIGN(u_qs, 16); MX_REQUIRE_ALIGN(g_d, 2); MX_REQUIRE_ALIGN(u_d, 2);
-    if (K % FmtQ8SoaW::K_ALIGN == 0) return launch_ffn_x<FmtQ8SoaW, 2>(s, {g_qs, g_d, K}, {u_qs, u_d, K}, x, x_is_f16, h, K, N);
+    if (q8_soa_interleaved(K)) return launch_ffn_x<FmtQ8SoaW, 2>(s, {g_qs, g_d, K}, {u_qs, u_d, K}, x, x_is_f16, h, K, N);
     return launch_ffn_x<FmtQ8Soa, 2>(s, {g_qs, g_d, K}, {u_qs, u_d, K}, x, x_is_f16, h, K, N);
 }
 static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, const void* W0, const void* W1, uint16_t* y, uint32_t K, uint32_t N) {
@@ -1340,7 +1346,7 @@ int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* q
     MX_REQUIRE_PTR(qs_W); MX_REQUIRE_PTR(d_W);
     MX_REQUIRE_ALIGN(qs_W, 16); MX_REQUIRE_ALIGN(d_W, 2);
     const FmtQ8Soa::W w{qs_W, d_W, K};
-    if (K % FmtQ8SoaW::K_ALIGN == 0) return launch_ffn_x<FmtQ8SoaW, 1>(s, w, w, x_f16, 1, y, K, N);
+    if (q8_soa_interleaved(K)) return launch_ffn_x<FmtQ8SoaW, 1>(s, w, w, x_f16, 1, y, K, N);
     return launch_ffn_x<FmtQ8Soa, 1>(s, w, w, x_f16, 1, y, K, N);
 }
 int mx_gemv_q4_K_f16q8(mx_stream_t s, const uint16_t* x_f16, const void* W, uint16_t* y, uint32_t K, uint32_t N) {

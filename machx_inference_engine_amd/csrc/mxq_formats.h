@@ -516,8 +516,8 @@ struct FmtQ8Soa {
 // read adjacent 16-byte pieces).  Here eight consecutive units share a 512-element span of the row and unit 8 U + m
 // takes its 16-byte pieces m, m + 8, m + 16, m + 24: eight lanes read 128 contiguous bytes per load, and a line is
 // consumed by a single instruction, so the loads carry the non-temporal hint.  Group g of a unit = elements
-// 512 U + 16 m + 128 g .. + 15 = half of Q8_0 block 16 U + (m >> 1) + 4 g: four blocks, so four weight scales (picked from
-// the span's sixteen, 32 bytes that the eight lanes fetch together) and four activation scales per unit.  K % 512 == 0.
+// 512 U + 16 m + 128 g .. + 15 = half of Q8_0 block 16 U + (m >> 1) + 4 g: four blocks, so four weight scales (each lane
+// loads two of the span's sixteen, the eight lanes exchange them) and four activation scales per unit.  K % 512 == 0.
 struct FmtQ8SoaW {
     typedef FmtQ8Soa::W W;
     typedef FmtQ8Soa::Bank Bank;
@@ -529,7 +529,7 @@ struct FmtQ8SoaW {
     };
     struct Raw {
         uint4 q[4];
-        uint4 d[2];   // the sixteen block scales of the span
+        uint32_t d2;   // scales 2 m, 2 m + 1 of the span's sixteen: the eight lanes of a span hold all of them
     };
     static constexpr int SUM_GRAN = 0;
     static constexpr bool PAIRED = false;
@@ -539,28 +539,29 @@ struct FmtQ8SoaW {
     __device__ static __forceinline__ uint32_t elem_off(uint32_t u) { return (u >> 3) * 512u + (u & 7u) * 16u; }
     __device__ static __forceinline__ Cursor cursor(const W& w, uint32_t n, uint32_t u) {
         return {reinterpret_cast<const uint4*>(w.qs + (size_t)n * w.K + (size_t)(u >> 3) * 512u + (u & 7u) * 16u),
-                reinterpret_cast<const uint8_t*>(w.d + (size_t)n * (w.K >> 5) + (size_t)(u >> 3) * 16u), u & 7u};
+                reinterpret_cast<const uint8_t*>(w.d + (size_t)n * (w.K >> 5) + (size_t)(u >> 3) * 16u + (u & 7u) * 2u), u & 7u};
     }
     template <int G>
     __device__ static __forceinline__ Raw load(const Cursor& cu, uint32_t i, bool = false) {
         static_assert(G % 8 == 0, "a lane keeps its place in the span from step to step");
         const uint4* p = cu.qs + (size_t)i * (G * 4);
-        const uint8_t* d = cu.d + (size_t)i * (G * 4);
         Raw r;
 #pragma unroll
         for (int g = 0; g < 4; ++g) r.q[g] = load_u4_stream(p + 8 * g);
-        r.d[0] = load_u4_a2(d);
-        r.d[1] = load_u4_a2(d + 16);
+        r.d2 = load_u1_a2(cu.d + (size_t)i * (G * 4));
         return r;
     }
+    // The lanes of a span sit in eight consecutive lanes of the wave (units 8 U .. 8 U + 7), all live or all idle together
+    // (unit counts are multiples of 8).  Group g needs scale (m >> 1) + 4 g: the dword of span lane (m >> 2) + 2 g, half
+    // (m >> 1) & 1, fetched across lanes.
     __device__ static __forceinline__ void decode(const Raw& r, const Cursor& cu, Unit& o) {
-        const bool hi = (cu.m & 4u) != 0;              // scale (m >> 1) + 4 g: word (m >> 2) + 2 g, half (m >> 1) & 1
-        const uint32_t sh = (cu.m & 2u) * 8u;
-        const uint32_t w[4] = {hi ? r.d[0].y : r.d[0].x, hi ? r.d[0].w : r.d[0].z, hi ? r.d[1].y : r.d[1].x, hi ? r.d[1].w : r.d[1].z};
+        const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        const uint32_t src = ((lane & ~7u) + (cu.m >> 2)) * 4u, sh = (cu.m & 2u) * 8u;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             o.q[g][0] = r.q[g].x; o.q[g][1] = r.q[g].y; o.q[g][2] = r.q[g].z; o.q[g][3] = r.q[g].w;
-            o.c[g] = h2f((w[g] >> sh) & 0xFFFFu);
+            const uint32_t w = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(src + 8u * g), (int)r.d2);
+            o.c[g] = h2f((w >> sh) & 0xFFFFu);
             o.m[g] = 0.f;
         }
     }
