@@ -95,6 +95,10 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / (5 * n_launch) * 1e3
 
+    def q6_planes(w, K, N):
+        """Q6_K GGUF blocks (device) -> the natural-order planes of repack_q6_K_to_soa (device), through the host repacker."""
+        return [torch.from_numpy(p).to(dev) for p in ops.repack_q6_K_to_soa(w.cpu().numpy(), K, N)]
+
     if args.shape:
         kind, T, K, N = args.shape.split(":")
         T, K, N = int(T), int(K), int(N)
@@ -107,14 +111,17 @@ def main():
                               "frac_mfma": round(2.0 * T * N * K / us / 1e6 / MFMA_PEAK, 4), "launches": 49}))
         else:
             fmt = kind[len("gemv_"):]
-            base = fmt.replace("_soa", "")
+            base = fmt.replace("_soa", "").replace("_planes", "")
             n_w = max(2, int(1.2e9 // (N * synth.row_bytes(base, K))))      # > 1 GB of weights in rotation
             wl = [synth.normal_weights(base, N, K, seed=70 + i, device=dev) for i in range(n_w)]
             if fmt.endswith("_soa"):
                 wl = [synth.split_q8_0(w) for w in wl]
             xsq = ops.quantize_q8_1(torch.randn((T, K), device=dev, generator=g).half())
             yt = torch.empty((T, N), dtype=torch.float16, device=dev)
-            if fmt.endswith("_soa"):
+            if fmt == "q6_K_planes":   # the same Q6_K bits as natural-order planes (repack_q6_K_to_soa)
+                wl = [q6_planes(w, K, N) for w in wl]
+                fn = lambda i: ops.gemv_q6_soa_q8(xsq, wl[i % n_w], K, N, T, yt)
+            elif fmt.endswith("_soa"):
                 fn = lambda i: ops.gemv_q8_0_soa_q8_batched(xsq, wl[i % n_w][0], wl[i % n_w][1], K, N, T, yt)
             else:
                 fn = lambda i: getattr(ops, "gemv_%s_q8_batched" % fmt)(xsq, wl[i % n_w], K, N, T, yt)

@@ -251,6 +251,11 @@ int mx_gemv_q6_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, con
                       const uint16_t* q6_d, uint16_t* y, uint32_t K, uint32_t N);
 int mx_gemv_q6_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi,
                               const int8_t* q6_sc, const uint16_t* q6_d, uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
+/* Two plane sets (gate and up of one FFN) against one q8 row in one launch; no counterpart in the reference (the fused
+ * gate + up form of mx_gemv_q6_K_q8_x2 for the planes of repack_q6_K_to_soa).  */
+int mx_gemv_q6_soa_q8_x2(mx_stream_t s, const void* x_q8, const uint8_t* a_lo, const uint8_t* a_hi, const int8_t* a_sc,
+                         const uint16_t* a_d, const uint8_t* b_lo, const uint8_t* b_hi, const int8_t* b_sc, const uint16_t* b_d,
+                         uint16_t* y_a, uint16_t* y_b, uint32_t K, uint32_t N);
 int mx_gemv_mxfp4_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* qs_plane, const uint8_t* e_plane,
                                  uint16_t* y, uint32_t K, uint32_t N, uint32_t T);
 /* fp32-output twins of the T = 1 int-dot kernels (no reference counterpart; for

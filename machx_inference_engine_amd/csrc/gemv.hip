@@ -1011,9 +1011,9 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
     MX_REQUIRE_ALIGN(x, 8);
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
-    if (T == 1 && q8_soa_interleaved(K)) {   // whole cache lines per load
+    if (T <= 4 && q8_soa_interleaved(K)) {   // whole cache lines per load
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
-        return launch_q8<FmtQ8SoaW, half_t>(s, g, g, 1, x, K, N, 1, false, ws);
+        return launch_q8<FmtQ8SoaW, half_t>(s, g, g, 1, x, K, N, T, false, ws);
     }
     GemvSeg<FmtQ8Soa, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
     return launch_q8<FmtQ8Soa, half_t>(s, g, g, 1, x, K, N, T, false, ws);
@@ -1103,8 +1103,31 @@ int mx_gemv_q6_soa_q8_batched(mx_stream_t s, const void* x_q8, const uint8_t* q6
     MX_REQUIRE_PTR(q6_lo); MX_REQUIRE_PTR(q6_hi); MX_REQUIRE_PTR(q6_sc); MX_REQUIRE_PTR(q6_d);
     MX_REQUIRE_ALIGN(x_q8, 8);
     MX_REQUIRE_ALIGN(q6_lo, 16); MX_REQUIRE_ALIGN(q6_hi, 16); MX_REQUIRE_ALIGN(q6_sc, 4);
+    if (T == 1) {   // one token: the plane kernel of gemv_q6_planes.hip where the shape allows
+        const int rc = launch_gemv_q6_planes(as_stream(s), 1, x_q8, &q6_lo, &q6_hi, &q6_sc, &q6_d, &y, K, N);
+        if (rc != MX_ERR_UNSUPPORTED) return rc;
+    }
     GemvSeg<FmtQ6KNat, half_t> g{{q6_lo, q6_hi, q6_sc, q6_d, K}, reinterpret_cast<half_t*>(y), nullptr};
     return launch_q8<FmtQ6KNat, half_t>(s, g, g, 1, x_q8, K, N, T);
+}
+// Two plane sets (gate and up) against one q8 row in one launch, as mx_gemv_q6_K_q8_x2 does for GGUF blocks.
+int mx_gemv_q6_soa_q8_x2(mx_stream_t s, const void* x_q8, const uint8_t* a_lo, const uint8_t* a_hi, const int8_t* a_sc, const uint16_t* a_d,
+                         const uint8_t* b_lo, const uint8_t* b_hi, const int8_t* b_sc, const uint16_t* b_d, uint16_t* y_a, uint16_t* y_b, uint32_t K,
+                         uint32_t N) {
+    if (int rc = check_common(x_q8, y_a, K, N, 1, 256)) return rc;
+    MX_REQUIRE_PTR(y_b); MX_REQUIRE_PTR(a_lo); MX_REQUIRE_PTR(a_hi); MX_REQUIRE_PTR(a_sc); MX_REQUIRE_PTR(a_d);
+    MX_REQUIRE_PTR(b_lo); MX_REQUIRE_PTR(b_hi); MX_REQUIRE_PTR(b_sc); MX_REQUIRE_PTR(b_d);
+    MX_REQUIRE_ALIGN(x_q8, 8);
+    MX_REQUIRE_ALIGN(a_lo, 16); MX_REQUIRE_ALIGN(a_hi, 16); MX_REQUIRE_ALIGN(a_sc, 4); MX_REQUIRE_ALIGN(b_lo, 16); MX_REQUIRE_ALIGN(b_hi, 16); MX_REQUIRE_ALIGN(b_sc, 4);
+    const uint8_t* lo[2] = {a_lo, b_lo};
+    const uint8_t* hi[2] = {a_hi, b_hi};
+    const int8_t* sc[2] = {a_sc, b_sc};
+    const uint16_t* d[2] = {a_d, b_d};
+    uint16_t* y[2] = {y_a, y_b};
+    const int rc = launch_gemv_q6_planes(as_stream(s), 2, x_q8, lo, hi, sc, d, y, K, N);
+    if (rc != MX_ERR_UNSUPPORTED) return rc;
+    GemvSeg<FmtQ6KNat, half_t> ga{{a_lo, a_hi, a_sc, a_d, K}, reinterpret_cast<half_t*>(y_a), nullptr}, gb{{b_lo, b_hi, b_sc, b_d, K}, reinterpret_cast<half_t*>(y_b), nullptr};
+    return launch_q8<FmtQ6KNat, half_t>(s, ga, gb, 2, x_q8, K, N, 1);
 }
 int mx_gemv_q6_soa_q8(mx_stream_t s, const void* x_q8, const uint8_t* q6_lo, const uint8_t* q6_hi, const int8_t* q6_sc, const uint16_t* q6_d,
                       uint16_t* y, uint32_t K, uint32_t N) {

@@ -59,6 +59,11 @@ inline int scratch_address(const Sym& symbol, std::atomic<void*> (&slot)[kMaxDev
     return MX_OK;
 }
 
+// gemv_q6_planes.hip: one token against one or two (gate and up) Q6_K plane sets; MX_ERR_UNSUPPORTED for a shape it
+// does not take (K % 512, K > 16384, planes of 4 GB and more, misaligned scale planes)
+int launch_gemv_q6_planes(hipStream_t st, int nseg, const void* x_q8, const uint8_t* const* lo, const uint8_t* const* hi, const int8_t* const* sc,
+                          const uint16_t* const* d, uint16_t* const* y, uint32_t K, uint32_t N);
+
 // per-device set-up of the translation units that own scratch arrays (mx_init)
 int gemv_init_device();
 int gemm_init_device();

@@ -446,10 +446,12 @@ def gemv_q4_K_down_accum(A, W, sh_g, y, K, N):
 
 
 def gemv_q8_x2(fmt, x_q8, W_a, W_b, K, N, y_a=None, y_b=None):
-    """Fused gate + up: fmt in ('q4_K', 'q6_K', 'q8_0') with W = GGUF blocks, or 'q8_0_soa' with W = (qs, d)."""
+    """Fused gate + up: fmt in ('q4_K', 'q6_K', 'q8_0') with W = GGUF blocks, 'q8_0_soa' with W = (qs, d), or 'q6_soa' with W = planes."""
     y_a, y_b = _out(y_a, (N,), torch.float16, x_q8), _out(y_b, (N,), torch.float16, x_q8)
     if fmt == "q8_0_soa":
         _call("mx_gemv_q8_0_soa_q8_x2", _u8(x_q8), _u8(W_a[0]), _ptr(W_a[1]), _u8(W_b[0]), _ptr(W_b[1]), _ptr(y_a), _ptr(y_b), K, N)
+    elif fmt == "q6_soa":   # W = (q6_lo, q6_hi, q6_sc, q6_d) from repack_q6_K_to_soa
+        _call("mx_gemv_q6_soa_q8_x2", _u8(x_q8), *[_ptr(t) for t in W_a], *[_ptr(t) for t in W_b], _ptr(y_a), _ptr(y_b), K, N)
     else:
         _call("mx_gemv_%s_q8_x2" % fmt, _u8(x_q8), _u8(W_a), _u8(W_b), _ptr(y_a), _ptr(y_b), K, N)
     return y_a, y_b

@@ -88,7 +88,17 @@ def test_gemv_q8_0_soa_matches_aos(mx):
     soa4 = host(mx.ops.gemv_q8_0_soa_q8_batched(dev(xq), dev(qs), dev(d), K, N, 4)).astype(np.float32)
     check(soa4, ref, "gemv_q8_0_soa_q8_batched")
     aos4 = run_q8(mx, O.Q8_0, W, xq, K, N, 4)
-    assert np.array_equal(aos4, soa4)   # same arithmetic, only the addresses differ
+    check(aos4, ref, "gemv_q8_0_q8_batched (GGUF blocks)")
+    # the same products; planes and blocks are walked in different orders, so the fp32 sums differ in their last bits
+    assert np.mean(aos4 == soa4) > 0.95 and np.abs(aos4 - soa4).max() <= 2e-3 * np.abs(ref).max()
+    # a K outside the interleaved walk's reach (not a multiple of 512) takes the plain unit walk: the same bits as the blocks
+    K2 = 4096 + 64
+    W2 = weights(O.Q8_0, 602, N, K2)
+    xq2 = O.quantize_q8_1(acts(603, 2, K2))
+    qs2, d2 = O.repack_q8_0_to_soa(W2)
+    soa2 = host(mx.ops.gemv_q8_0_soa_q8_batched(dev(xq2), dev(qs2), dev(d2), K2, N, 2)).astype(np.float32)
+    check(soa2, O.gemv_q8chain(O.Q8_0, W2, xq2, K2, N), "gemv_q8_0_soa_q8_batched, K = %d" % K2)
+    assert np.array_equal(run_q8(mx, O.Q8_0, W2, xq2, K2, N, 2), soa2)
 
 
 def test_gemv_mxfp4_x2_bias(mx):

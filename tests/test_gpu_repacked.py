@@ -32,7 +32,7 @@ def test_gemv_q4_K_reorder_and_soa(mx, K, N):
 
 
 @pytest.mark.parametrize("T", (1, 2, 4, 8, 16))
-@pytest.mark.parametrize("K,N", [(256, 5), (2048, 130), (14336, 64)])
+@pytest.mark.parametrize("K,N", [(256, 5), (2048, 130), (4096, 300), (14336, 64)])
 def test_gemv_q6_soa(mx, K, N, T):
     """gemv_q6_soa_q8 / _batched (src/ops/gemv_q6_soa.cpp:137-407): natural-order bit planes; the partial
     sums group differently from the AoS kernel, so the gate is the q8-chain oracle."""
@@ -44,6 +44,13 @@ def test_gemv_q6_soa(mx, K, N, T):
     ref = O.gemv_q8chain(O.Q6_K, W, xq, K, N)
     for t in range(T):
         check(y[t], ref[t], "gemv_q6_soa_q8 K=%d N=%d T=%d row %d" % (K, N, T, t))
+    if T == 1:
+        # two plane sets in one launch: each half equals the single launch bit for bit
+        W2 = weights(O.Q6_K, 2150 + K, N, K)
+        planes2 = [dev(p) for p in ops.repack_q6_K_to_soa(W2, K, N)]
+        ya, yb = ops.gemv_q8_x2("q6_soa", dev(xq), planes, planes2, K, N)
+        assert np.array_equal(host(ya).astype(np.float32), y[0])
+        check(host(yb).astype(np.float32), O.gemv_q8chain(O.Q6_K, W2, xq, K, N)[0], "gemv_q6_soa_q8_x2 second matrix K=%d N=%d" % (K, N))
 
 
 @pytest.mark.parametrize("K,N", [(256, 3), (1024, 70), (2880 // 32 * 32 + 256 - 2880 % 256, 9)])
