@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--shape", default=None, metavar="KIND:T:K:N",
                     help="profiling aid: only launches of one kernel at one shape (KIND in gemm_q4_K, gemv_q8_0_soa, gemv_q6_K, gemv_q4_K), "
                          "so that a rocprofv3 run holds exactly one (kernel, shape) pair; prints its HIP-event average")
+    ap.add_argument("--yardstick", action="store_true",
+                    help="read-only yardsticks of the device, as text: cold reads of the dominant launches' byte counts by launch shape, "
+                         "and the per-CU rate of 16-byte loads by lane -> address pattern (cache-resident)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures one GPU only (the path is data-parallel over output rows / experts, "
@@ -98,6 +101,42 @@ def main():
     def q6_planes(w, K, N):
         """Q6_K GGUF blocks (device) -> the natural-order planes of repack_q6_K_to_soa (device), through the host repacker."""
         return [torch.from_numpy(p).to(dev) for p in ops.repack_q6_K_to_soa(w.cpu().numpy(), K, N)]
+
+    if args.yardstick:
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        for n_bytes, what in ((124843008 // 1024 * 1024, "the fused Q8_0 gate + up launch"), (62390272 // 1024 * 1024, "one Q8_0 4096 -> 14336 matrix"),
+                              (48200192 // 1024 * 1024, "one Q6_K 4096 -> 14336 matrix")):
+            n_buf = max(2, (1200 << 20) // n_bytes)
+            bufs = [torch.empty(n_bytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(n_buf)]
+            print("cold read of %d bytes (%s), %d rotating buffers, %d CUs; cells: us per launch / TB/s" % (n_bytes, what, n_buf, cus))
+            print("%-46s" % "variant \\ workgroups per CU" + "".join("%12d" % w for w in (2, 3, 4, 6, 8)))
+            rows = [("registers, %2d x 16 B in flight per thread" % u, u, 0) for u in (2, 4, 8, 16)]
+            rows += [("registers, %2d x 16 B, nontemporal" % u, u, 1) for u in (4, 8)]
+            rows += [("LDS ring, %2d x 1 KB in flight per wave" % d, d, 2) for d in (4, 8, 16)]
+            for name, u, mode in rows:
+                cells = []
+                for w in (2, 3, 4, 6, 8):
+                    us = kernel_avg_us(lambda i: ops.probe_read_variant(bufs[i % n_buf], u, mode, cus * w), 2 * n_buf)
+                    cells.append("%6.1f/%5.2f" % (us, n_bytes / us / 1e6))
+                print("%-46s" % name + "".join(cells))
+            cells = []
+            for u in (4, 8, 16):   # not persistent: every workgroup reads one contiguous piece of u * 4 KB and leaves
+                us = kernel_avg_us(lambda i: ops.probe_read_variant(bufs[i % n_buf], u, 0, n_bytes // (u * 4096)), 2 * n_buf)
+                cells.append("%6.1f/%5.2f" % (us, n_bytes / us / 1e6))
+            print("%-46s" % "one 16 / 32 / 64 KB piece per workgroup" + "".join(cells))
+            print()
+            del bufs
+        pitch, rows_, iters, wgs = 2048, 4096, 20, 2 * cus
+        region = torch.empty(rows_ * pitch + 16, dtype=torch.uint8, device=dev).random_(0, 255)
+        print("16-byte-per-lane loads over a cache-resident region (%d rows of %d B), %d workgroups of 4 waves, %d passes" % (rows_, pitch, wgs, iters))
+        names = ("one row per lane: 16 contiguous bytes", "2 adjacent lanes: 32 contiguous bytes", "4 adjacent lanes: 64 contiguous bytes",
+                 "8 adjacent lanes: one 128-byte line", "128-byte line, pieces 2-byte aligned", "128-byte line, pieces 4-byte aligned",
+                 "128-byte line, pieces 8-byte aligned")
+        b = wgs * 4 * 64 * pitch * iters
+        t = [kernel_avg_us(lambda i: ops.probe_lane_pattern(region, pitch, pat, iters, wgs), 4) for pat in range(len(names))]
+        for name, us in zip(names, t):
+            print("%-42s %8.1f us  %6.2f TB/s  %5.1f B/us/CU  %4.2f of the whole-line rate" % (name, us, b / us / 1e6, b / cus / us, t[3] / us))
+        return
 
     if args.shape:
         kind, T, K, N = args.shape.split(":")

@@ -56,6 +56,16 @@ int mx_init(void);
  * launch geometry of the decode GEMV and no arithmetic, so that a GEMV launch can be priced against a pure read of
  * the same bytes on the same device.  `sink` may be NULL (a word that is practically never written).  */
 int mx_probe_stream_read(mx_stream_t s, const void* src, uint64_t n_bytes, uint32_t* sink);
+/* Measurement aids, no counterpart in the reference.  mx_probe_read_variant reads n_bytes (a multiple of 1024, 16-byte
+ * aligned) once with `workgroups` workgroups of 256 threads that stride over the buffer: `in_flight` 16-byte loads per
+ * thread (2, 4, 8, 16) with mode 0 (plain) or 1 (nontemporal), or mode 2: `in_flight` (4, 8, 16) loads of 1 KB per wave
+ * straight into LDS.  mx_probe_lane_pattern reads a region (region_bytes incl. 16 spare bytes at its end, rows of
+ * `pitch` bytes, pitch % 128 == 0) `iters` times with 16-byte loads whose lanes cover 16 (pattern 0), 32 (1), 64 (2) or
+ * 128 (3) contiguous bytes per row, or 128 bytes displaced by 2, 4, 8 bytes (4, 5, 6); each workgroup moves
+ * 4 * 64 * pitch * iters bytes.  Both are timed by the caller with events on `s`.  */
+int mx_probe_read_variant(mx_stream_t s, const void* src, uint64_t n_bytes, int in_flight, int mode, uint32_t workgroups, uint32_t* sink);
+int mx_probe_lane_pattern(mx_stream_t s, const void* region, uint64_t region_bytes, uint32_t pitch, int pattern, uint32_t iters,
+                          uint32_t workgroups, uint32_t* sink);
 
 /* ---------------------------------------------------------------- activation quantizers
  * quantize_q8_1   include/ie/ops.hpp:301-304, src/ops/gemv_q8dot.cpp:94-124

@@ -83,6 +83,17 @@ def probe_stream_read(buf, n_bytes=None):
     _call("mx_probe_stream_read", _ptr(buf), n, None)
 
 
+def probe_read_variant(buf, in_flight, mode, workgroups, n_bytes=None):
+    """One read of `buf` with a chosen launch shape (mode 0 plain / 1 nontemporal register loads, 2 loads into LDS)."""
+    n = buf.numel() * buf.element_size() if n_bytes is None else n_bytes
+    _call("mx_probe_read_variant", _ptr(buf), n, in_flight, mode, workgroups, None)
+
+
+def probe_lane_pattern(region, pitch, pattern, iters, workgroups):
+    """16-byte-per-lane loads over `region` (uint8, 16 spare bytes at its end) under lane -> address pattern 0..6."""
+    _call("mx_probe_lane_pattern", _ptr(region), region.numel() * region.element_size(), pitch, pattern, iters, workgroups, None)
+
+
 # ---------------------------------------------------------------- dequant
 def dequant(fmt, packed, n_elements, out=None, dtype=torch.float16):
     out = _out(out, (n_elements,), dtype, packed)
