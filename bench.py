@@ -150,6 +150,8 @@ def main():
                               "frac_mfma": round(2.0 * T * N * K / us / 1e6 / MFMA_PEAK, 4), "launches": 49}))
         else:
             fmt = kind[len("gemv_"):]
+            x2 = fmt.endswith("_x2")     # two matrices sharing the activation row in one launch (gate + up), T = 1
+            fmt = fmt[:-3] if x2 else fmt
             base = fmt.replace("_soa", "").replace("_planes", "")
             n_w = max(2, int(1.2e9 // (N * synth.row_bytes(base, K))))      # > 1 GB of weights in rotation
             wl = [synth.normal_weights(base, N, K, seed=70 + i, device=dev) for i in range(n_w)]
@@ -164,8 +166,13 @@ def main():
                 fn = lambda i: ops.gemv_q8_0_soa_q8_batched(xsq, wl[i % n_w][0], wl[i % n_w][1], K, N, T, yt)
             else:
                 fn = lambda i: getattr(ops, "gemv_%s_q8_batched" % fmt)(xsq, wl[i % n_w], K, N, T, yt)
+            if x2:
+                assert T == 1
+                yt2 = torch.empty((T, N), dtype=torch.float16, device=dev)
+                kind2 = {"q6_K_planes": "q6_soa", "q8_0_soa": "q8_0_soa"}.get(fmt, fmt)
+                fn = lambda i: ops.gemv_q8_x2(kind2, xsq, wl[i % n_w], wl[(i + 1) % n_w], K, N, yt, yt2)
             us = kernel_avg_us(fn, 2 * n_w)
-            b = gemv_bytes(synth.row_bytes(base, K), K, N, T)
+            b = gemv_bytes(synth.row_bytes(base, K), K, N, T) * (2 if x2 else 1)
             print(json.dumps({"shape": args.shape, "avg_launch_us": round(us, 2), "GBps": round(b / us / 1e3, 1),
                               "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4), "launches": 12 * n_w + 1}))
         return

@@ -47,8 +47,12 @@ __device__ __forceinline__ float swiglu_oai(float g, float u, float alpha, float
 }
 
 // NW = weight rows per output element (2: gate and up, 1: down); R outputs per lane group.
+// One-token launches of formats with small units (MXFP4: 36 bytes) request whole rows ahead (see below) and are held to
+// three resident waves per SIMD, which a decode launch of a few hundred workgroups needs to be resident at once.
+template <class F, int TT>
+constexpr bool kMoeWholeRow = TT == 1 && sizeof(typename F::Raw) <= 40;
 template <class F, int TT, int NW, int R, int G, int U, int EPI>
-__global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank bank0, typename F::Bank bank1, MoeArgs a) {
+__global__ __launch_bounds__(kGemvThreads, (TT == 1 && sizeof(typename F::Raw) <= 40) ? 3 : 1) void moe_gemv_kernel(typename F::Bank bank0, typename F::Bank bank1, MoeArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int GROUPS = 64 / G;
     constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
@@ -96,6 +100,55 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
                     cu[NW * r] = F::cursor(w0, n, k0 / 64 + gl);
                     if (NW == 2) cu[NW * r + 1] = F::cursor(w1, n, k0 / 64 + gl);
                 }
+                const uint32_t n_units = (kt + 63) / 64;
+                const bool half_tail = (kt & 63u) != 0;
+                if (kMoeWholeRow<F, TT> && n_tiles == 1 && !staged && !half_tail && n_units <= 3u * G) {
+                    // A workgroup of a decode launch lives for one row group.  The whole of its rows (up to three rounds
+                    // of units) is requested right behind the activation loads and in front of the barrier, so the launch
+                    // is one round trip to memory and the first round is summed while the later ones arrive.  Lanes
+                    // past the end of the row read their first unit again and drop the product.
+                    // (two rounds there and the third once the first is summed for gate + up: six units in flight per lane
+                    // would cost a resident wave per SIMD)
+                    constexpr int AHEAD = (NW == 2) ? 2 : 3;
+                    typename F::Raw pre[3][NW * R];
+                    auto request = [&]() {
+#pragma unroll
+                        for (int u = 0; u < AHEAD; ++u) {
+                            const bool lv = u * G + gl < n_units;
+#pragma unroll
+                            for (int r = 0; r < NW * R; ++r) pre[u][r] = load_unit<F, G>(cu[r], lv ? u : 0, false);
+                        }
+                    };
+                    if (a.act_f16) {
+                        auto hrow = [&](uint32_t t) { return a.act_f16 + (size_t)((t0 + (t < nt ? t : nt - 1)) / a.act_div) * K; };
+                        act = stage_act_f16<F::SUM_GRAN, TT>(lds, hrow, k0, kt, KT, request);
+                    } else {
+                        act = stage_act<F::SUM_GRAN, TT>(lds, xrow, k0, kt, KT, a.q8_split != 0, request);
+                    }
+                    __syncthreads();
+                    staged = true;
+#pragma unroll
+                    for (int u = 0; u < 3; ++u) {
+                        if (u > 0 && u - 1 + AHEAD < 3) {   // a round that was not requested ahead takes the registers of a summed one
+                            const bool lq = (u - 1 + AHEAD) * G + gl < n_units;
+#pragma unroll
+                            for (int r = 0; r < NW * R; ++r) pre[u - 1 + AHEAD][r] = load_unit<F, G>(cu[r], lq ? u - 1 + AHEAD : 0, false);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        const bool lv = u * G + gl < n_units;
+                        float part[NW * R][TT];
+#pragma unroll
+                        for (int r = 0; r < NW * R; ++r)
+#pragma unroll
+                            for (int t = 0; t < TT; ++t) part[r][t] = 0.f;
+                        gemv_step<F, TT, NW * R>(pre[u], cu, lv ? gl + u * G : gl, act, part);
+#pragma unroll
+                        for (int r = 0; r < NW * R; ++r)
+#pragma unroll
+                            for (int t = 0; t < TT; ++t) acc[r][t] += lv ? part[r][t] : 0.f;
+                    }
+                    continue;
+                }
                 if (n_tiles > 1 || !staged) {
                     __syncthreads();
                     if (a.act_f16) {
@@ -107,7 +160,7 @@ __global__ __launch_bounds__(kGemvThreads) void moe_gemv_kernel(typename F::Bank
                     __syncthreads();
                     staged = true;
                 }
-                gemv_rows<F, TT, NW * R, G, U>(cu, (kt + 63) / 64, (kt & 63u) != 0, gl, act, acc);
+                gemv_rows<F, TT, NW * R, G, U>(cu, n_units, half_tail, gl, act, acc);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r)

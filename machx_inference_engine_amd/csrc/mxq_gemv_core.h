@@ -114,12 +114,13 @@ __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t 
 // s = d * float(sum q) per 32-element block, exactly quantize_q8_1 (src/ops/gemv_q8dot.cpp:94-124), so the
 // staged tile is bit-identical to staging the quantizer's output.  A thread takes 16 elements; the two
 // threads of a block (adjacent lanes) exchange their maxima and sums.  `hrow(t)` -> first element of row t.
-template <int SUM_GRAN, int T, class RowFn>
-__device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc) {
+template <int SUM_GRAN, int T, class RowFn, class Hook = NoHook>
+__device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc, Hook between = Hook()) {
     uint4* qs = reinterpret_cast<uint4*>(lds);
     uint8_t* hdr = lds + (size_t)T * KT_alloc;
     const uint32_t halves = (kt + 63) / 64 * 4;
     const uint32_t total = (uint32_t)T * halves, total_up = (total + blockDim.x - 1) / blockDim.x * blockDim.x;
+    bool hooked = false;
     for (uint32_t i = threadIdx.x; i < total_up; i += blockDim.x) {   // whole passes: both threads of a block stay converged
         const bool in = i < total;
         const uint32_t t = in ? i / halves : 0, hb = in ? i - t * halves : 0;
@@ -127,9 +128,18 @@ __device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint3
         float v[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) v[j] = 0.f;
+        uint4 a = make_uint4(0, 0, 0, 0), b = a;
         if (live) {
             const half_t* p = hrow(t) + k0 + hb * 16;
-            const uint4 a = reinterpret_cast<const uint4*>(p)[0], b = reinterpret_cast<const uint4*>(p)[1];
+            a = reinterpret_cast<const uint4*>(p)[0];
+            b = reinterpret_cast<const uint4*>(p)[1];
+        }
+        if (!hooked) {   // as in stage_act: behind the first pass's activation loads, in front of their use
+            between();
+            __builtin_amdgcn_sched_barrier(0);
+            hooked = true;
+        }
+        if (live) {
             const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
