@@ -33,6 +33,23 @@ H, FF = 4096, 14336
 Q81X = 40
 
 
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "pmc_traffic_gemv_q8_0_soa_and_gemm_q4_K.txt")
+
+
+def counter_traffic(key):
+    """HBM bytes per launch (read + written) of one kernel from the tracked counter summary: its line
+    `traffic_bytes <key> read=<bytes> written=<bytes>` (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a
+    plain copy of known size; the file names the commit and the commands).  None when the file or the key is absent."""
+    try:
+        for line in open(TRAFFIC_FILE):
+            f = line.split()
+            if len(f) == 4 and f[0] == "traffic_bytes" and f[1] == key:
+                return int(f[2].split("=")[1]) + int(f[3].split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
 def gemv_bytes(fmt_row_bytes, K, N, T):
     """Algorithmic bytes of one GEMV launch: weights once, q8 activations, fp16 outputs."""
     return N * fmt_row_bytes + T * (K // 32) * Q81X + T * N * 2
@@ -282,12 +299,12 @@ def main():
         dom_us = kernel_avg_us(lambda i: ops.gemv_q8_0_soa_q8(xq, mats[i % len(mats)][0], mats[i % len(mats)][1], H, FF, y_ff[("q8_0", "gate")]),
                                4 * len(mats))
         dom_bytes = gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1)
-        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> K=4096 N=14336", 62483456 + 114790
+        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8SoaW,T=1> K=4096 N=14336", counter_traffic("gemv_q8_0_soa_T1_K4096_N14336")
     else:
         # the fused gate + up launch: two 4096 -> 14336 matrices, one activation row, two output rows
         dom_us = kernel_avg_us(lambda i: gate_up("q8_0", sets[i % len(sets)]), 4 * len(sets))
         dom_bytes = 2 * gemv_bytes(synth.row_bytes("q8_0", H), H, FF, 1) - (H // 32) * 40
-        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8Soa,T=1> gate+up fused, K=4096 N=2x14336", 125019703 + 230809
+        dom_name, dom_traffic = "gemv_q8_kernel<FmtQ8SoaW,T=1> gate+up fused, K=4096 N=2x14336", counter_traffic("gemv_q8_0_soa_gate_up_fused_T1")
     # yardstick: a pure read of the same number of bytes with the same launch geometry (rotating buffers, no arithmetic)
     n_read = (dom_bytes + 15) // 16 * 16
     rd = [torch.empty(n_read, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(8)]
@@ -296,7 +313,7 @@ def main():
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt)
+                # read from profiles/pmc_traffic_*.txt (counter run of `bench.py --probe`), not measured in this run
                 "traffic": dom_traffic,
                 "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 3),
                 # not part of the fraction above: what a read-only kernel reaches on the same bytes on this device
@@ -314,9 +331,8 @@ def main():
     roofline_gemm = {"bound": "mfma", "kernel": "gemm_kernel<GemmQ4K, dense, 128-token tiles> T=2048 K=4096 N=14336 (v_mfma_f32_32x32x16_f16)",
                      "achieved": round(gemm_tf, 1), "peak": MFMA_PEAK, "unit": "TFLOP/s", "frac": round(gemm_tf / MFMA_PEAK, 4),
                      "flop_per_launch": gemm_flop, "avg_launch_us": round(gemm_us, 2),
-                     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/pmc_traffic_*.txt);
-                     # algorithmic bytes: W 33,030,144 + A 16,777,216 + Y 58,720,256
-                     "traffic": 254396345 + 58720358, "algorithmic_bytes": Ng * synth.row_bytes("q4_K", Kg) + Tg * Kg * 2 + Tg * Ng * 2}
+                     # read from profiles/pmc_traffic_*.txt; algorithmic bytes: W 33,030,144 + A 16,777,216 + Y 58,720,256
+                     "traffic": counter_traffic("gemm_q4_K_T2048_K4096_N14336"), "algorithmic_bytes": Ng * synth.row_bytes("q4_K", Kg) + Tg * Kg * 2 + Tg * Ng * 2}
     del wq, a16, yg
 
     out = {"metric": "quant GEMV HBM GB/s (decode, Llama-3-8B FFN shapes, Q6_K + Q8_0, batch 1)", "value": round(value, 1),
@@ -358,6 +374,15 @@ def main():
                             us_c = kernel_avg_us(lambda i: fn(xsq, ws_l[0], K, N, T, yt), 24)
                             detail["%s_%s_T1_cache_resident" % (fmt, name)] = {"us": round(us_c, 2), "GBps": round(b / us_c / 1e3, 1)}
                     del ws_l
+            # Q6_K as natural-order planes (repack_q6_K_to_soa, the reference's gemv_q6_soa_q8 layout), one token
+            for name, (K, N) in (("gate_up", (H, FF)), ("down", (FF, H))):
+                pl = [q6_planes(synth.normal_weights("q6_K", N, K, seed=177 + i, device=dev), K, N) for i in range(6)]   # 289 MB in rotation
+                xsq = ops.quantize_q8_1(torch.randn((1, K), device=dev, generator=g).half())
+                yt = torch.empty((1, N), dtype=torch.float16, device=dev)
+                us = kernel_avg_us(lambda i: ops.gemv_q6_soa_q8(xsq, pl[i % len(pl)], K, N, 1, yt), 6 * len(pl))
+                b = gemv_bytes(synth.row_bytes("q6_K", K), K, N, 1)
+                detail["q6_K_planes_%s_T1" % name] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
+                del pl
         if want('ffn'):
             # one decode FFN (fp16 x in, fp16 y out) as the reference's launch chain and as the two fused launches
             xf = torch.randn(H, device=dev, generator=g).half()
@@ -421,6 +446,12 @@ def main():
                         ent["vendor_fp16_gemm_us"] = round(us_g, 1)
                         ent["vendor_fp16_gemm_TFLOPs"] = round(2.0 * T * N * K / us_g / 1e6, 1)
                         ent["dequant_plus_vendor_gemm_us"] = round(us_2, 1)
+                        if T == 2048:   # the library's own tiled fp16 kernel (mx_gemm_fp16, fp32 out) on the same operands
+                            y32 = torch.empty((T, N), dtype=torch.float32, device=dev)
+                            us_t = kernel_avg_us(lambda i: ops.gemm_fp16(a16, bt, T, N, K, torch.float32, y32), 4)
+                            ent["tiled_fp16_gemm_f32out_us"] = round(us_t, 1)
+                            ent["tiled_fp16_gemm_TFLOPs"] = round(2.0 * T * N * K / us_t / 1e6, 1)
+                            del y32
                         del bt
                     if T == 2048:
                         # the int-dot route over q8 rows (int8 matrix cores, fp32 fold per 32-element block): rows quantized once, outside the timing
