@@ -578,7 +578,7 @@ constexpr uint32_t kWgsPerCu = 4;    // persistent grid: workgroups per CU
 // token; batched, two rows share each activation read once the per-token work dominates
 // (T > 4, or T > 2 for the formats whose fold carries a min term), one row below that
 template <int T, int SUM_GRAN> struct GemvShape {
-    static constexpr int R = (T <= 2 || (T <= 4 && SUM_GRAN == 0)) ? 1 : 2, U = (T == 1) ? 2 : 1;
+    static constexpr int R = (T <= 2 || (T <= 4 && (SUM_GRAN == 0 || SUM_GRAN == 2))) ? 1 : 2, U = (T == 1) ? 2 : 1;
 };
 
 // Q8_0 planes, one token: rows that a wave covers in one round of loads (K <= 4096, whole 512-element spans) take the
@@ -604,7 +604,7 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     // N = 14336 18.1 -> 15.8 us; K = 14336, N = 4096 18.1 -> 16.6 us)
     constexpr int R = GemvShape<T, F::SUM_GRAN>::R, U = std::is_same<F, FmtQ8Aos>::value ? 1 : GemvShape<T, F::SUM_GRAN>::U;
     constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
-    const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);   // LDS bytes per 32 activation elements
+    const uint32_t per_elem_x32 = qs_bytes_per32(F::SUM_GRAN) + hdr_bytes_per32(F::SUM_GRAN);   // LDS bytes per 32 activation elements
     const uint32_t KT_max = (kLdsBudget / (per_elem_x32 * T)) * 32 / 256 * 256;
     if (KT_max == 0) return MX_ERR_SHAPE;
     const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
@@ -919,7 +919,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_ffn_kernel(typename F::W
 
 template <class F, int NW, bool XF16>
 static int launch_ffn(mx_stream_t s, const typename F::W& w0, const typename F::W& w1, const void* x, uint16_t* y, uint32_t K, uint32_t N) {
-    const uint32_t per_elem_x32 = 32 + hdr_bytes_per32(F::SUM_GRAN);
+    const uint32_t per_elem_x32 = qs_bytes_per32(F::SUM_GRAN) + hdr_bytes_per32(F::SUM_GRAN);
     const uint32_t KT = (K + 255) / 256 * 256;
     if ((uint64_t)KT / 32 * per_elem_x32 > kLdsBudget) return MX_ERR_SHAPE;   // the activation row has to fit one LDS tile
     const uint32_t G = pick_group((K + 63) / 64);

@@ -47,12 +47,13 @@ __device__ __forceinline__ float swiglu_oai(float g, float u, float alpha, float
 }
 
 // NW = weight rows per output element (2: gate and up, 1: down); R outputs per lane group.
-// One-token launches of formats with small units (MXFP4: 36 bytes) request whole rows ahead (see below) and are held to
-// three resident waves per SIMD, which a decode launch of a few hundred workgroups needs to be resident at once.
-template <class F, int TT>
-constexpr bool kMoeWholeRow = TT == 1 && sizeof(typename F::Raw) <= 40;
+// One-token down launches of MXFP4 (36-byte units, decoded by the convert instruction) request whole rows ahead (see below) and are
+// held to three resident waves per SIMD, which a decode launch of a few hundred workgroups needs to be resident at once.  (gate + up
+// the same way spills: 21 against 12 us.)
+template <class F, int TT, int NW>
+constexpr bool kMoeWholeRow = TT == 1 && NW == 1 && F::SUM_GRAN == 2;
 template <class F, int TT, int NW, int R, int G, int U, int EPI>
-__global__ __launch_bounds__(kGemvThreads, (TT == 1 && sizeof(typename F::Raw) <= 40) ? 3 : 1) void moe_gemv_kernel(typename F::Bank bank0, typename F::Bank bank1, MoeArgs a) {
+__global__ __launch_bounds__(kGemvThreads, (TT == 1 && NW == 1 && F::SUM_GRAN == 2) ? 3 : 1) void moe_gemv_kernel(typename F::Bank bank0, typename F::Bank bank1, MoeArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int GROUPS = 64 / G;
     constexpr int ROWS_PER_WG = kGemvWaves * GROUPS * R;
@@ -102,14 +103,12 @@ __global__ __launch_bounds__(kGemvThreads, (TT == 1 && sizeof(typename F::Raw) <
                 }
                 const uint32_t n_units = (kt + 63) / 64;
                 const bool half_tail = (kt & 63u) != 0;
-                if (kMoeWholeRow<F, TT> && n_tiles == 1 && !staged && !half_tail && n_units <= 3u * G) {
+                if (kMoeWholeRow<F, TT, NW> && n_tiles == 1 && !staged && !half_tail && n_units <= 3u * G) {
                     // A workgroup of a decode launch lives for one row group.  The whole of its rows (up to three rounds
                     // of units) is requested right behind the activation loads and in front of the barrier, so the launch
                     // is one round trip to memory and the first round is summed while the later ones arrive.  Lanes
                     // past the end of the row read their first unit again and drop the product.
-                    // (two rounds there and the third once the first is summed for gate + up: six units in flight per lane
-                    // would cost a resident wave per SIMD)
-                    constexpr int AHEAD = (NW == 2) ? 2 : 3;
+                    constexpr int AHEAD = 3;
                     typename F::Raw pre[3][NW * R];
                     auto request = [&]() {
 #pragma unroll
@@ -357,7 +356,7 @@ static int launch_moe_tg(hipStream_t st, const typename F::Bank& b0, const typen
     constexpr int R = (NW == 2 || TT == 1) ? 1 : 2;
     constexpr int U = (TT == 1) ? 2 : 1;
     constexpr uint32_t rows_per_wg = kGemvWaves * (64 / G) * R;
-    const uint32_t per32 = 32 + hdr_bytes_per32(F::SUM_GRAN);
+    const uint32_t per32 = qs_bytes_per32(F::SUM_GRAN) + hdr_bytes_per32(F::SUM_GRAN);
     const uint32_t KT_max = (kMoeLdsBudget / (per32 * TT)) * 32 / 256 * 256;
     if (KT_max == 0) return MX_ERR_SHAPE;
     const uint32_t K256 = (a.K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;

@@ -805,7 +805,7 @@ struct FmtMxfp4Soa {
         uint4 qa, qb;
         uint32_t e2;
     };
-    static constexpr int SUM_GRAN = 0;
+    static constexpr int SUM_GRAN = 2;   // int-dot GEMVs: fp16-pair activations, codes converted by the FP4 convert instruction (fp4())
     static constexpr bool PAIRED = true;
     static constexpr uint32_t GROUP_OFF = 16;
     static constexpr uint32_t K_ALIGN = 32;
@@ -830,6 +830,14 @@ struct FmtMxfp4Soa {
         }
         return r;
     }
+    // the unit as the convert instruction takes it: eight code words (two blocks) and the two half-scaled block scales
+    __device__ static __forceinline__ void fp4(const Raw& r, uint32_t (&w)[8], float (&c)[2]) {
+        w[0] = r.qa.x; w[1] = r.qa.y; w[2] = r.qa.z; w[3] = r.qa.w;
+        w[4] = r.qb.x; w[5] = r.qb.y; w[6] = r.qb.z; w[7] = r.qb.w;
+        c[0] = e8m0_half(r.e2 & 0xFFu);
+        c[1] = e8m0_half(r.e2 >> 8);
+    }
+    // doubled E2M1 values as int8 (the float-activation GEMV)
     __device__ static __forceinline__ void decode(const Raw& r, const Cursor&, Unit& o) {
         mxfp4_decode_word(r.qa.x, o.q[0][0], o.q[1][0]);
         mxfp4_decode_word(r.qa.y, o.q[0][1], o.q[1][1]);

@@ -27,9 +27,11 @@ constexpr int kGemvWaves = kGemvThreads / 64;
 //   SUM_GRAN 0  : float  d8                       (4 B / 32)
 //   SUM_GRAN 32 : float2 {d8, d8*sum32}           (8 B / 32)
 //   SUM_GRAN 16 : float2 {d8, d8*sum16} per 16    (16 B / 32)
-__host__ __device__ constexpr uint32_t hdr_bytes_per32(int sum_gran) { return sum_gran == 0 ? 4 : (sum_gran == 32 ? 8 : 16); }
+//   SUM_GRAN 2  : float  d8; the quants of this layout are fp16 (MXFP4, see stage_act)   (4 B / 32)
+__host__ __device__ constexpr uint32_t hdr_bytes_per32(int sum_gran) { return (sum_gran == 0 || sum_gran == 2) ? 4 : (sum_gran == 32 ? 8 : 16); }
+__host__ __device__ constexpr uint32_t qs_bytes_per32(int sum_gran) { return sum_gran == 2 ? 64 : 32; }
 __host__ __device__ constexpr uint32_t act_tile_bytes(uint32_t T, uint32_t KT, int sum_gran) {
-    return T * (KT + KT / 32 * hdr_bytes_per32(sum_gran));
+    return T * (KT / 32) * (qs_bytes_per32(sum_gran) + hdr_bytes_per32(sum_gran));
 }
 
 struct ActTile {
@@ -42,8 +44,24 @@ struct ActTile {
 // apart (units of consecutive elements) and the 16 lanes one ds_read_b128 pass serves would share four bank groups; the
 // XOR spreads them over all sixteen.  Units of consecutive elements (every format but Q6_K) permute the four chunks inside
 // a unit; Q6_K's units interleave two 128-element halves (K is a multiple of 256 there), so the bits one up are used.
+// SUM_GRAN 2 (fp16 quants, 128 B per unit): eight chunks per unit, permuted by the bits above the pair of units that
+// shares a 256-byte bank row.
 template <int SUM_GRAN>
-__device__ __forceinline__ uint32_t act_slot(uint32_t q) { return q ^ (((q >> 4) & 3u) << (SUM_GRAN == 16 ? 1 : 0)); }
+__device__ __forceinline__ uint32_t act_slot(uint32_t q) {
+    if (SUM_GRAN == 2) return q ^ ((q >> 4) & 7u);
+    return q ^ (((q >> 4) & 3u) << (SUM_GRAN == 16 ? 1 : 0));
+}
+
+// Four int8 of `lo` and of `hi` -> four fp16 pairs {half(lo[b]), half(hi[b])} (exact: |q| <= 127).
+__device__ __forceinline__ uint4 q8_pairs_f16(uint32_t lo, uint32_t hi) {
+    uint32_t o[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const half_t l = (half_t)(int)(int8_t)(lo >> (8 * b)), h = (half_t)(int)(int8_t)(hi >> (8 * b));
+        o[b] = (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
 
 // Stage T q8_1 rows, elements [k0, k0+kt), into LDS.  `xrow(t)` -> pointer to
 // the first block of activation row t.  All threads of the block call this.
@@ -62,6 +80,37 @@ template <int SUM_GRAN, int T, class RowFn, class Hook = NoHook>
 __device__ __forceinline__ ActTile stage_act(uint8_t* lds, RowFn xrow, uint32_t k0, uint32_t kt, uint32_t KT_alloc, bool split = false,
                                              Hook between = Hook()) {
     uint4* qs = reinterpret_cast<uint4*>(lds);
+    if constexpr (SUM_GRAN == 2) {
+        // MXFP4: the matching weights are converted by v_cvt_scalef32_pk_f16_fp4, one byte (elements j and j + 16 of a
+        // block) -> one fp16 pair, and summed by v_dot2_f32_f16; so the quants are staged as fp16 pairs
+        // {x[j], x[j + 16]}, j = 0..15 per block (four 16-byte chunks), exact integers.
+        uint8_t* hdr2 = lds + (size_t)T * KT_alloc * 2;
+        const uint32_t blocks = (kt + 63) / 64 * 2;   // padded to whole 64-element units with zeros
+        bool hooked2 = false;
+        for (uint32_t i = threadIdx.x; i < (uint32_t)T * blocks; i += blockDim.x) {
+            const uint32_t t = i / blocks, b = i - t * blocks;
+            uint2 q[4] = {make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0), make_uint2(0, 0)};
+            float d = 0.f;
+            if (b * 32 < kt) {
+                const uint8_t* blk = xrow(t) + (size_t)(k0 / 32 + b) * (split ? kQ81sBytes : kQ81xBytes);
+                const uint2* p = reinterpret_cast<const uint2*>(blk + (split ? 16 : 8));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) q[j] = p[j];
+                d = *reinterpret_cast<const float*>(blk);
+            }
+            if (!hooked2) {
+                between();
+                __builtin_amdgcn_sched_barrier(0);
+                hooked2 = true;
+            }
+            const uint32_t lo[4] = {q[0].x, q[0].y, q[1].x, q[1].y}, hi[4] = {q[2].x, q[2].y, q[3].x, q[3].y};
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) qs[(size_t)t * (KT_alloc / 8) + act_slot<2>(4u * b + c)] = q8_pairs_f16(lo[c], hi[c]);
+            reinterpret_cast<float*>(hdr2)[(size_t)t * (KT_alloc / 32) + b] = d;
+        }
+        if (!hooked2) between();
+        return ActTile{qs, hdr2, KT_alloc};
+    }
     uint8_t* hdr = lds + (size_t)T * KT_alloc;
     const uint32_t halves = (kt + 63) / 64 * 4;   // padded to whole 64-element units with zeros
     bool hooked = false;
@@ -166,6 +215,21 @@ __device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint3
             q[j] = pk;
         }
         const int s32 = s16 + __shfl_xor(s16, 1);
+        if constexpr (SUM_GRAN == 2) {
+            // fp16 pairs {x[j], x[j + 16]}: the other half of the block sits in the neighbouring lane; the thread of the
+            // first half writes pairs 0..7, the other one pairs 8..15
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (uint32_t)__shfl_xor((int)q[j], 1);
+            if (!in) continue;
+            const bool second = (hb & 1u) != 0;
+            const uint32_t b = hb >> 1, c0 = second ? 2u : 0u;
+            uint4* row = qs + (size_t)t * (KT_alloc / 8);
+            row[act_slot<2>(4u * b + c0)] = second ? q8_pairs_f16(o[2], q[2]) : q8_pairs_f16(q[0], o[0]);
+            row[act_slot<2>(4u * b + c0 + 1u)] = second ? q8_pairs_f16(o[3], q[3]) : q8_pairs_f16(q[1], o[1]);
+            if (!second) reinterpret_cast<float*>(lds + (size_t)T * KT_alloc * 2)[(size_t)t * (KT_alloc / 32) + b] = d;
+            continue;
+        }
         if (!in) continue;
         qs[(size_t)t * (KT_alloc / 16) + act_slot<SUM_GRAN>(hb)] = make_uint4(q[0], q[1], q[2], q[3]);
         if (SUM_GRAN == 16) {
@@ -177,6 +241,7 @@ __device__ __forceinline__ ActTile stage_act_f16(uint8_t* lds, RowFn hrow, uint3
                 reinterpret_cast<float*>(hdr)[(size_t)t * (KT_alloc / 32) + (hb >> 1)] = d;
         }
     }
+    if constexpr (SUM_GRAN == 2) return ActTile{qs, lds + (size_t)T * KT_alloc * 2, KT_alloc};
     return ActTile{qs, hdr, KT_alloc};
 }
 
@@ -192,6 +257,42 @@ __device__ __forceinline__ int dot16(const uint32_t (&w)[4], const uint4& x, int
 template <class F, int T, int R>
 __device__ __forceinline__ void gemv_step(const typename F::Raw (&raw)[R], const typename F::Cursor (&cu)[R], uint32_t ul,
                                           const ActTile& act, float (&acc)[R][T]) {
+    if constexpr (F::SUM_GRAN == 2) {
+        // MXFP4 against fp16-pair activations: one v_cvt_scalef32_pk_f16_fp4 per weight byte (scale 2: the doubled E2M1
+        // values 0..12, integers) and one v_dot2_f32_f16 per pair.  Every product and partial sum is an integer below
+        // 2^24, so the fp32 sum equals the int8 dot of the other formats exactly and the fold is the same expression.
+        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+        const uint32_t e0 = F::elem_off(ul);
+        uint32_t w[R][8];
+        float c[R][2];
+#pragma unroll
+        for (int r = 0; r < R; ++r) F::fp4(raw[r], w[r], c[r]);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            uint4 x[8];
+#pragma unroll
+            for (uint32_t k = 0; k < 8; ++k) x[k] = act.qs[(size_t)t * (act.KT / 8) + act_slot<2>((e0 >> 3) + k)];
+            const float* h = reinterpret_cast<const float*>(act.hdr) + (size_t)t * (act.KT / 32) + (e0 >> 5);
+            const float d0 = h[0], d1 = h[1];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float f[2] = {0.f, 0.f};
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t ww = w[r][4 * b + k];
+                        const uint4& xx = x[4 * b + k];
+                        f[b] = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(ww, 2.0f, 0), __builtin_bit_cast(h2_t, xx.x), f[b], false);
+                        f[b] = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(ww, 2.0f, 1), __builtin_bit_cast(h2_t, xx.y), f[b], false);
+                        f[b] = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(ww, 2.0f, 2), __builtin_bit_cast(h2_t, xx.z), f[b], false);
+                        f[b] = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(ww, 2.0f, 3), __builtin_bit_cast(h2_t, xx.w), f[b], false);
+                    }
+                acc[r][t] += c[r][0] * (d0 * f[0]) + c[r][1] * (d1 * f[1]);
+            }
+        }
+        return;
+    }
     Unit un[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) F::decode(raw[r], cu[r], un[r]);
@@ -363,7 +464,7 @@ __device__ __forceinline__ float fact_unit(const typename F::Raw& raw, const typ
                   x.z * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 2) + x.w * code_to_f<F::CODES_UNSIGNED>(un.q[g][i], 3);
         }
         v += un.c[g] * dq;
-        if (F::SUM_GRAN != 0) v -= un.m[g] * s16[eg >> 4];
+        if (F::SUM_GRAN != 0 && F::SUM_GRAN != 2) v -= un.m[g] * s16[eg >> 4];
     }
     return v;
 }
