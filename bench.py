@@ -68,7 +68,7 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for `rocprofv3 --pmc`: a few launches of the dominant kernels and of a plain copy of known size, no timing")
     ap.add_argument("--legs", default="all",
-                    help="comma-separated detail legs to run (batched, ffn, c1, lm_head, c3, c4, c5); with a list the headline legs are skipped "
+                    help="comma-separated detail legs to run (batched, gaps, ffn, c1, lm_head, c3, c4, c5); with a list the headline legs are skipped "
                          "and only the detail table is printed (development aid)")
     ap.add_argument("--shape", default=None, metavar="KIND:T:K:N",
                     help="profiling aid: only launches of one kernel at one shape (KIND in gemm_q4_K, gemv_q8_0_soa, gemv_q6_K, gemv_q4_K), "
@@ -383,6 +383,39 @@ def main():
                 b = gemv_bytes(synth.row_bytes("q6_K", K), K, N, 1)
                 detail["q6_K_planes_%s_T1" % name] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac_hbm": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
                 del pl
+        if want('gaps') and graphs:
+            # What the dependencies between the four launches of a step cost: the same step recorded with the Q6_K chain and
+            # the Q8_0 chain as two independent branches of the graph (gate + up -> down inside each), so that the tail of one
+            # launch overlaps the ramp of another.  Not the headline (a decode step of one model is one chain).
+            s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+            def step_branches(ws):
+                cur = torch.cuda.current_stream()
+                for st_, fmt in ((s1, "q6_K"), (s2, "q8_0")):
+                    st_.wait_stream(cur)
+                    with torch.cuda.stream(st_):
+                        gate_up(fmt, ws)
+                        gemv(fmt, hq, ws, "down", FF, H, y_h[fmt])
+                cur.wait_stream(s1)
+                cur.wait_stream(s2)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            gb = []
+            for ws in sets:
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    step_branches(ws)
+                gb.append(gr)
+            res = {}
+            for name, gl in (("one_chain", graphs), ("two_independent_chains", gb)):
+                for gr in gl:
+                    gr.replay()
+                torch.cuda.synchronize()
+                e0.record()
+                for i in range(40):
+                    gl[i % len(gl)].replay()
+                e1.record()
+                torch.cuda.synchronize()
+                res[name + "_us"] = round(e0.elapsed_time(e1) / 40 * 1e3, 2)
+            detail["step_launch_dependencies"] = res
         if want('ffn'):
             # one decode FFN (fp16 x in, fp16 y out) as the reference's launch chain and as the two fused launches
             xf = torch.randn(H, device=dev, generator=g).half()
