@@ -582,9 +582,10 @@ template <int T, int SUM_GRAN> struct GemvShape {
 };
 
 // Q8_0 planes, one token: rows that a wave covers in one round of loads (K <= 4096, whole 512-element spans) take the
-// interleaved unit walk (FmtQ8SoaW).  Longer rows keep the plain units: their kernels hold several rounds of units in
-// registers, and the interleaved form's cross-lane scale exchange costs them a workgroup per CU (14336 -> 4096:
-// 13.4 us plain, 15.7 - 18.4 us interleaved).
+// interleaved unit walk (FmtQ8SoaW).  Longer rows keep the plain units in the lane-group kernels: those hold several
+// rounds of units in registers, and the interleaved form's cross-lane scale exchange costs them a workgroup per CU
+// (14336 -> 4096: 13.4 us plain, 15.7 - 18.4 us interleaved); long rows of a short matrix take the interleaved units
+// in the workgroup-wide walk instead (gemv_q8_0_soa_batched).
 static bool q8_soa_interleaved(uint32_t K) { return K % FmtQ8SoaW::K_ALIGN == 0 && K <= 4096u; }
 
 // lanes per row: the G in {16, 32, 64} that wastes the fewest lane slots, larger on ties
@@ -1011,6 +1012,17 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
     MX_REQUIRE_ALIGN(x, 8);
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
+    if (T == 1 && K % FmtQ8SoaW::K_ALIGN == 0 && K >= 8192 && K <= 64u * kGemvThreads && N <= 16u * (uint32_t)cu_count()) {
+        // Long rows, few of them (the 14336 -> 4096 down projections): the workgroup-wide row walk with interleaved units.
+        // A row is one round of whole-line nontemporal loads of the whole workgroup (224 of 256 threads at K = 14336) and
+        // one round trip, and a short matrix still gives every CU four workgroups.  Measured against the two-round
+        // rotation of the plain units (gemv_q8_deep_kernel): 13.9 -> 12.1 us; two rows per pass 12.2 - 12.9 us.
+        GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
+        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * kWgsPerCu;
+        hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
+                           act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN), as_stream(s), g, g, static_cast<const uint8_t*>(x), K, N, KT, 1u, 0u);
+        return launch_status();
+    }
     if (T <= 4 && q8_soa_interleaved(K)) {   // whole cache lines per load
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
         return launch_q8<FmtQ8SoaW, half_t>(s, g, g, 1, x, K, N, T, false, ws);
