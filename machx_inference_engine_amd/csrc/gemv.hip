@@ -1012,15 +1012,22 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
     MX_REQUIRE_ALIGN(x, 8);
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
-    if (T == 1 && K % FmtQ8SoaW::K_ALIGN == 0 && K >= 8192 && K <= 64u * kGemvThreads && N <= 16u * (uint32_t)cu_count()) {
+    if (T <= 2 && K % FmtQ8SoaW::K_ALIGN == 0 && K >= 8192 && K <= 64u * kGemvThreads && N <= 16u * (uint32_t)cu_count()) {
         // Long rows, few of them (the 14336 -> 4096 down projections): the workgroup-wide row walk with interleaved units.
         // A row is one round of whole-line nontemporal loads of the whole workgroup (224 of 256 threads at K = 14336) and
-        // one round trip, and a short matrix still gives every CU four workgroups.  Measured against the two-round
-        // rotation of the plain units (gemv_q8_deep_kernel): 13.9 -> 12.1 us; two rows per pass 12.2 - 12.9 us.
+        // one round trip, and a short matrix still gives every CU its workgroups.  Measured against the two-round
+        // rotation of the plain units (gemv_q8_deep_kernel): 13.9 -> 12.1 us (two rows per pass: 12.2 - 12.9 us); two
+        // tokens against the lane-group walk: 15.7 -> 13.9 us.
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
-        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * kWgsPerCu;
-        hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
-                           act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN), as_stream(s), g, g, static_cast<const uint8_t*>(x), K, N, KT, 1u, 0u);
+        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * (T == 1 ? kWgsPerCu : 3u);
+        const dim3 gridw(N < capw ? N : capw, 1);
+        const uint8_t* xq = static_cast<const uint8_t*>(x);
+        if (T == 1)
+            hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN),
+                               as_stream(s), g, g, xq, K, N, KT, 1u, 0u);
+        else
+            hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 2, 1, half_t>), gridw, dim3(kGemvThreads), act_tile_bytes(2, KT, FmtQ8SoaW::SUM_GRAN),
+                               as_stream(s), g, g, xq, K, N, KT, 2u, 0u);
         return launch_status();
     }
     if (T <= 4 && q8_soa_interleaved(K)) {   // whole cache lines per load

@@ -42,17 +42,19 @@ struct Q6pRaw {
     uint32_t s01, s23, d2;
 };
 
-__global__ __launch_bounds__(kGemvThreads, 4) void gemv_q6_planes_kernel(Q6pSeg seg0, Q6pSeg seg1, const uint8_t* xq8, uint32_t K, uint32_t N) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    const Q6pSeg& seg = blockIdx.y ? seg1 : seg0;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, m = lane & 7u;
-    const uint32_t n_chunks = K / 16u;
-    uint4* x_lo = reinterpret_cast<uint4*>(lds);                 // [K/16] chunks, elements (0 2 4 6 | 1 3 5 7 | 8 10 12 14 | 9 11 13 15)
-    uint4* x_hi = x_lo + n_chunks;                               // [K/16] chunks, elements (0 4 8 12 | 1 5 9 13 | 2 6 10 14 | 3 7 11 15)
-    uint2* x_hd = reinterpret_cast<uint2*>(x_hi + n_chunks);     // [K/16] {d8 bits, sum of the 16 q8}
+struct Q6pTile {
+    const uint4* x_lo;   // [K/16] chunks, elements (0 2 4 6 | 1 3 5 7 | 8 10 12 14 | 9 11 13 15)
+    const uint4* x_hi;   // [K/16] chunks, elements (0 4 8 12 | 1 5 9 13 | 2 6 10 14 | 3 7 11 15)
+    const uint2* x_hd;   // [K/16] {d8 bits, sum of the 16 q8}
+};
 
-    // ---- stage the q8 row (block_q8_1x: {float d, float s, int8 qs[32]}, 40 bytes per 32 elements), one 16-chunk per thread and pass
-    for (uint32_t c = tid; c < n_chunks; c += kGemvThreads) {
+// Stage the q8 row (block_q8_1x: {float d, float s, int8 qs[32]}, 40 bytes per 32 elements), one 16-chunk per thread and pass.
+__device__ __forceinline__ Q6pTile q6p_stage(uint8_t* lds, const uint8_t* xq8, uint32_t K) {
+    const uint32_t n_chunks = K / 16u;
+    uint4* x_lo = reinterpret_cast<uint4*>(lds);
+    uint4* x_hi = x_lo + n_chunks;
+    uint2* x_hd = reinterpret_cast<uint2*>(x_hi + n_chunks);
+    for (uint32_t c = threadIdx.x; c < n_chunks; c += kGemvThreads) {
         const uint8_t* blk = xq8 + (size_t)(c >> 1) * kQ81xBytes;
         const uint2* q = reinterpret_cast<const uint2*>(blk + 8 + (c & 1u) * 16u);
         const uint2 qa = q[0], qb = q[1];
@@ -71,52 +73,66 @@ __global__ __launch_bounds__(kGemvThreads, 4) void gemv_q6_planes_kernel(Q6pSeg 
                               __builtin_amdgcn_perm(p3, p1, 0x05040100u), __builtin_amdgcn_perm(p3, p1, 0x07060302u));
         x_hd[at] = make_uint2(d8, (uint32_t)sum);
     }
+    return Q6pTile{x_lo, x_hi, x_hd};
+}
+
+// Unit u of row `row`: lane m = u & 7 of span u >> 3.
+__device__ __forceinline__ void q6p_request(Q6pRaw& r, const Q6pSeg& seg, uint32_t row, uint32_t u, uint32_t K) {
+    const uint32_t U = u >> 3, m = u & 7u;
+    const uint8_t* lo = seg.lo + (size_t)row * (K >> 1) + U * 256u + m * 16u;
+    const uint8_t* hi = seg.hi + (size_t)row * (K >> 2) + U * 128u + m * 8u;
+    const uint8_t* sc = seg.sc + (size_t)row * (K >> 4) + U * 32u + m * 2u;
+    r.l0 = load_u4_stream(lo);
+    r.l1 = load_u4_stream(lo + 128);
+    r.h0 = *reinterpret_cast<const uint2*>(hi);
+    r.h1 = *reinterpret_cast<const uint2*>(hi + 64);
+    r.s01 = *reinterpret_cast<const uint16_t*>(sc);
+    r.s23 = *reinterpret_cast<const uint16_t*>(sc + 16);
+    r.d2 = *reinterpret_cast<const uint32_t*>(seg.d + (size_t)row * ((K >> 8) * 2u) + U * 4u);
+}
+
+__device__ __forceinline__ float q6p_consume(const Q6pRaw& r, const Q6pTile& x, uint32_t u) {
+    const uint32_t c0 = (u >> 3) * 32u + 2u * (u & 7u);   // first chunk of the lane's 32 elements in the span's first half
+    const uint32_t lw[8] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w, r.l1.x, r.l1.y, r.l1.z, r.l1.w};
+    const uint32_t hw[4] = {r.h0.x, r.h0.y, r.h1.x, r.h1.y};
+    const uint32_t sc[4] = {r.s01 & 0xFFu, r.s01 >> 8, r.s23 & 0xFFu, r.s23 >> 8};
+    const float dsb[2] = {h2f(r.d2 & 0xFFFFu), h2f(r.d2 >> 16)};
+    float acc = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t at = q6p_slot(c0 + (uint32_t)((g & 1) + (g >> 1) * 16));
+        const uint4 xl = x.x_lo[at], xh = x.x_hi[at];
+        const uint2 hd = x.x_hd[at];
+        const uint32_t w0 = lw[2 * g], w1 = lw[2 * g + 1], h = hw[g];
+        int ih = dot4(h & 0x03030303u, xh.x, 0);
+        ih = dot4((h >> 2) & 0x03030303u, xh.y, ih);
+        ih = dot4((h >> 4) & 0x03030303u, xh.z, ih);
+        ih = dot4((h >> 6) & 0x03030303u, xh.w, ih);
+        int il = dot4(w0 & 0x0F0F0F0Fu, xl.x, ih * 16 - 32 * (int)hd.y);
+        il = dot4((w0 >> 4) & 0x0F0F0F0Fu, xl.y, il);
+        il = dot4(w1 & 0x0F0F0F0Fu, xl.z, il);
+        il = dot4((w1 >> 4) & 0x0F0F0F0Fu, xl.w, il);
+        acc += (dsb[g >> 1] * (float)(int)(int8_t)sc[g]) * (u2f(hd.x) * (float)il);
+    }
+    return acc;
+}
+
+__global__ __launch_bounds__(kGemvThreads, 4) void gemv_q6_planes_kernel(Q6pSeg seg0, Q6pSeg seg1, const uint8_t* xq8, uint32_t K, uint32_t N) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const Q6pSeg& seg = blockIdx.y ? seg1 : seg0;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const Q6pTile xt = q6p_stage(lds, xq8, K);
 
     // ---- rows of this wave, rounds of 64 units per row
     const uint32_t n_units = K / 64u, rounds = (n_units + 63u) / 64u;
     const uint32_t wave_id = blockIdx.x * kGemvWaves + (tid >> 6), n_waves = gridDim.x * kGemvWaves;
-    const uint32_t lo_pitch = K >> 1, hi_pitch = K >> 2, sc_pitch = K >> 4, d_pitch = (K >> 8) * 2u;
     auto request = [&](Q6pRaw& r, uint32_t row, uint32_t round) {
         const uint32_t u = round * 64u + lane;
-        if (row < N && u < n_units) {
-            const uint32_t U = u >> 3;
-            const uint8_t* lo = seg.lo + (size_t)row * lo_pitch + U * 256u + m * 16u;
-            const uint8_t* hi = seg.hi + (size_t)row * hi_pitch + U * 128u + m * 8u;
-            const uint8_t* sc = seg.sc + (size_t)row * sc_pitch + U * 32u + m * 2u;
-            r.l0 = load_u4_stream(lo);
-            r.l1 = load_u4_stream(lo + 128);
-            r.h0 = *reinterpret_cast<const uint2*>(hi);
-            r.h1 = *reinterpret_cast<const uint2*>(hi + 64);
-            r.s01 = *reinterpret_cast<const uint16_t*>(sc);
-            r.s23 = *reinterpret_cast<const uint16_t*>(sc + 16);
-            r.d2 = *reinterpret_cast<const uint32_t*>(seg.d + (size_t)row * d_pitch + U * 4u);
-        }
+        if (row < N && u < n_units) q6p_request(r, seg, row, u, K);
     };
     auto consume = [&](const Q6pRaw& r, uint32_t row, uint32_t round, float& acc) {
         const uint32_t u = round * 64u + lane;
-        if (row < N && u < n_units) {
-            const uint32_t c0 = (u >> 3) * 32u + 2u * m;   // first chunk of the lane's 32 elements in the span's first half
-            const uint32_t lw[8] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w, r.l1.x, r.l1.y, r.l1.z, r.l1.w};
-            const uint32_t hw[4] = {r.h0.x, r.h0.y, r.h1.x, r.h1.y};
-            const uint32_t sc[4] = {r.s01 & 0xFFu, r.s01 >> 8, r.s23 & 0xFFu, r.s23 >> 8};
-            const float dsb[2] = {h2f(r.d2 & 0xFFFFu), h2f(r.d2 >> 16)};
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const uint32_t at = q6p_slot(c0 + (uint32_t)((g & 1) + (g >> 1) * 16));
-                const uint4 xl = x_lo[at], xh = x_hi[at];
-                const uint2 hd = x_hd[at];
-                const uint32_t w0 = lw[2 * g], w1 = lw[2 * g + 1], h = hw[g];
-                int ih = dot4(h & 0x03030303u, xh.x, 0);
-                ih = dot4((h >> 2) & 0x03030303u, xh.y, ih);
-                ih = dot4((h >> 4) & 0x03030303u, xh.z, ih);
-                ih = dot4((h >> 6) & 0x03030303u, xh.w, ih);
-                int il = dot4(w0 & 0x0F0F0F0Fu, xl.x, ih * 16 - 32 * (int)hd.y);
-                il = dot4((w0 >> 4) & 0x0F0F0F0Fu, xl.y, il);
-                il = dot4(w1 & 0x0F0F0F0Fu, xl.z, il);
-                il = dot4((w1 >> 4) & 0x0F0F0F0Fu, xl.w, il);
-                acc += (dsb[g >> 1] * (float)(int)(int8_t)sc[g]) * (u2f(hd.x) * (float)il);
-            }
-        }
+        if (row < N && u < n_units) acc += q6p_consume(r, xt, u);
     };
     auto finish = [&](uint32_t row, float acc) {
         const float v = group_sum<64>(acc);
@@ -125,7 +141,8 @@ __global__ __launch_bounds__(kGemvThreads, 4) void gemv_q6_planes_kernel(Q6pSeg 
 
     // item = (row, round).  Two register sets take turns (the loop is unrolled over them, so no set is ever copied: a
     // copy would wait for its load): one item is in flight while the other is summed.  Four sets, three items in flight,
-    // measured slower (4096 -> 14336: 12.0 -> 13.8 us).  The first item is requested before the barrier behind the staging.
+    // measured slower (4096 -> 14336: 12.0 -> 13.8 us), and so did a workgroup-wide walk of long rows (thread t takes unit t,
+    // one round per row: 14336 -> 4096 13.6 us either way).  The first item is requested before the barrier behind the staging.
     struct Item {
         uint32_t row, round;
     };
