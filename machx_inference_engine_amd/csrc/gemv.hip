@@ -227,7 +227,14 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, O
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const size_t q8_row_bytes = (size_t)(K / 32) * (q8_split ? kQ81sBytes : kQ81xBytes);
     auto xrow = [&](uint32_t t) { return xq8 + (size_t)(t < T_real ? t : T_real - 1) * q8_row_bytes; };
-    const ActTile act = stage_act<F::SUM_GRAN, T>(lds, xrow, 0, K, KT, q8_split != 0);
+    // q8_split == 2: `xq8` is one fp16 row, quantized while it is staged (T = 1; the same tile as staging quantize_q8_1's output)
+    ActTile act;
+    if (T == 1 && q8_split == 2u) {
+        auto hrow = [&](uint32_t) { return reinterpret_cast<const half_t*>(xq8); };
+        act = stage_act_f16<F::SUM_GRAN, T>(lds, hrow, 0, K, KT);
+    } else {
+        act = stage_act<F::SUM_GRAN, T>(lds, xrow, 0, K, KT, q8_split != 0);
+    }
     __syncthreads();
     const uint32_t n_units = (K + 63) / 64, n_rg = (N + R - 1) / R;
     const bool half_tail = (K & 63u) != 0;
@@ -588,6 +595,11 @@ template <int T, int SUM_GRAN> struct GemvShape {
 // in the workgroup-wide walk instead (gemv_q8_0_soa_batched).
 static bool q8_soa_interleaved(uint32_t K) { return K % FmtQ8SoaW::K_ALIGN == 0 && K <= 4096u; }
 
+// long rows of a short matrix (one round of the whole workgroup per row): see gemv_q8_0_soa_batched
+static bool q8_soa_wide(uint32_t K, uint32_t N) {
+    return K % FmtQ8SoaW::K_ALIGN == 0 && K >= 8192u && K <= 64u * (uint32_t)kGemvThreads && N <= 16u * (uint32_t)cu_count();
+}
+
 // lanes per row: the G in {16, 32, 64} that wastes the fewest lane slots, larger on ties
 static uint32_t pick_group(uint32_t units) {
     uint32_t best = 64, waste = (units + 63) / 64 * 64 - units;
@@ -614,6 +626,7 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     if constexpr (T == 1 && F::SUM_GRAN == 16) {
         // long rows, too few of them to give every CU its workgroups: the workgroup-wide row walk.  Measured at
         // K = 14336, N = 4096: Q6_K 14.4 -> 12.7 us; no gain for the formats with 64-byte units or for T = 2.
+        // (mx_gemv_q6_K_f16q8 takes the same launch under the same condition, so that both forms give the same bits.)
         if (n_tiles == 1 && K >= 8192 && n_rg <= 2u * (uint32_t)cu_count()) {
             const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu / nseg;
             dim3 gridw(N < capw ? N : capw, nseg);
@@ -1012,7 +1025,7 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
     MX_REQUIRE_ALIGN(x, 8);
     MX_REQUIRE_ALIGN(qs_W, 16);
     MX_REQUIRE_ALIGN(d_W, 2);
-    if (T <= 2 && K % FmtQ8SoaW::K_ALIGN == 0 && K >= 8192 && K <= 64u * kGemvThreads && N <= 16u * (uint32_t)cu_count()) {
+    if (T <= 2 && q8_soa_wide(K, N)) {
         // Long rows, few of them (the 14336 -> 4096 down projections): the workgroup-wide row walk with interleaved units.
         // A row is one round of whole-line nontemporal loads of the whole workgroup (224 of 256 threads at K = 14336) and
         // one round trip, and a short matrix still gives every CU its workgroups.  Measured against the two-round
@@ -1370,6 +1383,19 @@ static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, 
     }
     if (fmt == 2) {
         const FmtQ6K::W wa{a, K / 256 * (uint32_t)kQ6KBytes}, wb{b, K / 256 * (uint32_t)kQ6KBytes};
+        // the single GEMV on a long row of a short matrix: the workgroup-wide walk, as mx_gemv_q6_K_q8 takes it
+        // (launch_q8_tg: one K tile, K >= 8192, at most two row groups of eight rows per CU)
+        const uint32_t KT = (K + 255) / 256 * 256;
+        if (nw == 1 && x_is_f16 && K >= 8192 && act_tile_bytes(1, KT, FmtQ6K::SUM_GRAN) <= kLdsBudget &&
+            (N + kGemvWaves * (64 / pick_group(K / 64)) - 1) / (kGemvWaves * (64 / pick_group(K / 64))) <= 2u * (uint32_t)cu_count()) {
+            if (int rc = check_common(x, y, K, N, 1, 256)) return rc;
+            MX_REQUIRE_ALIGN(x, 16);
+            GemvSeg<FmtQ6K, half_t> g{wa, reinterpret_cast<half_t*>(y), nullptr};
+            const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu;
+            hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ6K, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
+                               act_tile_bytes(1, KT, FmtQ6K::SUM_GRAN), as_stream(s), g, g, static_cast<const uint8_t*>(x), K, N, KT, 1u, 2u);
+            return launch_status();
+        }
         return nw == 2 ? launch_ffn_x<FmtQ6K, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ6K, 1>(s, wa, wb, x, x_is_f16, y, K, N);
     }
     const FmtQ8Aos::W wa{a, K / 32 * (uint32_t)kQ8_0Bytes}, wb{b, K / 32 * (uint32_t)kQ8_0Bytes};
@@ -1388,6 +1414,15 @@ int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* q
     MX_REQUIRE_PTR(qs_W); MX_REQUIRE_PTR(d_W);
     MX_REQUIRE_ALIGN(qs_W, 16); MX_REQUIRE_ALIGN(d_W, 2);
     const FmtQ8Soa::W w{qs_W, d_W, K};
+    if (q8_soa_wide(K, N)) {   // the same launch as mx_gemv_q8_0_soa_q8 takes for this shape, the row quantized while it is staged
+        if (int rc = check_common(x_f16, y, K, N, 1, 32)) return rc;
+        MX_REQUIRE_ALIGN(x_f16, 16);
+        GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
+        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * kWgsPerCu;
+        hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
+                           act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN), as_stream(s), g, g, reinterpret_cast<const uint8_t*>(x_f16), K, N, KT, 1u, 2u);
+        return launch_status();
+    }
     if (q8_soa_interleaved(K)) return launch_ffn_x<FmtQ8SoaW, 1>(s, w, w, x_f16, 1, y, K, N);
     return launch_ffn_x<FmtQ8Soa, 1>(s, w, w, x_f16, 1, y, K, N);
 }

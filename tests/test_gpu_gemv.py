@@ -279,11 +279,12 @@ def test_gemv_q8_x2_equals_two_single_launches(mx, fmt):
 
 
 @pytest.mark.parametrize("fmt", (O.Q4_K, O.Q6_K, O.Q8_0))
-@pytest.mark.parametrize("K,N", [(2048, 320), (4096, 1056), (1280, 96)])
+@pytest.mark.parametrize("K,N", [(2048, 320), (4096, 1056), (1280, 96), (14336, 64)])
 def test_decode_ffn_forms_equal_the_launch_chain(mx, fmt, K, N):
     """gate + up + SwiGLU in one launch, and GEMVs that quantize the fp16 activation row while staging it: the bits of
     quantize_q8_1 -> gemv x2 -> swiglu and of quantize_q8_1 -> gemv, whose parts are gated against the oracle above.
-    K = 2048 / 4096 / 1280 walk 32, 64 and 16 lanes per row (1280 leaves lanes of the last round without a unit)."""
+    K = 2048 / 4096 / 1280 walk 32, 64 and 16 lanes per row (1280 leaves lanes of the last round without a unit);
+    K = 14336 with few rows is the down-projection shape (Q8_0 planes: the workgroup-wide walk in both forms)."""
     ops = mx.ops
     name = O.FMT_NAMES[fmt]
     Wg, Wu = weights(fmt, 1600 + fmt, N, K), weights(fmt, 1610 + fmt, N, K)
@@ -297,8 +298,9 @@ def test_decode_ffn_forms_equal_the_launch_chain(mx, fmt, K, N):
         h_chain, hq_chain = ops.swiglu_q8(g, u)
         h1 = ops.gemv_x2_silu(nm, xq, g_w, u_w, K, N)
         h2 = ops.gemv_x2_silu(nm, x16.reshape(-1), g_w, u_w, K, N)
-        assert torch.equal(h1, h_chain), "%s: fused gate/up/silu on the q8 row != the three launches" % nm
-        assert torch.equal(h2, h_chain), "%s: fused gate/up/silu on the fp16 row != the four launches" % nm
+        assert torch.equal(h1, h2), "%s: fused gate/up/silu on the fp16 row != on the q8 row" % nm
+        if K < 8192:   # long rows of a short matrix: the separate launches walk a row with the whole workgroup, another summation order
+            assert torch.equal(h1, h_chain), "%s: fused gate/up/silu != the launch chain" % nm
         single = (lambda w: ops.gemv_q8_0_soa_q8(xq, w[0], w[1], K, N)) if nm == "q8_0_soa" else (lambda w: getattr(ops, "gemv_%s_q8" % nm)(xq, w, K, N))
         assert torch.equal(ops.gemv_f16q8(nm, x16.reshape(-1), g_w, K, N), single(g_w)), "%s: gemv on the fp16 row != quantize + gemv" % nm
     # and the fused result against the oracle chain directly (q8-chain dots, fp16 roundings of g and u, SwiGLU)
@@ -323,7 +325,10 @@ def test_gemv_long_rows_few_of_them(mx, fmt, K):
         qs, d = (dev(p) for p in O.repack_q8_0_to_soa(W))
         got2 = mx.ops.gemv_q8_0_soa_q8(dev(xq), qs, d, K, N)
         check(host(got2).astype(np.float32), ref[0], "gemv_q8_0_soa_q8 K=%d N=%d" % (K, N))
-        assert torch.equal(got, got2)
+        # blocks and planes walk a long row in different orders (lane groups / the whole workgroup): same products,
+        # fp32 sums that differ in the last bits, so nearly every fp16 output is the same and none is far
+        a, b = host(got).astype(np.float32), host(got2).astype(np.float32)
+        assert (a == b).mean() > 0.97 and np.abs(a - b).max() <= 2e-3 * np.abs(a).max()
 
 
 @pytest.mark.parametrize("K,N", [(1312, 96), (4128, 64), (14368, 32)])
