@@ -581,6 +581,7 @@ static uint32_t resident_wgs(const void* kernel, uint32_t lds) {
 }
 constexpr int kRows = 2;             // rows per lane group, float-activation kernels
 constexpr uint32_t kWgsPerCu = 4;    // persistent grid: workgroups per CU
+constexpr uint32_t kWideF16WgsPerCu = 3;   // the workgroup-wide walk on an fp16 row: every workgroup quantizes the whole row while staging it
 // rows per lane group / unroll of the unit walk: one row and two units in flight for a single
 // token; batched, two rows share each activation read once the per-token work dominates
 // (T > 4, or T > 2 for the formats whose fold carries a min term), one row below that
@@ -1391,7 +1392,7 @@ static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, 
             if (int rc = check_common(x, y, K, N, 1, 256)) return rc;
             MX_REQUIRE_ALIGN(x, 16);
             GemvSeg<FmtQ6K, half_t> g{wa, reinterpret_cast<half_t*>(y), nullptr};
-            const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu;
+            const uint32_t capw = (uint32_t)cu_count() * kWideF16WgsPerCu;
             hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ6K, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
                                act_tile_bytes(1, KT, FmtQ6K::SUM_GRAN), as_stream(s), g, g, static_cast<const uint8_t*>(x), K, N, KT, 1u, 2u);
             return launch_status();
@@ -1418,7 +1419,7 @@ int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* q
         if (int rc = check_common(x_f16, y, K, N, 1, 32)) return rc;
         MX_REQUIRE_ALIGN(x_f16, 16);
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
-        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * kWgsPerCu;
+        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * kWideF16WgsPerCu;
         hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
                            act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN), as_stream(s), g, g, reinterpret_cast<const uint8_t*>(x_f16), K, N, KT, 1u, 2u);
         return launch_status();
