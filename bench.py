@@ -571,6 +571,19 @@ def main():
             tf = 2.0 * TK5 * H5 * EF5 * 3 / us / 1e6
             detail["config5_moe_grouped_gemm_q8_0"] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK, 4),
                                                        "route": "fp16 rows, fp16 MFMA (mx_moe_gemm_*)"}
+            # the same layer from the unsorted token rows: gather launch + the two GEMMs, against the gather folded into the row loads
+            si5d = torch.from_numpy(si5).to(dev)
+
+            def layer5_gather(i):
+                ops.moe_gather_rows(x5, si5d, TK5, H5, xp5)
+                layer5(i)
+
+            def layer5_fused(i):
+                ops.moe_gemm_gate_up_silu_q8(x5, gq5, gd5, uq5, ud5, EF5 * H5, EF5 * H5 // 32, off5d, TK5, E5, H5, EF5, h5, sorted_idx=si5d)
+                ops.moe_gemm_down_q8(h5, dq5, dd5, H5 * EF5, H5 * EF5 // 32, off5d, wp5d, TK5, E5, H5, EF5, o5)
+
+            detail["config5_from_unsorted_rows"] = {"gather_launch_plus_gemms_us": round(kernel_avg_us(layer5_gather, 3), 1),
+                                                    "gather_in_the_row_loads_us": round(kernel_avg_us(layer5_fused, 3), 1)}
             # the same layer through the reference's own signatures: q8 rows (quantize_q8_1) -> moe_prefill_gate_up_silu_q8 ->
             # quantize_q8_1 -> moe_prefill_down_q8, int8 MFMA with the per-block fp32 fold (peak 5 POP/s dense int8)
             xq5 = torch.empty(TK5 * (H5 // 32) * 40, dtype=torch.uint8, device=dev)

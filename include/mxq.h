@@ -371,6 +371,24 @@ int mx_moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x_packed, const i
 int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride,
                         uint64_t d_stride, const uint32_t* expert_offsets, const uint16_t* sorted_w, uint16_t* out_packed,
                         uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+/* Gather forms of the grouped gate/up GEMMs: moe_gather_rows (include/ie/ops.hpp, src/ops/moe.cpp:423-446) folded into the
+ * load of the activation rows.  x is the unsorted [n_tokens, H] fp16 matrix and sorted_idx[r] (device, total_rows
+ * entries, each in [0, n_tokens)) the source row of sorted row r, as build_moe_packing returns it; no gathered copy
+ * is written or read.  Same results as mx_moe_gather_rows followed by the entry of the same name, bit for bit.
+ * n_tokens * H * 2 < 2^32.  */
+int mx_moe_gemm_gate_up_silu_q8_gather(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens,
+                                       const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d,
+                                       uint64_t qs_stride, uint64_t d_stride, const uint32_t* expert_offsets, uint16_t* h_packed,
+                                       uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows);
+int mx_moe_gemm_gate_up_silu_q4k_gather(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens,
+                                        const void* gate_W, const void* up_W, const uint32_t* expert_offsets, uint16_t* h_packed,
+                                        uint32_t E, uint32_t H, uint32_t E_ffn, uint64_t expert_stride_bytes, int soa,
+                                        uint32_t total_rows);
+int mx_moe_gemm_gate_up_oai_mxfp4_gather(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens,
+                                         const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
+                                         uint64_t qs_stride, uint64_t e_stride, const float* gate_bias, const float* up_bias,
+                                         const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H,
+                                         uint32_t E_ffn, uint32_t total_rows, float alpha, float limit);
 /* The same for AoS K-quant expert banks (expert e at W + e*expert_stride_bytes, include/ie/ops.hpp:1027-1029):
  *   moe_prefill_gate_up_silu_q4k (fp16 x_packed) / _q4k_xmx   include/ie/ops.hpp:922-929, src/ops/moe_fused.cpp:727-901,
  *                                                             src/ops/gemm_q4k_xmx.cpp:662-847

@@ -644,6 +644,7 @@ struct GemmArgs {
     half_t* Y;                        // [M, N]
     const uint32_t* expert_offsets;   // grouped: [E+1]
     const half_t* route_w;            // GEMM_MOE_DOWN: [TK] fp16 row weights, or NULL for unweighted rows
+    const int32_t* a_row_index;       // grouped gate/up, gather form: A row of sorted row r is a_row_index[r] (A = the unsorted [T, K] rows)
     const int32_t* row_token;         // GEMM_MOE_DOWN, accumulate form: token of each sorted row
     float* y_acc;                     //   and the fp32 [T, N] buffer w * acc is atomically added into (Y unused)
     uint32_t M, K, N, E;
@@ -920,14 +921,18 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const typename QF::
     // A staging: wave w brings rows (BM/4) w .. of the chunk, 4 rows (1 KB) per load; lane L fills LDS slot
     // (row 4j + L/16, column L%16) of that 1 KB with global column (L%16) ^ (row & 15).  Rows past the end of
     // the tile re-read its last row (never used).
+    // Gather form (grouped gate/up): the rows are read where they lie in the unsorted [T, K] matrix, through the sorted
+    // row -> source row index, so no gathered copy is written and read back (moe_gather_rows folded into the A load).
+    const bool gather = MODE != GEMM_DENSE && g.a_row_index != nullptr;
     uint32_t a_off[NL];
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
         const uint32_t R = (BM / 4u) * wave + 4u * j + (lane >> 4);
         const uint32_t Rc = R < live_rows ? R : live_rows - 1u;
-        a_off[j] = Rc * (g.K * 2u) + (((lane & 15u) ^ (R & 15u)) << 4);
+        const uint32_t src = gather ? (uint32_t)g.a_row_index[row_lo + Rc] : Rc;
+        a_off[j] = src * (g.K * 2u) + (((lane & 15u) ^ (R & 15u)) << 4);
     }
-    const uint8_t* a_glb = reinterpret_cast<const uint8_t*>(g.A + (size_t)row_lo * g.K) + (size_t)c0 * (kBK * 2u);
+    const uint8_t* a_glb = reinterpret_cast<const uint8_t*>(g.A + (gather ? (size_t)0 : (size_t)row_lo * g.K)) + (size_t)c0 * (kBK * 2u);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds_raw;
     const uint32_t a_dst = lds_base + wave * (BM / 4u) * 256u;   // this wave's quarter of the rows inside an A buffer
     // step-0 fragment address of this lane inside an A buffer
@@ -1417,7 +1422,7 @@ static int check_gemm(const void* A, const void* W, const void* y, uint32_t M, u
 template <class QF, int MODE>
 static int moe_gemm_aos(mx_stream_t s, const uint16_t* rows, const void* W0, const void* W1, uint64_t expert_stride_bytes, const uint32_t* expert_offsets,
                         const uint16_t* sorted_w, uint16_t* out, uint32_t E, uint32_t K, uint32_t N, uint32_t total_rows, uint32_t block_bytes,
-                        uint32_t w_align, const int32_t* row_token = nullptr, float* y_acc = nullptr) {
+                        uint32_t w_align, const int32_t* row_token = nullptr, float* y_acc = nullptr, const int32_t* a_row_index = nullptr) {
     if (int rc = check_gemm(rows, W0, y_acc ? static_cast<const void*>(y_acc) : out, total_rows, K, N, 256, w_align)) return rc;
     MX_REQUIRE_PTR(W1); MX_REQUIRE_PTR(expert_offsets);
     MX_REQUIRE_SHAPE(E > 0 && expert_stride_bytes % w_align == 0);
@@ -1425,7 +1430,7 @@ static int moe_gemm_aos(mx_stream_t s, const uint16_t* rows, const void* W0, con
     GemmArgs g{};
     g.A = reinterpret_cast<const half_t*>(rows); g.Y = reinterpret_cast<half_t*>(out); g.expert_offsets = expert_offsets;
     g.route_w = reinterpret_cast<const half_t*>(sorted_w); g.M = total_rows; g.K = K; g.N = N; g.E = E;
-    g.row_token = row_token; g.y_acc = y_acc;
+    g.row_token = row_token; g.y_acc = y_acc; g.a_row_index = a_row_index;
     if constexpr (std::is_same<QF, GemmQ4KStr>::value || std::is_same<QF, GemmQ6KStr>::value) {
         const uint64_t nb = (uint64_t)N * (K / 256);
         typename QF::Bank b0{static_cast<const uint8_t*>(W0), expert_stride_bytes, nb, K / 256}, b1{static_cast<const uint8_t*>(W1), expert_stride_bytes, nb, K / 256};
@@ -1520,18 +1525,38 @@ int mx_gemm_q8_0_soa_ws(mx_stream_t s, const uint16_t* A, const int8_t* qs_W, co
     return gemm_dense_q8_soa(s, A, qs_W, d_W, y, M, K, N, &w);
 }
 
-int mx_moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
-                                const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const uint32_t* expert_offsets, uint16_t* h_packed,
-                                uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
-    if (int rc = check_gemm(x_packed, g_qs, h_packed, total_rows, H, E_ffn, 128)) return rc;
+// gather form: x = the unsorted rows [n_tokens, H], sorted_idx[r] = source row of sorted row r (NULL: x is already sorted)
+static int check_gather(const int32_t* sorted_idx, uint32_t n_tokens, uint32_t H) {
+    if (!sorted_idx) return MX_OK;
+    MX_REQUIRE_ALIGN(sorted_idx, 4);
+    MX_REQUIRE_SHAPE(n_tokens > 0 && (uint64_t)n_tokens * H * 2u < (1ull << 32));   // the A loads address rows with 32-bit byte offsets
+    return MX_OK;
+}
+static int moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens, const int8_t* g_qs, const uint16_t* g_d,
+                                    const int8_t* u_qs, const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const uint32_t* expert_offsets,
+                                    uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    if (int rc = check_gemm(x, g_qs, h_packed, total_rows, H, E_ffn, 128)) return rc;
+    if (int rc = check_gather(sorted_idx, n_tokens, H)) return rc;
     MX_REQUIRE_PTR(g_d); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_d); MX_REQUIRE_PTR(expert_offsets);
     MX_REQUIRE_SHAPE(E > 0 && qs_stride % 16 == 0 && d_stride % 2 == 0);
     MX_REQUIRE_ALIGN(u_qs, 16); MX_REQUIRE_ALIGN(g_d, 4); MX_REQUIRE_ALIGN(u_d, 4);
     GemmArgs g{};
-    g.A = reinterpret_cast<const half_t*>(x_packed); g.Y = reinterpret_cast<half_t*>(h_packed); g.expert_offsets = expert_offsets;
+    g.A = reinterpret_cast<const half_t*>(x); g.Y = reinterpret_cast<half_t*>(h_packed); g.expert_offsets = expert_offsets;
+    g.a_row_index = sorted_idx;
     g.M = total_rows; g.K = H; g.N = E_ffn; g.E = E;
     GemmQ8Soa::Bank bg{g_qs, g_d, qs_stride, d_stride, H}, bu{u_qs, u_d, qs_stride, d_stride, H};
     return launch_gemm<GemmQ8Soa, GEMM_MOE_GATE_UP_SILU>(s, bg, bu, g, total_rows);
+}
+int mx_moe_gemm_gate_up_silu_q8(mx_stream_t s, const uint16_t* x_packed, const int8_t* g_qs, const uint16_t* g_d, const int8_t* u_qs,
+                                const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride, const uint32_t* expert_offsets, uint16_t* h_packed,
+                                uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    return moe_gemm_gate_up_silu_q8(s, x_packed, nullptr, 0, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, h_packed, E, H, E_ffn, total_rows);
+}
+int mx_moe_gemm_gate_up_silu_q8_gather(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens, const int8_t* g_qs,
+                                       const uint16_t* g_d, const int8_t* u_qs, const uint16_t* u_d, uint64_t qs_stride, uint64_t d_stride,
+                                       const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows) {
+    MX_REQUIRE_PTR(sorted_idx);
+    return moe_gemm_gate_up_silu_q8(s, x, sorted_idx, n_tokens, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, h_packed, E, H, E_ffn, total_rows);
 }
 
 int mx_moe_gemm_down_q8(mx_stream_t s, const uint16_t* h_packed, const int8_t* d_qs, const uint16_t* d_d, uint64_t qs_stride, uint64_t d_stride,
@@ -1556,6 +1581,18 @@ int mx_moe_gemm_gate_up_silu_q4k(mx_stream_t s, const uint16_t* x_packed, const 
                                                                total_rows, kQ4KBytes, 16);
     return moe_gemm_aos<GemmQ4K, GEMM_MOE_GATE_UP_SILU>(s, x_packed, gate_W, up_W, expert_stride_bytes, expert_offsets, nullptr, h_packed, E, H, E_ffn,
                                                         total_rows, kQ4KBytes, 16);
+}
+
+int mx_moe_gemm_gate_up_silu_q4k_gather(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens, const void* gate_W, const void* up_W,
+                                        const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn,
+                                        uint64_t expert_stride_bytes, int soa, uint32_t total_rows) {
+    MX_REQUIRE_PTR(sorted_idx);
+    if (int rc = check_gather(sorted_idx, n_tokens, H)) return rc;
+    if (soa)
+        return moe_gemm_aos<GemmQ4KStr, GEMM_MOE_GATE_UP_SILU>(s, x, gate_W, up_W, expert_stride_bytes, expert_offsets, nullptr, h_packed, E, H, E_ffn,
+                                                               total_rows, kQ4KBytes, 16, nullptr, nullptr, sorted_idx);
+    return moe_gemm_aos<GemmQ4K, GEMM_MOE_GATE_UP_SILU>(s, x, gate_W, up_W, expert_stride_bytes, expert_offsets, nullptr, h_packed, E, H, E_ffn,
+                                                        total_rows, kQ4KBytes, 16, nullptr, nullptr, sorted_idx);
 }
 
 int mx_moe_gemm_down_q4k(mx_stream_t s, const uint16_t* h_packed, const void* down_W, const uint32_t* expert_offsets, const uint16_t* sorted_w,
@@ -1589,15 +1626,36 @@ int mx_gemm_mxfp4_soa(mx_stream_t s, const uint16_t* A, const uint8_t* qs_W, con
     GemmMxfp4Soa::Bank b{qs_W, e_W, 0, 0, K};
     return launch_gemm<GemmMxfp4Soa, GEMM_DENSE>(s, b, b, g, M, nullptr);
 }
+static int moe_gemm_gate_up_oai_mxfp4(mx_stream_t s, const uint16_t* x_packed, const int32_t* sorted_idx, uint32_t n_tokens, const uint8_t* g_qs,
+                                      const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride,
+                                      const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E,
+                                      uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha, float limit);
 int mx_moe_gemm_gate_up_oai_mxfp4(mx_stream_t s, const uint16_t* x_packed, const uint8_t* g_qs, const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e,
                                   uint64_t qs_stride, uint64_t e_stride, const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets,
                                   uint16_t* h_packed, uint32_t E, uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha, float limit) {
+    return moe_gemm_gate_up_oai_mxfp4(s, x_packed, nullptr, 0, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, expert_offsets, h_packed, E, H,
+                                      E_ffn, total_rows, alpha, limit);
+}
+int mx_moe_gemm_gate_up_oai_mxfp4_gather(mx_stream_t s, const uint16_t* x, const int32_t* sorted_idx, uint32_t n_tokens, const uint8_t* g_qs,
+                                         const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride,
+                                         const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E,
+                                         uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha, float limit) {
+    MX_REQUIRE_PTR(sorted_idx);
+    return moe_gemm_gate_up_oai_mxfp4(s, x, sorted_idx, n_tokens, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, expert_offsets, h_packed, E, H,
+                                      E_ffn, total_rows, alpha, limit);
+}
+static int moe_gemm_gate_up_oai_mxfp4(mx_stream_t s, const uint16_t* x_packed, const int32_t* sorted_idx, uint32_t n_tokens, const uint8_t* g_qs,
+                                      const uint8_t* g_e, const uint8_t* u_qs, const uint8_t* u_e, uint64_t qs_stride, uint64_t e_stride,
+                                      const float* gate_bias, const float* up_bias, const uint32_t* expert_offsets, uint16_t* h_packed, uint32_t E,
+                                      uint32_t H, uint32_t E_ffn, uint32_t total_rows, float alpha, float limit) {
     if (int rc = check_gemm(x_packed, g_qs, h_packed, total_rows, H, E_ffn, 64)) return rc;
+    if (int rc = check_gather(sorted_idx, n_tokens, H)) return rc;
     MX_REQUIRE_PTR(g_e); MX_REQUIRE_PTR(u_qs); MX_REQUIRE_PTR(u_e); MX_REQUIRE_PTR(expert_offsets);
     MX_REQUIRE_SHAPE(E > 0 && qs_stride % 16 == 0);
     MX_REQUIRE_ALIGN(u_qs, 16);
     GemmArgs g{};
     g.A = reinterpret_cast<const half_t*>(x_packed); g.Y = reinterpret_cast<half_t*>(h_packed); g.expert_offsets = expert_offsets;
+    g.a_row_index = sorted_idx;
     g.M = total_rows; g.K = H; g.N = E_ffn; g.E = E; g.bias0 = gate_bias; g.bias1 = up_bias; g.alpha = alpha; g.limit = limit;
     GemmMxfp4Soa::Bank bg{g_qs, g_e, qs_stride, e_stride, H}, bu{u_qs, u_e, qs_stride, e_stride, H};
     return launch_gemm<GemmMxfp4Soa, GEMM_MOE_GATE_UP_OAI>(s, bg, bu, g, total_rows);

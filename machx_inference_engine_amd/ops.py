@@ -737,9 +737,14 @@ def gemm_q8_0(A, W, M, K, N, y=None):
     return y
 
 
-def moe_gemm_gate_up_silu_q4k(x_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None, soa=False):
-    """soa: the expert regions hold per-field streams (repack_moe_kquant_soa) instead of GGUF blocks."""
+def moe_gemm_gate_up_silu_q4k(x_packed, gate_W, up_W, expert_offsets, TK, E, H, E_ffn, expert_stride_bytes, h_packed=None, soa=False, sorted_idx=None):
+    """soa: the expert regions hold per-field streams (repack_moe_kquant_soa) instead of GGUF blocks.
+    sorted_idx (int32 [TK]): x_packed is the unsorted [T, H] matrix and the rows are gathered while they are loaded."""
     h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
+    if sorted_idx is not None:
+        _call("mx_moe_gemm_gate_up_silu_q4k_gather", _f16(x_packed), _ptr(sorted_idx), x_packed.numel() // H, _u8(gate_W), _u8(up_W), _ptr(expert_offsets),
+              _ptr(h_packed), E, H, E_ffn, expert_stride_bytes, 1 if soa else 0, TK)
+        return h_packed
     _call("mx_moe_gemm_gate_up_silu_q4k", _f16(x_packed), _u8(gate_W), _u8(up_W), _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn,
           expert_stride_bytes, 1 if soa else 0, TK)
     return h_packed
@@ -767,8 +772,14 @@ def gemm_mxfp4_soa(A, qs_plane, e_plane, M, K, N, y=None):
 
 
 def moe_gemm_gate_up_oai_mxfp4(x_packed, g_qs, g_e, u_qs, u_e, qs_stride, e_stride, gate_bias, up_bias, expert_offsets, TK, E, H, E_ffn,
-                               alpha=1.702, limit=7.0, h_packed=None):
+                               alpha=1.702, limit=7.0, h_packed=None, sorted_idx=None):
+    """sorted_idx (int32 [TK]): x_packed is the unsorted [T, H] matrix and the rows are gathered while they are loaded."""
     h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
+    if sorted_idx is not None:
+        _call("mx_moe_gemm_gate_up_oai_mxfp4_gather", _f16(x_packed), _ptr(sorted_idx), x_packed.numel() // H, _u8(g_qs), _u8(g_e), _u8(u_qs), _u8(u_e),
+              qs_stride, e_stride, _ptr(gate_bias) if gate_bias is not None else None, _ptr(up_bias) if up_bias is not None else None,
+              _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn, TK, float(alpha), float(limit))
+        return h_packed
     _call("mx_moe_gemm_gate_up_oai_mxfp4", _f16(x_packed), _u8(g_qs), _u8(g_e), _u8(u_qs), _u8(u_e), qs_stride, e_stride,
           _ptr(gate_bias) if gate_bias is not None else None, _ptr(up_bias) if up_bias is not None else None, _ptr(expert_offsets), _ptr(h_packed),
           E, H, E_ffn, TK, float(alpha), float(limit))
@@ -788,8 +799,13 @@ def gemm_q8_0_soa(A, qs_W, d_W, M, K, N, y=None):
     return y
 
 
-def moe_gemm_gate_up_silu_q8(x_packed, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, TK, E, H, E_ffn, h_packed=None):
+def moe_gemm_gate_up_silu_q8(x_packed, g_qs, g_d, u_qs, u_d, qs_stride, d_stride, expert_offsets, TK, E, H, E_ffn, h_packed=None, sorted_idx=None):
+    """sorted_idx (int32 [TK]): x_packed is the unsorted [T, H] matrix and the rows are gathered while they are loaded."""
     h_packed = _out(h_packed, (TK, E_ffn), torch.float16, x_packed)
+    if sorted_idx is not None:
+        _call("mx_moe_gemm_gate_up_silu_q8_gather", _f16(x_packed), _ptr(sorted_idx), x_packed.numel() // H, _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d),
+              qs_stride, d_stride, _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn, TK)
+        return h_packed
     _call("mx_moe_gemm_gate_up_silu_q8", _f16(x_packed), _u8(g_qs), _ptr(g_d), _u8(u_qs), _ptr(u_d), qs_stride, d_stride,
           _ptr(expert_offsets), _ptr(h_packed), E, H, E_ffn, TK)
     return h_packed

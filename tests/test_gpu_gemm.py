@@ -168,6 +168,9 @@ def test_moe_grouped_gemm_q8(mx, T, E, Kt, H, EF):
     print("rows per expert: min %d max %d, empty %d" % (counts.min(), counts.max(), (counts == 0).sum()))
     xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
     hp = ops.moe_gemm_gate_up_silu_q8(xp, dev(gq), dev(gd), dev(uq), dev(ud), EF * H, EF * H // 32, dev(off), TK, E, H, EF)
+    # the gather folded into the row loads: the unsorted rows and the sorted -> source index, the same bits
+    hp_g = ops.moe_gemm_gate_up_silu_q8(dev(x).half(), dev(gq), dev(gd), dev(uq), dev(ud), EF * H, EF * H // 32, dev(off), TK, E, H, EF, sorted_idx=dev(si))
+    assert torch.equal(hp_g, hp), "gather form differs from gather_rows + grouped GEMM"
     hp_h = host(hp).astype(np.float32)
     xs = x[si]
     h_ref = np.zeros((TK, EF), np.float32)
@@ -269,6 +272,9 @@ def test_moe_grouped_gemm_kquant(mx, T, E, Kt, H, EF):
     Wg_s, Wu_s = ops.repack_moe_kquant_soa("q4k", Wg, E, nb_gu), ops.repack_moe_kquant_soa("q4k", Wu, E, nb_gu)
     hp_s = ops.moe_gemm_gate_up_silu_q4k(xp, dev(Wg_s), dev(Wu_s), dev(off), TK, E, H, EF, stride_gu, soa=True)
     assert torch.equal(hp_s, hp), "soa gate/up differs from the AoS bank"
+    for soa, (a, b) in ((False, (Wg, Wu)), (True, (Wg_s, Wu_s))):
+        hp_g = ops.moe_gemm_gate_up_silu_q4k(dev(x).half(), dev(a), dev(b), dev(off), TK, E, H, EF, stride_gu, soa=soa, sorted_idx=dev(si))
+        assert torch.equal(hp_g, hp), "gather form differs from gather_rows + grouped GEMM"
     for fmt, F in (("q4k", O.Q4_K), ("q6k", O.Q6_K)):
         Wd = mk(F, 5100, H, EF)
         o_ref = np.zeros((TK, H), np.float64)
@@ -365,6 +371,9 @@ def test_moe_grouped_gemm_mxfp4(mx, T, E, Kt, H, EF):
     TK = T * Kt
     xp = ops.moe_gather_rows(dev(x).half(), dev(si), TK, H)
     hp = ops.moe_gemm_gate_up_oai_mxfp4(xp, dev(gq), dev(ge), dev(uq), dev(ue), qs_st, e_st, dev(bg), dev(bu), dev(off), TK, E, H, EF)
+    hp_g = ops.moe_gemm_gate_up_oai_mxfp4(dev(x).half(), dev(gq), dev(ge), dev(uq), dev(ue), qs_st, e_st, dev(bg), dev(bu), dev(off), TK, E, H, EF,
+                                          sorted_idx=dev(si))
+    assert torch.equal(hp_g, hp), "gather form differs from gather_rows + grouped GEMM"
     hp_h = host(hp).astype(np.float32)
     xs = x[si]
     rows = np.arange(TK) if TK <= 256 else np.random.default_rng(9).choice(TK, 48, replace=False)
