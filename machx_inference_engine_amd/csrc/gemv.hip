@@ -675,6 +675,13 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t lds = act_tile_bytes(T, KT, F::SUM_GRAN);
     uint32_t per_cu = resident_wgs(reinterpret_cast<const void*>(&gemv_q8_kernel<F, T, R, G, U, OutT>), lds);
     if (per_cu > kWgsPerCu) per_cu = kWgsPerCu;
+    if constexpr (T == 1 && std::is_same<F, FmtQ8SoaW>::value) {
+        // The interleaved Q8_0 units keep two rows per wave in flight, and more waves than the memory system can serve only
+        // lengthen its queues: two workgroups per CU for launches of 24576 rows and more (fused gate + up 20.8 -> 20.45 us,
+        // 4096 -> 128256 88.3 -> 85.2 us), three below that (4096 -> 14336: 12.0 us with two, three or four).
+        const uint32_t fewer = (uint64_t)nseg * N >= 24576u ? 2u : 3u;
+        if (per_cu > fewer) per_cu = fewer;
+    }
     const uint32_t cap = (uint32_t)cu_count() * per_cu / nseg;
     dim3 grid(n_rg < cap ? n_rg : (cap ? cap : 1u), nseg);
     hipLaunchKernelGGL((gemv_q8_kernel<F, T, R, G, U, OutT>), grid, dim3(kGemvThreads), lds, st, s0, s1, xq8, K, N, KT, T_real, split ? 1u : 0u);
@@ -1033,7 +1040,8 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
         // rotation of the plain units (gemv_q8_deep_kernel): 13.9 -> 12.1 us (two rows per pass: 12.2 - 12.9 us); two
         // tokens against the lane-group walk: 15.7 -> 13.9 us.
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
-        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * (T == 1 ? kWgsPerCu : 3u);
+        // three workgroups per CU (one token: 12.5 us with four, 12.1 with three, 13.1 with two)
+        const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * 3u;
         const dim3 gridw(N < capw ? N : capw, 1);
         const uint8_t* xq = static_cast<const uint8_t*>(x);
         if (T == 1)
