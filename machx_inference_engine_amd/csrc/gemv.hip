@@ -675,11 +675,19 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t lds = act_tile_bytes(T, KT, F::SUM_GRAN);
     uint32_t per_cu = resident_wgs(reinterpret_cast<const void*>(&gemv_q8_kernel<F, T, R, G, U, OutT>), lds);
     if (per_cu > kWgsPerCu) per_cu = kWgsPerCu;
-    if constexpr (T == 1 && std::is_same<F, FmtQ8SoaW>::value) {
-        // The interleaved Q8_0 units keep two rows per wave in flight, and more waves than the memory system can serve only
-        // lengthen its queues: two workgroups per CU for launches of 24576 rows and more (fused gate + up 20.8 -> 20.45 us,
-        // 4096 -> 128256 88.3 -> 85.2 us), three below that (4096 -> 14336: 12.0 us with two, three or four).
-        const uint32_t fewer = (uint64_t)nseg * N >= 24576u ? 2u : 3u;
+    {
+        // More waves than the memory system can serve only lengthen its queues; measured per format (K = 4096, us with
+        // four workgroups per CU -> with the number chosen here).  Q8_0 planes, interleaved units (two rows per wave in
+        // flight): fused gate + up 20.8 -> 20.45 and 128256 rows 88.3 -> 85.2 with two, 14336 rows 12.0 with two, three
+        // or four.  GGUF Q8_0 blocks: one token 13.0 -> 12.15 and two 14.1 -> 13.4 with two, four tokens 15.6 -> 14.6
+        // with three.  Q4_K, one token: 8.2 -> 8.0 with three (4096 rows, q8 activations: 4.47 -> 4.15).  Q6_K, one token:
+        // 151936 rows 95.1 -> 92.0 with three; 14336 rows and the fused launch are fastest with four.
+        const uint64_t rows = (uint64_t)nseg * N;
+        uint32_t fewer = kWgsPerCu;
+        if constexpr (T == 1 && std::is_same<F, FmtQ8SoaW>::value) fewer = rows >= 24576u ? 2u : 3u;
+        else if constexpr (std::is_same<F, FmtQ8Aos>::value) fewer = T <= 2 ? 2u : (T <= 4 ? 3u : kWgsPerCu);
+        else if constexpr (T == 1 && std::is_same<F, FmtQ4K>::value) fewer = 3u;
+        else if constexpr (T == 1 && std::is_same<F, FmtQ6K>::value) fewer = rows >= 65536u ? 3u : kWgsPerCu;
         if (per_cu > fewer) per_cu = fewer;
     }
     const uint32_t cap = (uint32_t)cu_count() * per_cu / nseg;
