@@ -22,10 +22,10 @@ struct GemvSeg {
 
 // Formats whose T = 1 kernels hold a second set of units in registers (requested ahead of the row group being
 // summed, or ahead of the activation staging): the ones where that was measured to pay and that stay within the
-// 128 VGPRs the four-workgroups-per-CU launch wants.  Q6_K does not gain from it (12.1 -> 12.2 us on 4096 -> 14336,
-// 95.8 -> 98.5 us on the 151936-row output projection with the two alternating sets).
+// 128 VGPRs the four-workgroups-per-CU launch wants.  Q6_K gains nothing from it with four workgroups per CU (12.1 ->
+// 12.2 us on 4096 -> 14336, 95.8 -> 98.5 us on the 151936-row output projection) and a tenth with two (launch_q8_tg).
 template <class F>
-constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ8SoaW>::value || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value;
+constexpr bool kPrefetchAcrossRows = std::is_same<F, FmtQ8Soa>::value || std::is_same<F, FmtQ8SoaW>::value || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value || std::is_same<F, FmtQ6K>::value;
 
 // Persistent workgroups: each stages the activation tile(s) and then streams
 // its share of row groups.  With a single K-tile (every decode shape at T <= 2)
@@ -680,14 +680,17 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
         // four workgroups per CU -> with the number chosen here).  Q8_0 planes, interleaved units (two rows per wave in
         // flight): fused gate + up 20.8 -> 20.45 and 128256 rows 88.3 -> 85.2 with two, 14336 rows 12.0 with two, three
         // or four.  GGUF Q8_0 blocks: one token 13.0 -> 12.15 and two 14.1 -> 13.4 with two, four tokens 15.6 -> 14.6
-        // with three.  Q4_K, one token: 8.2 -> 8.0 with three (4096 rows, q8 activations: 4.47 -> 4.15).  Q6_K, one token:
-        // 151936 rows 95.1 -> 92.0 with three; 14336 rows and the fused launch are fastest with four.
+        // with three.  Q4_K, one token: 8.2 -> 8.0 with three (4096 rows, q8 activations: 4.47 -> 4.15).  Q6_K, one or two
+        // tokens, with the two register sets of the one-unit-per-lane path (the same bytes in flight per CU as four
+        // workgroups with one set, half the waves competing for the vector pipe): fused gate + up 19.7 -> 17.6 with two
+        // (21.9 with one, 19.4 with three), 14336 rows 12.45 -> 11.3, 151936 rows 94.2 -> 88.5, 4096 rows 6.4 -> 5.1, two
+        // tokens 14.5 -> 13.3; K = 8192: 16.1 -> 13.9 with three.
         const uint64_t rows = (uint64_t)nseg * N;
         uint32_t fewer = kWgsPerCu;
         if constexpr (T == 1 && std::is_same<F, FmtQ8SoaW>::value) fewer = rows >= 24576u ? 2u : 3u;
         else if constexpr (std::is_same<F, FmtQ8Aos>::value) fewer = T <= 2 ? 2u : (T <= 4 ? 3u : kWgsPerCu);
         else if constexpr (T == 1 && std::is_same<F, FmtQ4K>::value) fewer = 3u;
-        else if constexpr (T == 1 && std::is_same<F, FmtQ6K>::value) fewer = rows >= 65536u ? 3u : kWgsPerCu;
+        else if constexpr (T <= 2 && std::is_same<F, FmtQ6K>::value) fewer = K <= 4096u ? 2u : 3u;
         if (per_cu > fewer) per_cu = fewer;
     }
     const uint32_t cap = (uint32_t)cu_count() * per_cu / nseg;
