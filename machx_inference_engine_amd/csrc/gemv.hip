@@ -679,8 +679,8 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
         // More waves than the memory system can serve only lengthen its queues; measured per format (K = 4096, us with
         // four workgroups per CU -> with the number chosen here).  Q8_0 planes, interleaved units (two rows per wave in
         // flight): fused gate + up 20.8 -> 20.45 and 128256 rows 88.3 -> 85.2 with two, 14336 rows 12.0 with two, three
-        // or four.  GGUF Q8_0 blocks: one token 13.0 -> 12.15 and two 14.1 -> 13.4 with two, four tokens 15.6 -> 14.6
-        // with three.  Q4_K, one token: 8.2 -> 8.0 with three (4096 rows, q8 activations: 4.47 -> 4.15).  Q6_K, one or two
+        // or four.  GGUF Q8_0 blocks: one token 16.4 -> 14.9 and two 17.6 -> 16.0 with two, four tokens 19.1 -> 18.8
+        // with three.  Q4_K, one token: 8.3 -> 8.0 with three (4096 rows: 4.37 -> 4.09).  Q6_K, one or two
         // tokens, with the two register sets of the one-unit-per-lane path (the same bytes in flight per CU as four
         // workgroups with one set, half the waves competing for the vector pipe): fused gate + up 19.7 -> 17.6 with two
         // (21.9 with one, 19.4 with three), 14336 rows 12.45 -> 11.3, 151936 rows 94.2 -> 88.5, 4096 rows 6.4 -> 5.1, two
