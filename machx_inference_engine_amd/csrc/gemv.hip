@@ -271,6 +271,66 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, O
     }
 }
 
+// The workgroup-wide walk when a row's units fill a whole number of half waves but not of waves (K = 14336: 224 units,
+// three and a half waves, so one lane in eight of gemv_q8_wide_kernel idles): a workgroup of 2 * units threads takes
+// two rows at a time, thread t unit t % units of row t / units; the middle wave holds the end of one row in its first
+// 32 lanes and the start of the other in the rest.  Every wave sums its two halves separately; after the barrier one
+// thread per row adds that row's half-wave sums in order.  Measured against gemv_q8_wide_kernel at 14336 -> 4096, three
+// workgroups per CU: Q6_K 13.2 -> 12.2 us, Q8_0 planes 12.2 -> 12.05; both down projections inside the decode step
+// 65.3 -> 63.3 us (two workgroups per CU: 12.5 / 12.1 us, one: 17.0 / 14.7, four: the step 66.9).
+// q8_split == 2: `xq8` is one fp16 row, quantized while it is staged.
+template <class F, class OutT>
+__global__ __launch_bounds__(512) void gemv_q8_wide_pair_kernel(GemvSeg<F, OutT> seg, const uint8_t* xq8, uint32_t K, uint32_t N, uint32_t KT,
+                                                                 uint32_t q8_split) {
+    static_assert(F::K_ALIGN % 64 == 0, "whole units only");
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ float red[2][16];   // [buffer][half wave]
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t n_units = K / 64, halves_per_row = n_units / 32;
+    const uint32_t slot = tid >= n_units ? 1u : 0u, unit = tid - slot * n_units;
+    auto xrow = [&](uint32_t) { return xq8; };
+    ActTile act;
+    if (q8_split == 2u) {
+        auto hrow = [&](uint32_t) { return reinterpret_cast<const half_t*>(xq8); };
+        act = stage_act_f16<F::SUM_GRAN, 1>(lds, hrow, 0, K, KT);
+    } else {
+        act = stage_act<F::SUM_GRAN, 1>(lds, xrow, 0, K, KT, q8_split != 0);
+    }
+    __syncthreads();
+    const uint32_t n_rg = (N + 1) / 2;
+    uint32_t par = 0;
+    for (uint32_t rg = blockIdx.x; rg < n_rg; rg += gridDim.x, par ^= 1u) {
+        const uint32_t row = 2 * rg + slot;
+        typename F::Cursor cu[1];
+        typename F::Raw raw[1];
+        cu[0] = F::cursor(seg.w, row < N ? row : N - 1, unit);
+        raw[0] = load_unit<F, kGemvThreads>(cu[0], 0, false);
+        float acc[1][1] = {{0.f}};
+        gemv_step<F, 1, 1>(raw, cu, unit, act, acc);
+        const float v = group_sum<32>(acc[0][0]);
+        if ((lane & 31u) == 31u) red[par][2 * wave + (lane >> 5)] = v;
+        __syncthreads();   // one barrier per row pair: the sums alternate between two buffers
+        if (tid < 2 && 2 * rg + tid < N) {
+            float r = 0.f;
+            for (uint32_t hw = tid * halves_per_row; hw < (tid + 1) * halves_per_row; ++hw) r += red[par][hw];
+            if (seg.bias) r += seg.bias[2 * rg + tid];
+            store_out(seg.y + 2 * rg + tid, r);
+        }
+    }
+}
+
+// true if the launch was made: one matrix, one token, units per row = 32 mod 64 and at most 256
+static int cu_count();
+constexpr uint32_t kWidePairWgsPerCu = 3;
+template <class F, class OutT>
+static bool launch_wide_pair(hipStream_t st, const GemvSeg<F, OutT>& g, const uint8_t* x, uint32_t K, uint32_t N, uint32_t KT, uint32_t q8_split) {
+    const uint32_t units = K / 64;
+    if (K % 64 != 0 || units % 64 != 32 || units > 256) return false;
+    const uint32_t cap = (uint32_t)cu_count() * kWidePairWgsPerCu, n_rg = (N + 1) / 2;
+    hipLaunchKernelGGL((gemv_q8_wide_pair_kernel<F, OutT>), dim3(n_rg < cap ? n_rg : cap), dim3(2 * units), act_tile_bytes(1, KT, F::SUM_GRAN), st, g, x, K, N, KT, q8_split);
+    return true;
+}
+
 // Batched launches with long rows and few of them (T >= 2, K >= 8192: the down projections in a speculative-verify
 // batch): the row-group grid alone leaves CUs idle and every workgroup restages several activation tiles.  Here
 // the grid is (row groups, K slices): a workgroup stages one slice once and writes its partial sums to a scratch
@@ -629,6 +689,7 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
         // K = 14336, N = 4096: Q6_K 14.4 -> 12.7 us; no gain for the formats with 64-byte units or for T = 2.
         // (mx_gemv_q6_K_f16q8 takes the same launch under the same condition, so that both forms give the same bits.)
         if (n_tiles == 1 && K >= 8192 && n_rg <= 2u * (uint32_t)cu_count()) {
+            if (nseg == 1 && launch_wide_pair<F, OutT>(st, s0, xq8, K, N, KT, split ? 1u : 0u)) return launch_status();
             const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu / nseg;
             dim3 gridw(N < capw ? N : capw, nseg);
             hipLaunchKernelGGL((gemv_q8_wide_kernel<F, 1, 1, OutT>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, F::SUM_GRAN), st, s0, s1, xq8, K, N, KT,
@@ -1055,6 +1116,7 @@ static int gemv_q8_0_soa_batched(mx_stream_t s, const void* x, const int8_t* qs_
         const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * 3u;
         const dim3 gridw(N < capw ? N : capw, 1);
         const uint8_t* xq = static_cast<const uint8_t*>(x);
+        if (T == 1 && launch_wide_pair<FmtQ8SoaW, half_t>(as_stream(s), g, xq, K, N, KT, 0u)) return launch_status();
         if (T == 1)
             hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN),
                                as_stream(s), g, g, xq, K, N, KT, 1u, 0u);
@@ -1411,6 +1473,7 @@ static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, 
             if (int rc = check_common(x, y, K, N, 1, 256)) return rc;
             MX_REQUIRE_ALIGN(x, 16);
             GemvSeg<FmtQ6K, half_t> g{wa, reinterpret_cast<half_t*>(y), nullptr};
+            if (launch_wide_pair<FmtQ6K, half_t>(as_stream(s), g, static_cast<const uint8_t*>(x), K, N, KT, 2u)) return launch_status();
             const uint32_t capw = (uint32_t)cu_count() * kWideF16WgsPerCu;
             hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ6K, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
                                act_tile_bytes(1, KT, FmtQ6K::SUM_GRAN), as_stream(s), g, g, static_cast<const uint8_t*>(x), K, N, KT, 1u, 2u);
@@ -1439,6 +1502,7 @@ int mx_gemv_q8_0_soa_f16q8(mx_stream_t s, const uint16_t* x_f16, const int8_t* q
         MX_REQUIRE_ALIGN(x_f16, 16);
         GemvSeg<FmtQ8SoaW, half_t> g{{qs_W, d_W, K}, reinterpret_cast<half_t*>(y), nullptr};
         const uint32_t KT = (K + 255) / 256 * 256, capw = (uint32_t)cu_count() * kWideF16WgsPerCu;
+        if (launch_wide_pair<FmtQ8SoaW, half_t>(as_stream(s), g, reinterpret_cast<const uint8_t*>(x_f16), K, N, KT, 2u)) return launch_status();
         hipLaunchKernelGGL((gemv_q8_wide_kernel<FmtQ8SoaW, 1, 1, half_t>), dim3(N < capw ? N : capw, 1), dim3(kGemvThreads),
                            act_tile_bytes(1, KT, FmtQ8SoaW::SUM_GRAN), as_stream(s), g, g, reinterpret_cast<const uint8_t*>(x_f16), K, N, KT, 1u, 2u);
         return launch_status();
