@@ -271,8 +271,8 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, O
     }
 }
 
-// The workgroup-wide walk when a row's units fill a whole number of half waves but not of waves (K = 14336: 224 units,
-// three and a half waves, so one lane in eight of gemv_q8_wide_kernel idles): a workgroup of 2 * units threads takes
+// The workgroup-wide walk when a row's units fill a whole number of half waves but fewer than four waves (K = 14336:
+// 224 units, three and a half waves, so one lane in eight of gemv_q8_wide_kernel idles): a workgroup of 2 * units threads takes
 // two rows at a time, thread t unit t % units of row t / units; the middle wave holds the end of one row in its first
 // 32 lanes and the start of the other in the rest.  Every wave sums its two halves separately; after the barrier one
 // thread per row adds that row's half-wave sums in order.  Measured against gemv_q8_wide_kernel at 14336 -> 4096, three
@@ -319,13 +319,14 @@ __global__ __launch_bounds__(512) void gemv_q8_wide_pair_kernel(GemvSeg<F, OutT>
     }
 }
 
-// true if the launch was made: one matrix, one token, units per row = 32 mod 64 and at most 256
+// true if the launch was made: one matrix, one token, a whole number of half waves per row and fewer than four waves
+// (K = 8192, Q8_0 planes: 9.45 -> 8.35 us; K = 12288: 11.1 -> 10.9; with 256 units gemv_q8_wide_kernel has no idle lane)
 static int cu_count();
 constexpr uint32_t kWidePairWgsPerCu = 3;
 template <class F, class OutT>
 static bool launch_wide_pair(hipStream_t st, const GemvSeg<F, OutT>& g, const uint8_t* x, uint32_t K, uint32_t N, uint32_t KT, uint32_t q8_split) {
     const uint32_t units = K / 64;
-    if (K % 64 != 0 || units % 64 != 32 || units > 256) return false;
+    if (K % 64 != 0 || units % 32 != 0 || units >= 256) return false;
     const uint32_t cap = (uint32_t)cu_count() * kWidePairWgsPerCu, n_rg = (N + 1) / 2;
     hipLaunchKernelGGL((gemv_q8_wide_pair_kernel<F, OutT>), dim3(n_rg < cap ? n_rg : cap), dim3(2 * units), act_tile_bytes(1, KT, F::SUM_GRAN), st, g, x, K, N, KT, q8_split);
     return true;
