@@ -685,17 +685,20 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
     const uint32_t KT = (K256 + n_tiles - 1) / n_tiles * 256;   // balanced tiles
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
-    if constexpr (T == 1 && F::SUM_GRAN == 16) {
+    if constexpr (T == 1 && (F::SUM_GRAN == 16 || std::is_same<F, FmtQ4K>::value)) {
         // long rows, too few of them to give every CU its workgroups: the workgroup-wide row walk.  Measured at
-        // K = 14336, N = 4096: Q6_K 14.4 -> 12.7 us; no gain for the formats with 64-byte units or for T = 2.
-        // (mx_gemv_q6_K_f16q8 takes the same launch under the same condition, so that both forms give the same bits.)
+        // K = 14336, N = 4096: Q6_K 14.4 -> 12.7 us, 12.2 with paired rows; Q4_K gains nothing from the 256-thread walk
+        // and 9.65 -> 8.8 us from the paired rows; no gain for T = 2.
+        // (mx_gemv_q6_K_f16q8 / mx_gemv_q4_K_f16q8 take the same launch under the same condition, so that both forms give the same bits.)
         if (n_tiles == 1 && K >= 8192 && n_rg <= 2u * (uint32_t)cu_count()) {
             if (nseg == 1 && launch_wide_pair<F, OutT>(st, s0, xq8, K, N, KT, split ? 1u : 0u)) return launch_status();
-            const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu / nseg;
-            dim3 gridw(N < capw ? N : capw, nseg);
-            hipLaunchKernelGGL((gemv_q8_wide_kernel<F, 1, 1, OutT>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, F::SUM_GRAN), st, s0, s1, xq8, K, N, KT,
-                               T_real, split ? 1u : 0u);
-            return launch_status();
+            if constexpr (F::SUM_GRAN == 16) {
+                const uint32_t capw = (uint32_t)cu_count() * kWgsPerCu / nseg;
+                dim3 gridw(N < capw ? N : capw, nseg);
+                hipLaunchKernelGGL((gemv_q8_wide_kernel<F, 1, 1, OutT>), gridw, dim3(kGemvThreads), act_tile_bytes(1, KT, F::SUM_GRAN), st, s0, s1, xq8, K, N, KT,
+                                   T_real, split ? 1u : 0u);
+                return launch_status();
+            }
         }
     }
     if constexpr (T >= 2) {
@@ -1462,6 +1465,15 @@ static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, 
     const uint8_t *a = static_cast<const uint8_t*>(W0), *b = static_cast<const uint8_t*>(W1);
     if (fmt == 1) {
         const FmtQ4K::W wa{a, K / 256 * (uint32_t)kQ4KBytes}, wb{b, K / 256 * (uint32_t)kQ4KBytes};
+        // the single GEMV on a long row of a short matrix: the paired-row walk, as mx_gemv_q4_K_q8 takes it (launch_q8_tg)
+        const uint32_t KT4 = (K + 255) / 256 * 256;
+        if (nw == 1 && x_is_f16 && K >= 8192 && act_tile_bytes(1, KT4, FmtQ4K::SUM_GRAN) <= kLdsBudget &&
+            (N + kGemvWaves * (64 / pick_group(K / 64)) - 1) / (kGemvWaves * (64 / pick_group(K / 64))) <= 2u * (uint32_t)cu_count()) {
+            if (int rc = check_common(x, y, K, N, 1, 256)) return rc;
+            MX_REQUIRE_ALIGN(x, 16);
+            GemvSeg<FmtQ4K, half_t> g{wa, reinterpret_cast<half_t*>(y), nullptr};
+            if (launch_wide_pair<FmtQ4K, half_t>(as_stream(s), g, static_cast<const uint8_t*>(x), K, N, KT4, 2u)) return launch_status();
+        }
         return nw == 2 ? launch_ffn_x<FmtQ4K, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ4K, 1>(s, wa, wb, x, x_is_f16, y, K, N);
     }
     if (fmt == 2) {
