@@ -282,7 +282,6 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_q8_wide_kernel(GemvSeg<F, O
 template <class F, class OutT>
 __global__ __launch_bounds__(512) void gemv_q8_wide_pair_kernel(GemvSeg<F, OutT> seg, const uint8_t* xq8, uint32_t K, uint32_t N, uint32_t KT,
                                                                  uint32_t q8_split) {
-    static_assert(F::K_ALIGN % 64 == 0, "whole units only");
     extern __shared__ __align__(16) uint8_t lds[];
     __shared__ float red[2][16];   // [buffer][half wave]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -685,7 +684,7 @@ static int launch_q8_tg(hipStream_t st, const GemvSeg<F, OutT>& s0, const GemvSe
     const uint32_t K256 = (K + 255) / 256, n_tiles = (K256 * 256 + KT_max - 1) / KT_max;
     const uint32_t KT = (K256 + n_tiles - 1) / n_tiles * 256;   // balanced tiles
     const uint32_t n_rg = (N + rows_per_wg - 1) / rows_per_wg;
-    if constexpr (T == 1 && (F::SUM_GRAN == 16 || std::is_same<F, FmtQ4K>::value)) {
+    if constexpr (T == 1 && (F::SUM_GRAN == 16 || std::is_same<F, FmtQ4K>::value || std::is_same<F, FmtQ8Aos>::value)) {
         // long rows, too few of them to give every CU its workgroups: the workgroup-wide row walk.  Measured at
         // K = 14336, N = 4096: Q6_K 14.4 -> 12.7 us, 12.2 with paired rows; Q4_K gains nothing from the 256-thread walk
         // and 9.65 -> 8.8 us from the paired rows; no gain for T = 2.
@@ -1495,6 +1494,16 @@ static int ffn_aos(int fmt, int nw, mx_stream_t s, const void* x, int x_is_f16, 
         return nw == 2 ? launch_ffn_x<FmtQ6K, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ6K, 1>(s, wa, wb, x, x_is_f16, y, K, N);
     }
     const FmtQ8Aos::W wa{a, K / 32 * (uint32_t)kQ8_0Bytes}, wb{b, K / 32 * (uint32_t)kQ8_0Bytes};
+    {   // the single GEMV on a long row of a short matrix: the paired-row walk, as mx_gemv_q8_0_q8 takes it (launch_q8_tg)
+        const uint32_t KT8 = (K + 255) / 256 * 256;
+        if (nw == 1 && x_is_f16 && K >= 8192 && act_tile_bytes(1, KT8, FmtQ8Aos::SUM_GRAN) <= kLdsBudget &&
+            (N + kGemvWaves * (64 / pick_group((K + 63) / 64)) - 1) / (kGemvWaves * (64 / pick_group((K + 63) / 64))) <= 2u * (uint32_t)cu_count()) {
+            if (int rc = check_common(x, y, K, N, 1, 32)) return rc;
+            MX_REQUIRE_ALIGN(x, 16);
+            GemvSeg<FmtQ8Aos, half_t> g{wa, reinterpret_cast<half_t*>(y), nullptr};
+            if (launch_wide_pair<FmtQ8Aos, half_t>(as_stream(s), g, static_cast<const uint8_t*>(x), K, N, KT8, 2u)) return launch_status();
+        }
+    }
     return nw == 2 ? launch_ffn_x<FmtQ8Aos, 2>(s, wa, wb, x, x_is_f16, y, K, N) : launch_ffn_x<FmtQ8Aos, 1>(s, wa, wb, x, x_is_f16, y, K, N);
 }
 int mx_gemv_q4_K_x2_silu(mx_stream_t s, const void* x, int x_is_f16, const void* gate_W, const void* up_W, uint16_t* h, uint32_t K, uint32_t N) {
